@@ -1,0 +1,122 @@
+// Embedding gather, RMSNorm (with the residual add fused in), SwiGLU and element type casts.
+//
+// Formulas follow the reference: embedding rows widened to 32-bit (engine/engine.cpp:332-357);
+// y = x * (1/sqrt(mean(x^2) + eps)) * w with the statistics in 32-bit (kernels/norm.cpp:13-31,
+// engine/cuda_ops.cu:114-138); fused residual update then norm (engine/cuda_ops.cu:140-170);
+// out = g / (1 + exp(-g)) * u over merged [gate | up] rows (engine/cuda_ops.cu:100-112).
+#include "common.h"
+
+PALM_DEFINE_LAST_ERROR()
+
+PALM_API int palm_page_tokens() { return PAGE_TOKENS; }
+
+// ---- embedding ------------------------------------------------------------------------------------
+// One block per token.  An id outside the table gives a row of NaN: visible, and no read out of bounds.
+template <typename TW>
+__global__ void embed_kernel(const TW* __restrict__ table, const int* __restrict__ ids, float* __restrict__ out,
+                             int hidden, int vocab) {
+    const int t = blockIdx.x;
+    const int id = ids[t];
+    float* dst = out + (size_t)t * hidden;
+    if (id < 0 || id >= vocab) {
+        for (int d = threadIdx.x; d < hidden; d += blockDim.x) dst[d] = NAN;
+        return;
+    }
+    const TW* src = table + (size_t)id * hidden;
+    for (int d = threadIdx.x; d < hidden; d += blockDim.x) dst[d] = to_float(src[d]);
+}
+
+PALM_API int palm_embed(hipStream_t stream, const void* table, int table_dtype, const int* ids, int n_tokens,
+                        int hidden, int vocab, float* out) {
+    PALM_CHECK(n_tokens >= 0 && hidden > 0 && vocab > 0, "embed: n_tokens=%d hidden=%d vocab=%d", n_tokens, hidden, vocab);
+    if (n_tokens == 0) return 0;
+    PALM_DTYPE_SWITCH(table_dtype, TW,
+        embed_kernel<TW><<<n_tokens, 256, 0, stream>>>((const TW*)table, ids, out, hidden, vocab));
+    PALM_LAUNCHED();
+    return 0;
+}
+
+// ---- RMSNorm --------------------------------------------------------------------------------------
+// One block per output row.  src row = rows ? rows[r] : r.  v = x[src] (+ delta[src]).  If update_x the
+// sum is written back to x (only without `rows`), so the residual stream is updated and normed in one
+// pass over it.  Statistics and products in 32-bit; the product order is (v * r) * w.
+template <typename TX, typename TD, typename TO>
+__global__ void rmsnorm_kernel(TX* __restrict__ x, const TD* __restrict__ delta, const float* __restrict__ w,
+                               const int* __restrict__ rows, TO* __restrict__ out, int width, float eps,
+                               int update_x) {
+    __shared__ float scratch[16];
+    const int r = blockIdx.x;
+    const size_t src = rows ? (size_t)rows[r] : (size_t)r;
+    TX* xr = x + src * width;
+    const TD* dr = delta ? delta + src * width : nullptr;
+    float ss = 0.f;
+    for (int d = threadIdx.x; d < width; d += blockDim.x) {
+        float v = to_float(xr[d]);
+        if (dr) v += to_float(dr[d]);
+        ss += v * v;
+    }
+    ss = block_sum(ss, scratch);
+    const float inv = 1.0f / sqrtf(ss / (float)width + eps);
+    TO* o = out + (size_t)r * width;
+    for (int d = threadIdx.x; d < width; d += blockDim.x) {
+        float v = to_float(xr[d]);
+        if (dr) v += to_float(dr[d]);
+        if (update_x) xr[d] = from_float<TX>(v);
+        o[d] = from_float<TO>(v * inv * w[d]);
+    }
+}
+
+PALM_API int palm_rmsnorm(hipStream_t stream, void* x, int x_dtype, const void* delta, int delta_dtype,
+                          const float* weight, float eps, const int* rows, int n_out_rows, int width,
+                          void* out, int out_dtype, int update_x) {
+    PALM_CHECK(n_out_rows >= 0 && width > 0, "rmsnorm: rows=%d width=%d", n_out_rows, width);
+    PALM_CHECK(!(update_x && rows), "rmsnorm: the residual cannot be updated through a row selection");
+    PALM_CHECK(!(update_x && !delta), "rmsnorm: update_x without a delta has nothing to add");
+    if (n_out_rows == 0) return 0;
+    const int threads = width >= 1024 ? 256 : (width >= 256 ? 128 : 64);
+    PALM_DTYPE_SWITCH(x_dtype, TX, PALM_DTYPE_SWITCH(delta_dtype, TD, PALM_DTYPE_SWITCH(out_dtype, TO,
+        rmsnorm_kernel<TX, TD, TO><<<n_out_rows, threads, 0, stream>>>(
+            (TX*)x, (const TD*)delta, weight, rows, (TO*)out, width, eps, update_x))));
+    PALM_LAUNCHED();
+    return 0;
+}
+
+// ---- SwiGLU ---------------------------------------------------------------------------------------
+template <typename T>
+__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int n_rows, int inter) {
+    const size_t total = (size_t)n_rows * inter;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        const size_t r = i / inter, c = i % inter;
+        const float g = to_float(gu[r * 2 * inter + c]);
+        const float u = to_float(gu[r * 2 * inter + inter + c]);
+        out[i] = from_float<T>(g / (1.0f + expf(-g)) * u);
+    }
+}
+
+PALM_API int palm_swiglu(hipStream_t stream, const void* gate_up, int dtype, void* out, int n_rows, int inter) {
+    PALM_CHECK(n_rows >= 0 && inter > 0, "swiglu: rows=%d intermediate=%d", n_rows, inter);
+    if (n_rows == 0) return 0;
+    const size_t total = (size_t)n_rows * inter;
+    const int blocks = (int)((total + 255) / 256 < 65536 ? (total + 255) / 256 : 65536);
+    PALM_DTYPE_SWITCH(dtype, T,
+        swiglu_kernel<T><<<blocks, 256, 0, stream>>>((const T*)gate_up, (T*)out, n_rows, inter));
+    PALM_LAUNCHED();
+    return 0;
+}
+
+// ---- casts ----------------------------------------------------------------------------------------
+template <typename TS, typename TD>
+__global__ void cast_kernel(const TS* __restrict__ src, TD* __restrict__ dst, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+        dst[i] = from_float<TD>(to_float(src[i]));
+}
+
+PALM_API int palm_cast(hipStream_t stream, const void* src, int src_dtype, void* dst, int dst_dtype, long long n) {
+    PALM_CHECK(n >= 0, "cast: n=%lld", n);
+    if (n == 0) return 0;
+    const int blocks = (int)((n + 255) / 256 < 65536 ? (n + 255) / 256 : 65536);
+    PALM_DTYPE_SWITCH(src_dtype, TS, PALM_DTYPE_SWITCH(dst_dtype, TD,
+        cast_kernel<TS, TD><<<blocks, 256, 0, stream>>>((const TS*)src, (TD*)dst, (size_t)n)));
+    PALM_LAUNCHED();
+    return 0;
+}

@@ -1,0 +1,5 @@
+"""The model built from its description, the step function, the generation loop and trace replay."""
+from .engine import Engine, StepEntry, StepError, resolve_dtype
+from .model import DecoderModel
+
+__all__ = ["Engine", "StepEntry", "StepError", "resolve_dtype", "DecoderModel"]

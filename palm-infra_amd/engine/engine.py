@@ -1,0 +1,172 @@
+"""The engine: a model, its cache, and the one step function that everything above it uses.
+
+The reference has two entry points for one sequence, ``prefill_chunk(ids, past)`` and ``decode(id)``
+(engine/engine.cpp:1248-1381, 1383-1460): embed, rotation table, mask, graph, final norm, head on the
+last row.  Here one ``step`` takes a batch of sequences, each with its next tokens (a whole prompt, a
+piece of one, or a single token), runs only those tokens from what the cache holds, and returns the
+logits at the places asked for.  Sequences are packed without padding, so a sequence's result cannot
+depend on its companions' lengths.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from pathlib import Path
+
+import torch
+
+from ..cache import ModelCache
+from ..config import config_from_dict, config_from_dir
+from ..parts import make_context
+from ..weights import ModelFiles, load_weights, random_weights
+from .model import DecoderModel
+
+DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32}
+
+
+class StepError(ValueError):
+    """A step was asked for something that cannot run: a token outside the vocabulary, a slot that is
+    not open, a place outside the tokens given."""
+
+
+@dataclass
+class StepEntry:
+    """The next tokens of one sequence and the places among them whose logits are wanted."""
+    slot: int
+    tokens: list
+    want: list = field(default_factory=list)
+
+
+def resolve_dtype(dtype) -> torch.dtype:
+    if isinstance(dtype, torch.dtype):
+        if dtype not in (torch.bfloat16, torch.float32):
+            raise ValueError(f"dtype {dtype} is neither bfloat16 nor float32")
+        return dtype
+    if dtype not in DTYPES:
+        raise ValueError(f"dtype {dtype!r} is not one of {sorted(DTYPES)}")
+    return DTYPES[dtype]
+
+
+class Engine:
+    def __init__(self, config, spec, weights, dtype: torch.dtype, max_tokens: int, max_seqs: int | None = None,
+                 device="cuda:0", graphs: bool = True):
+        self.device = torch.device(device)
+        if self.device.type != "cuda":
+            raise RuntimeError(f"the engine runs on a GPU; device {device!r} was asked for and there is no CPU path")
+        if not torch.cuda.is_available():
+            raise RuntimeError("no GPU is visible to torch; the engine cannot run")
+        torch.cuda.set_device(self.device)
+        self.config, self.spec, self.dtype = config, spec, dtype
+        self.model = DecoderModel(spec, weights, dtype, self.device)
+        needs, shares = self.model.cache_plan()
+        self.cache = ModelCache(needs, shares, max_tokens, max_seqs, spec.max_positions, dtype, self.device)
+        self.vocab_size = spec.vocab_size
+        self.graphs_enabled = bool(graphs)
+        self._decode_graphs: dict = {}
+        # a windowed group gives pages back only between steps, so long prompts go through it in pieces
+        windows = [g.need.window for g in self.cache.kv_groups if g.need.window]
+        self.step_tokens_per_seq = max(1024, 2 * max(windows)) if windows else None
+
+    # ---- construction ------------------------------------------------------------------------
+    @classmethod
+    def from_dir(cls, model_dir, dtype="bfloat16", max_tokens: int | None = None, device="cuda:0", **options):
+        """A folder with config.json and safetensors; the model class is chosen by config.json."""
+        dt = resolve_dtype(dtype)
+        model_dir = Path(model_dir)
+        config = config_from_dir(model_dir)
+        files = ModelFiles(model_dir)
+        spec = config.spec(files.names())
+        weights = load_weights(spec, files, dt, device)
+        return cls(config, spec, weights, dt, max_tokens or 16384, device=device, **options)
+
+    @classmethod
+    def from_config(cls, config, seed: int = 0, dtype="bfloat16", max_tokens: int | None = None, device="cuda:0",
+                    **options):
+        """Random weights made on the device (no folder is written)."""
+        dt = resolve_dtype(dtype)
+        if isinstance(config, dict):
+            config = config_from_dict(config)
+        spec = config.spec()
+        weights = random_weights(spec, seed, dt, device)
+        return cls(config, spec, weights, dt, max_tokens or 16384, device=device, **options)
+
+    # ---- sequences ---------------------------------------------------------------------------
+    def open(self) -> int:
+        """A slot for a new sequence."""
+        return self.cache.open()
+
+    def close(self, slot: int) -> None:
+        """The sequence is over: what it holds goes back."""
+        self.cache.close(slot)
+
+    def length(self, slot: int) -> int:
+        return self.cache.lengths[slot]
+
+    # ---- the step ----------------------------------------------------------------------------
+    def _validate(self, entries) -> None:
+        if not entries:
+            raise StepError("a step needs at least one sequence")
+        seen = set()
+        for e in entries:
+            if e.slot in seen:
+                raise StepError(f"slot {e.slot} appears twice in one step")
+            seen.add(e.slot)
+            if not self.cache.slots.is_held(e.slot):
+                raise StepError(f"slot {e.slot} is not open")
+            if len(e.tokens) == 0:
+                raise StepError(f"slot {e.slot} brings no tokens")
+            for t in e.tokens:
+                if not 0 <= int(t) < self.vocab_size:
+                    raise StepError(f"token id {t} lies outside the vocabulary of {self.vocab_size}")
+            for w in e.want:
+                if not 0 <= int(w) < len(e.tokens):
+                    raise StepError(f"slot {e.slot}: logits wanted at place {w} of {len(e.tokens)} tokens")
+
+    def step(self, entries) -> torch.Tensor:
+        """Run the entries' tokens as one batch from the cache; float32 logits [wanted, vocab] in the
+        order of the entries and of each entry's ``want``.  Nothing changes if the step is refused."""
+        entries = [e if isinstance(e, StepEntry) else StepEntry(*e) for e in entries]
+        self._validate(entries)
+        limit = self.step_tokens_per_seq
+        if limit is None or all(len(e.tokens) <= limit for e in entries):
+            return self._run(entries)
+        # pieces of at most `limit` tokens per sequence, one after the other
+        results = {}
+        n_pieces = max((len(e.tokens) + limit - 1) // limit for e in entries)
+        for c in range(n_pieces):
+            piece, back = [], []
+            for i, e in enumerate(entries):
+                toks = e.tokens[c * limit:(c + 1) * limit]
+                if not toks:
+                    continue
+                want = [w - c * limit for w in e.want if c * limit <= w < (c + 1) * limit]
+                piece.append(StepEntry(e.slot, toks, want))
+                back.extend((i, w + c * limit) for w in want)
+            logits = self._run(piece)
+            for r, key in enumerate(back):
+                results[key] = logits[r]
+        rows = [results[(i, w)] for i, e in enumerate(entries) for w in e.want]
+        if not rows:
+            return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
+        return torch.stack(rows)
+
+    def _run(self, entries) -> torch.Tensor:
+        cache = self.cache
+        growth = [(e.slot, len(e.tokens)) for e in entries]
+        cache.reserve(growth)
+        starts = [cache.lengths[e.slot] for e in entries]
+        ctx = make_context([e.slot for e in entries], starts, [list(map(int, e.tokens)) for e in entries],
+                           self.dtype, self.device)
+        want_rows = [ctx.host["cu"][b] + int(w) for b, e in enumerate(entries) for w in e.want]
+        if want_rows:
+            rows = torch.tensor(want_rows, dtype=torch.int32).to(self.device)
+        else:
+            # nothing is wanted: the layers still run (they fill the cache); the head does not
+            rows = torch.empty((0,), dtype=torch.int32, device=self.device)
+        logits = self.model.forward(ctx, cache, rows)
+        cache.commit(growth)
+        return logits
+
+    # ---- facts -------------------------------------------------------------------------------
+    def memory_report(self) -> dict:
+        return {"weights_bytes": self.model.weights.nbytes(), "cache_bytes": self.cache.nbytes(),
+                "cache_tokens": self.cache.max_tokens, "slots": self.cache.max_seqs}

@@ -1,0 +1,70 @@
+"""Trace replay: feed given token ids through a model step by step and write logits.
+
+It samples nothing and has no forward pass, cache or loader of its own: it drives the engine's
+``step``, the one that generation uses.  The reference's nearest tools are ``prefill_hidden`` /
+``decode_hidden`` / ``run_lmhead_raw(all_positions)`` (engine/engine.cpp:1062-1246, 1669-1720,
+487-555), which its chunked-prefill test drives (tests/test_e2e.cpp:413-529).
+
+Input, one JSON object a line::
+
+    {"step": 0, "entries": [{"id": "a", "tokens": [5, 17, 3], "want": [0, 2]}], "end": []}
+
+For a step in which something is wanted, ``<out>/<step>.f32`` holds the logits at the wanted places in
+the order of the entries and of ``want``, little-endian float32 [wanted, vocab].  After every step a
+line ``done <step>`` is printed and flushed.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import sys
+from pathlib import Path
+
+import numpy as np
+
+
+def replay(engine, lines, out_dir, report=print) -> None:
+    out_dir = Path(out_dir)
+    out_dir.mkdir(parents=True, exist_ok=True)
+    from .engine import StepEntry
+    slots: dict[str, int] = {}
+    for line in lines:
+        line = line.strip()
+        if not line:
+            continue
+        rec = json.loads(line)
+        step_no = rec["step"]
+        entries = []
+        for e in rec.get("entries", []):
+            rid = str(e["id"])
+            if rid not in slots:
+                slots[rid] = engine.open()
+            entries.append(StepEntry(slots[rid], list(e["tokens"]), list(e.get("want", []))))
+        if entries:
+            logits = engine.step(entries)
+            if logits.shape[0] > 0:
+                arr = logits.detach().to("cpu").numpy().astype("<f4", copy=False)
+                arr.tofile(out_dir / f"{step_no}.f32")
+        for rid in rec.get("end", []):
+            rid = str(rid)
+            if rid in slots:
+                engine.close(slots.pop(rid))
+        report(f"done {step_no}")
+
+
+def main(argv=None) -> int:
+    ap = argparse.ArgumentParser(prog="trace_run", description="Replay token ids through a model and write logits.")
+    ap.add_argument("--model", required=True, help="folder with config.json and model.safetensors")
+    ap.add_argument("--dtype", required=True, choices=["bfloat16", "float32"])
+    ap.add_argument("--out", required=True, help="folder for <step>.f32 files")
+    ap.add_argument("--max-tokens", type=int, required=True,
+                    help="the most tokens that live requests hold at any time (each rounded up to 64)")
+    args = ap.parse_args(argv)
+    from .engine import Engine
+    engine = Engine.from_dir(args.model, dtype=args.dtype, max_tokens=args.max_tokens)
+
+    def report(msg):
+        print(msg, flush=True)
+
+    replay(engine, sys.stdin, args.out, report)
+    return 0

@@ -1,0 +1,302 @@
+"""The kernels as functions on torch tensors.
+
+Every function checks on the host what its kernel assumes (device, element types, contiguity, shapes
+that fit each other) before it launches anything, and launches on torch's current stream.  Tensors
+are only memory here: no torch operator computes on the product path.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_float, c_int, c_longlong, c_void_p
+
+import torch
+
+from . import library
+from .library import KernelError
+
+F32, BF16 = torch.float32, torch.bfloat16
+_CODES = {F32: 0, BF16: 1}
+PAGE_TOKENS = 64
+
+_SIGNATURES = {
+    "palm_embed": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_void_p],
+    "palm_rmsnorm": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_float, c_void_p, c_int, c_int,
+                     c_void_p, c_int, c_int],
+    "palm_swiglu": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int],
+    "palm_cast": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_longlong],
+    "palm_linear": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int],
+    "palm_qk_norm_rope_store": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
+                                c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                                c_int, c_int, c_int],
+    "palm_rope_table": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int],
+    "palm_attention_simple": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
+                              c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
+    "palm_argmax": [c_void_p, c_void_p, c_int, c_int, c_void_p],
+    "palm_apply_penalties": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_float, c_float, c_float],
+    "palm_sample": [c_void_p, c_void_p, c_int, c_int, c_void_p, c_float, c_int, c_float, c_float, c_void_p, c_void_p],
+}
+
+_core = None
+
+
+def core():
+    """The core library, with the argument types of its entry points declared."""
+    global _core
+    if _core is None:
+        lib = library.load("core")
+        for name, argtypes in _SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.argtypes, fn.restype = argtypes, c_int
+        if lib.palm_page_tokens() != PAGE_TOKENS:
+            raise KernelError(f"the kernels were built for pages of {lib.palm_page_tokens()} tokens, "
+                              f"the cache uses {PAGE_TOKENS}")
+        _core = lib
+    return _core
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _p(t):
+    return None if t is None else t.data_ptr()
+
+
+def _code(t: torch.Tensor, what: str) -> int:
+    if t.dtype not in _CODES:
+        raise KernelError(f"{what}: element type {t.dtype} is neither float32 nor bfloat16")
+    return _CODES[t.dtype]
+
+
+def _dev(what: str, *tensors) -> None:
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise KernelError(f"{what}: a tensor lies on {t.device}; the kernels run on the GPU only "
+                              "(there is no CPU path)")
+        if not t.is_contiguous():
+            raise KernelError(f"{what}: a tensor of shape {tuple(t.shape)} is not contiguous")
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise KernelError(f"{what}: tensors lie on {dev} and {t.device}")
+
+
+def _need(cond: bool, msg: str) -> None:
+    if not cond:
+        raise KernelError(msg)
+
+
+def _i32(what: str, *tensors) -> None:
+    for t in tensors:
+        if t is not None and t.dtype != torch.int32:
+            raise KernelError(f"{what}: an index tensor has element type {t.dtype}, not int32")
+
+
+# ---- elementwise ----------------------------------------------------------------------------------
+
+def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    """out[t, :] = table[ids[t], :] as float32."""
+    _dev("embed", table, ids, out)
+    _i32("embed", ids)
+    _need(table.dim() == 2 and ids.dim() == 1, f"embed: table {tuple(table.shape)}, ids {tuple(ids.shape)}")
+    vocab, hidden = table.shape
+    n = ids.shape[0]
+    if out is None:
+        out = torch.empty((n, hidden), dtype=F32, device=table.device)
+    _need(out.shape == (n, hidden) and out.dtype == F32, f"embed: out {tuple(out.shape)} {out.dtype}")
+    library.call(core(), "palm_embed", _stream(), _p(table), _code(table, "embed table"), _p(ids), n, hidden, vocab, _p(out))
+    return out
+
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.dtype, delta: torch.Tensor | None = None,
+            update_x: bool = False, rows: torch.Tensor | None = None) -> torch.Tensor:
+    """out[r] = norm(x[src] + delta[src]) * weight, src = rows[r] or r; with update_x the sum is written
+    back to x (the residual stream).  x is [n, width]; statistics in float32."""
+    _dev("rmsnorm", x, weight, delta, rows)
+    _i32("rmsnorm", rows)
+    _need(x.dim() == 2, f"rmsnorm: x {tuple(x.shape)} is not [rows, width]")
+    n, width = x.shape
+    _need(weight.shape == (width,) and weight.dtype == F32, f"rmsnorm: weight {tuple(weight.shape)} {weight.dtype}, "
+          f"width {width} (norm weights are float32)")
+    _need(delta is None or delta.shape == x.shape, "rmsnorm: delta and x differ in shape")
+    _need(not update_x or (delta is not None and rows is None), "rmsnorm: update_x needs a delta and no row selection")
+    n_out = n if rows is None else rows.shape[0]
+    out = torch.empty((n_out, width), dtype=out_dtype, device=x.device)
+    library.call(core(), "palm_rmsnorm", _stream(), _p(x), _code(x, "rmsnorm x"), _p(delta),
+                 _code(delta, "rmsnorm delta") if delta is not None else 0, _p(weight), float(eps), _p(rows), n_out, width,
+                 _p(out), _code(out, "rmsnorm out"), int(update_x))
+    return out
+
+
+def swiglu(gate_up: torch.Tensor) -> torch.Tensor:
+    """[n, 2I] -> [n, I]: silu(first half) * second half."""
+    _dev("swiglu", gate_up)
+    _need(gate_up.dim() == 2 and gate_up.shape[1] % 2 == 0, f"swiglu: input {tuple(gate_up.shape)}")
+    n, two_i = gate_up.shape
+    out = torch.empty((n, two_i // 2), dtype=gate_up.dtype, device=gate_up.device)
+    library.call(core(), "palm_swiglu", _stream(), _p(gate_up), _code(gate_up, "swiglu"), _p(out), n, two_i // 2)
+    return out
+
+
+def cast(src: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    _dev("cast", src)
+    if src.dtype == dtype:
+        return src
+    out = torch.empty(src.shape, dtype=dtype, device=src.device)
+    library.call(core(), "palm_cast", _stream(), _p(src), _code(src, "cast"), _p(out), _code(out, "cast"), src.numel())
+    return out
+
+
+# ---- linear ---------------------------------------------------------------------------------------
+
+def linear_exact(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = None, out: torch.Tensor | None = None,
+                 accumulate: bool = False) -> torch.Tensor:
+    """a [M, K] . w [N, K]^T with plain 32-bit FMA; any mix of float32 and bfloat16 operands."""
+    _dev("linear", a, w, out)
+    _need(a.dim() == 2 and w.dim() == 2 and a.shape[1] == w.shape[1],
+          f"linear: a {tuple(a.shape)} and w {tuple(w.shape)} do not share the inner size")
+    M, K = a.shape
+    N = w.shape[0]
+    if out is None:
+        _need(not accumulate, "linear: accumulate needs an output to add to")
+        out = torch.empty((M, N), dtype=out_dtype or a.dtype, device=a.device)
+    _need(out.shape == (M, N), f"linear: out {tuple(out.shape)} is not {(M, N)}")
+    library.call(core(), "palm_linear", _stream(), _p(a), _code(a, "linear a"), _p(w), _code(w, "linear w"), _p(out),
+                 _code(out, "linear out"), M, N, K, int(accumulate))
+    return out
+
+
+# ---- attention ------------------------------------------------------------------------------------
+
+def _check_cache(what, k_cache, v_cache, block_table, nkv, hd):
+    _need(k_cache.dim() == 4 and k_cache.shape[1:] == (nkv, PAGE_TOKENS, hd),
+          f"{what}: key cache {tuple(k_cache.shape)} is not [pages, {nkv}, {PAGE_TOKENS}, {hd}]")
+    _need(v_cache.shape == k_cache.shape and v_cache.dtype == k_cache.dtype, f"{what}: value cache differs from key cache")
+    _need(block_table.dim() == 2, f"{what}: page table {tuple(block_table.shape)} is not [slots, pages]")
+
+
+def qk_norm_rope_store(qkv: torch.Tensor, nh: int, nkv: int, hd: int, positions: torch.Tensor, *, q_norm_w=None,
+                       k_norm_w=None, eps: float = 0.0, cos=None, sin=None, rotary_dim: int = 0, pairing: int = 0,
+                       k_cache=None, v_cache=None, block_table=None, tok_slot=None, write_cache: bool = True) -> torch.Tensor:
+    """qkv [n, (nh + 2 nkv) hd] -> q [n, nh hd], normed and rotated by the cos/sin rows [n, rotary_dim/2];
+    k (normed, rotated) and v go to the cache page of (tok_slot[t], positions[t])."""
+    _dev("qk_norm_rope_store", qkv, positions, q_norm_w, k_norm_w, cos, sin, k_cache, v_cache, block_table, tok_slot)
+    _i32("qk_norm_rope_store", positions, block_table, tok_slot)
+    n = qkv.shape[0]
+    _need(qkv.dim() == 2 and qkv.shape[1] == (nh + 2 * nkv) * hd, f"qk_norm_rope_store: qkv {tuple(qkv.shape)} is not "
+          f"[n, ({nh} + 2*{nkv}) * {hd}]")
+    _need(positions.shape == (n,), "qk_norm_rope_store: one position for each token")
+    for w, nm in ((q_norm_w, "q"), (k_norm_w, "k")):
+        _need(w is None or (w.shape == (hd,) and w.dtype == F32), f"qk_norm_rope_store: {nm} norm weight must be float32 [{hd}]")
+    _need((cos is None) == (sin is None), "qk_norm_rope_store: cos and sin come together")
+    if cos is not None:
+        _need(0 < rotary_dim <= hd and rotary_dim % 2 == 0, f"qk_norm_rope_store: rotary_dim {rotary_dim}, head_dim {hd}")
+        for tab in (cos, sin):
+            _need(tab.dtype == F32 and tab.shape == (n, rotary_dim // 2),
+                  f"qk_norm_rope_store: rotation table {tuple(tab.shape)} {tab.dtype} is not float32 [{n}, {rotary_dim // 2}]")
+    max_pages = 0
+    if write_cache:
+        _need(k_cache is not None and v_cache is not None and block_table is not None and tok_slot is not None,
+              "qk_norm_rope_store: writing the cache needs cache, page table and slots")
+        _check_cache("qk_norm_rope_store", k_cache, v_cache, block_table, nkv, hd)
+        _need(k_cache.dtype == qkv.dtype, f"qk_norm_rope_store: cache is {k_cache.dtype}, activations are {qkv.dtype}")
+        _need(tok_slot.shape == (n,), "qk_norm_rope_store: one slot for each token")
+        max_pages = block_table.shape[1]
+    q_out = torch.empty((n, nh * hd), dtype=qkv.dtype, device=qkv.device)
+    library.call(core(), "palm_qk_norm_rope_store", _stream(), _p(qkv), _code(qkv, "qkv"), _p(q_out), _p(k_cache), _p(v_cache),
+                 _p(block_table), max_pages, _p(tok_slot), _p(positions), _p(q_norm_w), _p(k_norm_w), float(eps),
+                 _p(cos), _p(sin), int(rotary_dim if cos is not None else 0), int(pairing), n, nh, nkv, hd, int(write_cache))
+    return q_out
+
+
+def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor):
+    """cos, sin [n, half] float32 of positions[t] * inv_freq[i]."""
+    _dev("rope_table", positions, inv_freq)
+    _i32("rope_table", positions)
+    _need(positions.dim() == 1 and inv_freq.dim() == 1 and inv_freq.dtype == F32, "rope_table: positions [n] int32, inv_freq [half] float32")
+    n, half = positions.shape[0], inv_freq.shape[0]
+    cos = torch.empty((n, half), dtype=F32, device=positions.device)
+    sin = torch.empty_like(cos)
+    library.call(core(), "palm_rope_table", _stream(), _p(positions), _p(inv_freq), _p(cos), _p(sin), n, half)
+    return cos, sin
+
+
+def attention_exact(q: torch.Tensor, k_cache, v_cache, block_table, seq_slot, seq_start, seq_new, cu_new, max_new: int,
+                    nh: int, nkv: int, hd: int, scale: float, window: int | None) -> torch.Tensor:
+    """Causal attention of the step's queries over the cache, 32-bit arithmetic, any head size.
+    q [n, nh hd]; sequence b has seq_new[b] queries starting at row cu_new[b] and position seq_start[b]."""
+    _dev("attention", q, k_cache, v_cache, block_table, seq_slot, seq_start, seq_new, cu_new)
+    _i32("attention", block_table, seq_slot, seq_start, seq_new, cu_new)
+    n = q.shape[0]
+    _need(q.dim() == 2 and q.shape[1] == nh * hd, f"attention: q {tuple(q.shape)} is not [n, {nh}*{hd}]")
+    _check_cache("attention", k_cache, v_cache, block_table, nkv, hd)
+    _need(k_cache.dtype == q.dtype, f"attention: cache is {k_cache.dtype}, queries are {q.dtype}")
+    B = seq_slot.shape[0]
+    _need(seq_start.shape == (B,) and seq_new.shape == (B,) and cu_new.shape == (B + 1,),
+          "attention: per-sequence arrays differ in length")
+    out = torch.empty((n, nh * hd), dtype=q.dtype, device=q.device)
+    library.call(core(), "palm_attention_simple", _stream(), _p(q), _code(q, "attention q"), _p(k_cache), _p(v_cache),
+                 _p(block_table), block_table.shape[1], _p(seq_slot), _p(seq_start), _p(seq_new), _p(cu_new), B, int(max_new),
+                 nh, nkv, hd, float(scale), int(window or 0), _p(out))
+    return out
+
+
+# ---- sampling -------------------------------------------------------------------------------------
+
+def argmax(logits: torch.Tensor) -> torch.Tensor:
+    _dev("argmax", logits)
+    _need(logits.dim() == 2 and logits.dtype == F32, f"argmax: logits {tuple(logits.shape)} {logits.dtype}")
+    out = torch.empty((logits.shape[0],), dtype=torch.int32, device=logits.device)
+    library.call(core(), "palm_argmax", _stream(), _p(logits), logits.shape[0], logits.shape[1], _p(out))
+    return out
+
+
+def apply_penalties(logits: torch.Tensor, rows, tokens, counts, repeat_penalty: float, presence: float, frequency: float) -> None:
+    """In place, for each (row, token, count)."""
+    _dev("penalties", logits, rows, tokens, counts)
+    _i32("penalties", rows, tokens, counts)
+    _need(logits.dim() == 2 and logits.dtype == F32, "penalties: logits must be float32 [rows, vocab]")
+    _need(rows.shape == tokens.shape == counts.shape and rows.dim() == 1, "penalties: rows, tokens, counts differ in length")
+    library.call(core(), "palm_apply_penalties", _stream(), _p(logits), logits.shape[1], _p(rows), _p(tokens), _p(counts),
+                 rows.shape[0], float(repeat_penalty), float(presence), float(frequency))
+
+
+def sample(logits: torch.Tensor, uniforms: torch.Tensor | None, temperature: float, top_k: int = 0, top_p: float = 0.0,
+           min_p: float = 0.0, want_probs: bool = False):
+    """One token for each row.  ``uniforms`` [rows] float32 in [0, 1).  With want_probs also the
+    distribution that was drawn from, [rows, vocab]."""
+    _dev("sample", logits, uniforms)
+    _need(logits.dim() == 2 and logits.dtype == F32, f"sample: logits {tuple(logits.shape)} {logits.dtype}")
+    n, V = logits.shape
+    _need(uniforms is None or (uniforms.shape == (n,) and uniforms.dtype == F32), "sample: uniforms must be float32 [rows]")
+    out = torch.empty((n,), dtype=torch.int32, device=logits.device)
+    probs = torch.empty((n, V), dtype=F32, device=logits.device) if want_probs else None
+    library.call(core(), "palm_sample", _stream(), _p(logits), n, V, _p(uniforms), float(temperature), int(top_k), float(top_p),
+                 float(min_p), _p(out), _p(probs))
+    return (out, probs) if want_probs else out
+
+
+# ---- dispatch: which kernel serves a call -----------------------------------------------------------
+
+def linear_library(a: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """bfloat16 a [M, K] . w [N, K]^T through the BLAS library (hipBLASLt under torch.matmul), 32-bit
+    accumulation, bfloat16 result: the one place where a library computes on the product path."""
+    _dev("linear", a, w)
+    _need(a.dtype == BF16 and w.dtype == BF16, "linear_library serves bfloat16 operands only")
+    _need(a.dim() == 2 and w.dim() == 2 and a.shape[1] == w.shape[1],
+          f"linear: a {tuple(a.shape)} and w {tuple(w.shape)} do not share the inner size")
+    return torch.matmul(a, w.t())
+
+
+def linear_thin(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    """bfloat16 operands, few rows: the weight is streamed once."""
+    return linear_exact(a, w, out_dtype)
+
+
+def attention(q, k_cache, v_cache, block_table, ctx, nh: int, nkv: int, hd: int, scale: float, window: int | None):
+    """The step's queries over the cache; picks the kernel by element type, head size and step shape."""
+    return attention_exact(q, k_cache, v_cache, block_table, ctx.seq_slot, ctx.seq_start, ctx.seq_new, ctx.cu_new,
+                           ctx.max_new, nh, nkv, hd, scale, window)

@@ -1,0 +1,7 @@
+"""The parts that layers are put together from: norms, position encodings, mixers, feed-forwards,
+blocks, and the embedding and head at the two ends."""
+from .base import (CATEGORIES, Builder, StepContext, cache_needs, make_context, part_class, register_part)
+from . import norm, position, attention, feedforward, block, embedding  # noqa: F401  (registers the kinds)
+from .linear import Linear
+
+__all__ = ["CATEGORIES", "Builder", "StepContext", "cache_needs", "make_context", "part_class", "register_part", "Linear"]

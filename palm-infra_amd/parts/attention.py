@@ -1,0 +1,68 @@
+"""Causal grouped-query attention over the cache, with optional per-head RMSNorm of q and k, a
+rotation of both, and an optional window.
+
+Order of operations as the reference builds it (models/qwen3.py:290-349): one joined q/k/v projection;
+per-head norm of q and k over head_dim with one weight vector for all heads; rotation of q and k; the
+step's k and v are appended to the cache; every query attends the cached keys of its own sequence up
+to its own position with scale ``scale`` (head_dim^-0.5 for Qwen3); head h reads kv head
+h // (heads / kv_heads) (kernels/attention.cpp:1161); output projection.  No bias anywhere.
+"""
+from __future__ import annotations
+
+import torch
+
+from ..cache import KVNeed
+from ..kernels import ops
+from .base import register_part
+from .linear import Linear
+from .position import PAIRINGS
+
+
+@register_part("mixer", "attention")
+class Attention:
+    def __init__(self, spec, builder):
+        p = spec.params
+        self.hidden = int(p["hidden_size"])
+        self.nh, self.nkv, self.hd = int(p["num_heads"]), int(p["num_kv_heads"]), int(p["head_dim"])
+        self.scale = float(p["scale"])
+        self.window = int(p["window"]) if p.get("window") else None
+        if self.nh % self.nkv:
+            raise ValueError(f"{self.nh} heads are not a multiple of {self.nkv} kv heads")
+        self.qkv = Linear(builder.tensor(spec, "qkv"))
+        self.out = Linear(builder.tensor(spec, "out"))
+        if self.qkv.weight.shape != ((self.nh + 2 * self.nkv) * self.hd, self.hidden):
+            raise ValueError(f"attention: joined q/k/v weight {tuple(self.qkv.weight.shape)} does not fit "
+                             f"{self.nh}+2*{self.nkv} heads of {self.hd} over hidden {self.hidden}")
+        if self.out.weight.shape != (self.hidden, self.nh * self.hd):
+            raise ValueError(f"attention: output weight {tuple(self.out.weight.shape)} does not fit")
+        self.q_norm = builder.build(spec.parts["q_norm"]) if "q_norm" in spec.parts else None
+        self.k_norm = builder.build(spec.parts["k_norm"]) if "k_norm" in spec.parts else None
+        if (self.q_norm is None) != (self.k_norm is None):
+            raise ValueError("attention: q_norm and k_norm come together")
+        if self.q_norm is not None and (self.q_norm.width != self.hd or self.k_norm.width != self.hd
+                                        or self.q_norm.eps != self.k_norm.eps):
+            raise ValueError("attention: q_norm and k_norm must be over head_dim with one eps")
+        self.position = builder.build(spec.parts["position"]) if "position" in spec.parts else None
+        self.dtype = builder.dtype
+
+    @staticmethod
+    def cache_needs(spec):
+        p = spec.params
+        return [KVNeed(int(p["num_kv_heads"]), int(p["head_dim"]), int(p["window"]) if p.get("window") else None)]
+
+    def forward(self, h: torch.Tensor, ctx) -> torch.Tensor:
+        lc = ctx.layer_cache
+        if lc is None or lc.kv is None:
+            raise RuntimeError("attention needs the keys and values of its layer; the step gave it no cache")
+        qkv = self.qkv(h)
+        tables = self.position.tables(ctx) if self.position is not None else None
+        cos, sin = tables if tables is not None else (None, None)
+        q = ops.qk_norm_rope_store(
+            qkv, self.nh, self.nkv, self.hd, ctx.positions,
+            q_norm_w=self.q_norm.weight if self.q_norm else None, k_norm_w=self.k_norm.weight if self.k_norm else None,
+            eps=self.q_norm.eps if self.q_norm else 0.0, cos=cos, sin=sin,
+            rotary_dim=self.position.rotary_dim if tables is not None else 0,
+            pairing=PAIRINGS[self.position.pairing] if tables is not None else 0,
+            k_cache=lc.k, v_cache=lc.v, block_table=lc.kv.table_dev, tok_slot=ctx.tok_slot, write_cache=lc.writes)
+        o = ops.attention(q, lc.k, lc.v, lc.kv.table_dev, ctx, self.nh, self.nkv, self.hd, self.scale, self.window)
+        return self.out(o)

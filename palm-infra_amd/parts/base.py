@@ -1,0 +1,118 @@
+"""What every part has in common: a registry by (category, kind), the builder that turns a
+description into parts, and the context a step hands to them.
+
+A part is built from its ``PartSpec`` alone (sizes, constants, parameters, sub-parts); it does not know
+which model it is in.  Interfaces, by category:
+
+  norm          ``__call__(x, delta=None, update=False, rows=None, out_dtype=None)`` -> normed rows.  x is the
+                float32 residual stream [n, width]; ``delta`` is a branch output still to be added (added in
+                32-bit; with ``update`` the sum is written back to x); ``rows`` selects rows.
+  position      ``tables(ctx)`` -> (cos, sin) float32 [n, rotary_dim/2] for the step's tokens, or None; fields
+                ``rotary_dim`` and ``pairing`` ("half_split" | "interleaved").
+  mixer         ``forward(h, ctx)`` -> branch output [n, hidden]; ``cache_needs(spec)`` (static) -> what it
+                keeps per sequence (``KVNeed`` / ``StateNeed``); reads ``ctx.layer_cache``.
+  feed_forward  ``forward(h, ctx)`` -> branch output [n, hidden].
+  block         ``forward(x, pending, ctx)`` -> (x, pending): the arrangement of norms, mixer and feed-forward
+                around the residual stream; ``pending`` is a branch output that the next norm adds.
+  embedding     ``forward(token_ids)`` -> float32 [n, hidden].
+  head          ``forward(h)`` -> float32 logits [rows, vocab].
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+import torch
+
+from ..config.spec import PartSpec
+
+CATEGORIES = ("norm", "position", "mixer", "feed_forward", "block", "embedding", "head")
+_REGISTRY: dict[tuple[str, str], type] = {}
+
+
+def register_part(category: str, kind: str):
+    """Class decorator: make ``kind`` available under ``category``.  Registering a kind again replaces
+    it (a test may swap a toy part in and out)."""
+    if category not in CATEGORIES:
+        raise ValueError(f"part category {category!r} is not one of {CATEGORIES}")
+
+    def deco(cls):
+        _REGISTRY[(category, kind)] = cls
+        cls.category, cls.kind = category, kind
+        return cls
+    return deco
+
+
+def part_class(category: str, kind: str) -> type:
+    try:
+        return _REGISTRY[(category, kind)]
+    except KeyError:
+        known = sorted(k for c, k in _REGISTRY if c == category)
+        raise KeyError(f"no {category} part of kind {kind!r}; registered: {', '.join(known)}") from None
+
+
+def cache_needs(spec: PartSpec) -> list:
+    """What the part described by ``spec`` keeps per sequence (blocks pass their mixer's needs on)."""
+    cls = part_class(spec.category, spec.kind)
+    fn = getattr(cls, "cache_needs", None)
+    return list(fn(spec)) if fn else []
+
+
+class Builder:
+    """Builds parts from descriptions; hands them their parameters and the run's precision."""
+
+    def __init__(self, weights, dtype: torch.dtype, device):
+        self.weights, self.dtype, self.device = weights, dtype, torch.device(device)
+
+    def build(self, spec: PartSpec):
+        return part_class(spec.category, spec.kind)(spec, self)
+
+    def tensor(self, spec: PartSpec, name: str) -> torch.Tensor:
+        return self.weights.get(spec.tensors[name])
+
+
+@dataclass
+class StepContext:
+    """The tokens of one step, packed: sequence b brings ``seq_new[b]`` tokens, rows
+    ``cu_new[b] .. cu_new[b+1]`` of every [n, ...] tensor, at positions ``seq_start[b] ..``."""
+    n_tokens: int
+    n_seqs: int
+    max_new: int                 # the longest run of new tokens in the step
+    max_total: int               # the longest sequence after the step
+    dtype: torch.dtype           # element type of activations
+    token_ids: torch.Tensor      # int32 [n]
+    positions: torch.Tensor      # int32 [n]
+    tok_slot: torch.Tensor       # int32 [n]   the cache slot of each token's sequence
+    seq_slot: torch.Tensor       # int32 [B]
+    seq_start: torch.Tensor      # int32 [B]   length before the step
+    seq_new: torch.Tensor        # int32 [B]
+    cu_new: torch.Tensor         # int32 [B + 1]
+    is_decode: bool = False      # every sequence brings exactly one token
+    layer_cache: object = None   # the LayerCache of the run-order entry that is running
+    memo: dict = field(default_factory=dict)   # what parts make once per step (rotation tables)
+    host: dict = field(default_factory=dict)   # the same facts as Python lists, for parts that plan on the host
+
+
+def make_context(slots, starts, new_tokens, dtype, device, max_total=None) -> StepContext:
+    """A context from host lists: ``new_tokens[b]`` is the list of token ids of sequence b."""
+    counts = [len(t) for t in new_tokens]
+    ids = [t for seq in new_tokens for t in seq]
+    pos = [starts[b] + j for b in range(len(slots)) for j in range(counts[b])]
+    tslot = [slots[b] for b in range(len(slots)) for _ in range(counts[b])]
+    cu = [0]
+    for c in counts:
+        cu.append(cu[-1] + c)
+    n, B = len(ids), len(slots)
+    # one transfer for all index arrays
+    flat = torch.tensor(ids + pos + tslot + list(slots) + list(starts) + counts + cu, dtype=torch.int32).to(device)
+    o = 0
+    parts = []
+    for size in (n, n, n, B, B, B, B + 1):
+        parts.append(flat[o:o + size])
+        o += size
+    return StepContext(
+        n_tokens=n, n_seqs=B, max_new=max(counts) if counts else 0,
+        max_total=max_total if max_total is not None else max((s + c for s, c in zip(starts, counts)), default=0),
+        dtype=dtype, token_ids=parts[0], positions=parts[1], tok_slot=parts[2], seq_slot=parts[3], seq_start=parts[4],
+        seq_new=parts[5], cu_new=parts[6], is_decode=all(c == 1 for c in counts),
+        host={"slots": list(slots), "starts": list(starts), "counts": counts, "cu": cu},
+    )

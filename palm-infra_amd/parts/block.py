@@ -1,0 +1,28 @@
+"""The arrangement of a layer's parts around the residual stream.
+
+``pre_norm``: x += mixer(norm(x)); x += feed_forward(norm(x)) (models/qwen3.py:254-287).  The residual
+stream x is float32; a branch's output is not added at once but handed on as ``pending``, and the next
+norm adds it in the same pass in which it norms (the sum is made in 32-bit and written back to x).
+"""
+from __future__ import annotations
+
+from .base import cache_needs, register_part
+
+
+@register_part("block", "pre_norm")
+class PreNormBlock:
+    def __init__(self, spec, builder):
+        self.mixer_norm = builder.build(spec.parts["mixer_norm"])
+        self.mixer = builder.build(spec.parts["mixer"])
+        self.feed_forward_norm = builder.build(spec.parts["feed_forward_norm"])
+        self.feed_forward = builder.build(spec.parts["feed_forward"])
+
+    @staticmethod
+    def cache_needs(spec):
+        return cache_needs(spec.parts["mixer"])
+
+    def forward(self, x, pending, ctx):
+        h = self.mixer_norm(x, delta=pending, update=pending is not None)
+        a = self.mixer.forward(h, ctx)
+        h = self.feed_forward_norm(x, delta=a, update=True)
+        return x, self.feed_forward.forward(h, ctx)

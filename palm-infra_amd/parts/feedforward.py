@@ -1,0 +1,24 @@
+"""The gated feed-forward: down( silu(gate(h)) * up(h) ), silu(z) = z / (1 + exp(-z)), with gate and up
+joined into one [2I, H] product (models/qwen3.py:276-287; kernels/elementwise.cpp:529-583)."""
+from __future__ import annotations
+
+import torch
+
+from ..kernels import ops
+from .base import register_part
+from .linear import Linear
+
+
+@register_part("feed_forward", "gated_silu")
+class GatedSiluFeedForward:
+    def __init__(self, spec, builder):
+        self.hidden = int(spec.params["hidden_size"])
+        self.inter = int(spec.params["intermediate_size"])
+        self.gate_up = Linear(builder.tensor(spec, "gate_up"))
+        self.down = Linear(builder.tensor(spec, "down"))
+        if self.gate_up.weight.shape != (2 * self.inter, self.hidden) or self.down.weight.shape != (self.hidden, self.inter):
+            raise ValueError(f"feed-forward: weights {tuple(self.gate_up.weight.shape)}, {tuple(self.down.weight.shape)} "
+                             f"do not fit hidden {self.hidden}, intermediate {self.inter}")
+
+    def forward(self, h: torch.Tensor, ctx) -> torch.Tensor:
+        return self.down(ops.swiglu(self.gate_up(h)))

@@ -1,0 +1,32 @@
+"""y = x W^T for a weight in the checkpoint's [out, in] layout: the one place that picks the kernel.
+
+  float32 run, or a 32-bit weight under bfloat16 activations   the exact FMA kernel
+  bfloat16 x bfloat16, few rows (decode)                        the matrix-core kernel for thin products
+  bfloat16 x bfloat16, many rows (prompts)                      the BLAS library, as the reference's GPU path
+                                                                does for its products (engine/cuda_matmul.cu:245-260)
+"""
+from __future__ import annotations
+
+import torch
+
+from ..kernels import ops
+
+# above this many rows the library's large tiles win over streaming the weight once per 64 rows
+THIN_ROWS = 64
+
+
+class Linear:
+    def __init__(self, weight: torch.Tensor):
+        if weight.dim() != 2:
+            raise ValueError(f"a linear weight must be [out, in], got {tuple(weight.shape)}")
+        self.weight = weight
+        self.out_features, self.in_features = weight.shape
+
+    def __call__(self, x: torch.Tensor, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+        out_dtype = out_dtype or x.dtype
+        w = self.weight
+        if x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16:
+            if x.shape[0] <= THIN_ROWS or out_dtype != torch.bfloat16:
+                return ops.linear_thin(x, w, out_dtype)
+            return ops.linear_library(x, w)
+        return ops.linear_exact(x, w, out_dtype)

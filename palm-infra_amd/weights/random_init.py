@@ -1,0 +1,56 @@
+"""The random-weights mode: write a model folder (config.json, model.safetensors) from a
+configuration and a seed.
+
+The reference has this only as a test fixture (tests/run_tiny_qwen3_cpu_e2e.py:52-95).  Here matrices
+and the embedding are N(0, 0.02) and norm weights 1 + N(0, 0.02), as each parameter's description
+says.  A tensor's values depend on the seed and on the tensor's name only, so a model with more layers
+starts with the same layers.
+"""
+from __future__ import annotations
+
+import hashlib
+import json
+from pathlib import Path
+
+import torch
+
+from ..config.registry import config_from_dict
+from .safetensors_io import write_safetensors
+
+_STORE = {"bfloat16": torch.bfloat16, "float32": torch.float32, "float16": torch.float16}
+
+
+def _tensor_seed(seed: int, name: str) -> int:
+    digest = hashlib.sha256(f"{int(seed)}:{name}".encode()).digest()
+    return int.from_bytes(digest[:8], "little") & 0x7FFFFFFFFFFFFFFF
+
+
+def random_tensors(spec, seed: int, dtype: str = "bfloat16") -> dict[str, torch.Tensor]:
+    if dtype not in _STORE:
+        raise ValueError(f"dtype {dtype!r} is not one of {sorted(_STORE)}")
+    out = {}
+    for ref in spec.tensor_refs():
+        for name, shape in zip(ref.names, ref.shapes):
+            if ref.role == "integer":
+                out[name] = torch.zeros(shape, dtype=torch.int32)
+                continue
+            g = torch.Generator()
+            g.manual_seed(_tensor_seed(seed, name))
+            _, mean, std = ref.init
+            t = torch.empty(shape, dtype=torch.float32).normal_(mean, std, generator=g)
+            out[name] = t.to(_STORE[dtype])
+    return out
+
+
+def write_random_model(config, seed: int, out_dir, dtype: str = "bfloat16") -> Path:
+    """``config`` is a typed configuration or the dict of a config.json."""
+    if isinstance(config, dict):
+        config = config_from_dict(config)
+    out_dir = Path(out_dir)
+    out_dir.mkdir(parents=True, exist_ok=True)
+    raw = config.to_dict()
+    raw["torch_dtype"] = dtype
+    (out_dir / "config.json").write_text(json.dumps(raw, indent=2))
+    write_safetensors(out_dir / "model.safetensors", random_tensors(config.spec(), seed, dtype),
+                      metadata={"format": "pt", "seed": seed})
+    return out_dir
