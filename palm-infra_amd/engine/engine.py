@@ -170,3 +170,20 @@ class Engine:
     def memory_report(self) -> dict:
         return {"weights_bytes": self.model.weights.nbytes(), "cache_bytes": self.cache.nbytes(),
                 "cache_tokens": self.cache.max_tokens, "slots": self.cache.max_seqs}
+
+    # ---- generation --------------------------------------------------------------------------
+    def generate(self, prompts, sampling=None, max_new_tokens: int = 2048, stop_token_ids=None, ignore_eos: bool = False,
+                 max_batch: int = 64, on_token=None):
+        """Token ids in, token ids out: ``prompts`` is a list of lists of ids; returns (results, metrics),
+        the results in the order of the prompts.  ``stop_token_ids`` defaults to config.json's
+        ``eos_token_id``; ``ignore_eos`` switches stopping off, as the reference's benchmark does
+        (examples/bench.cpp:583)."""
+        from ..sampling import DeviceSampler, SamplingParams
+        from .generate import generate
+        sampler = DeviceSampler(sampling or SamplingParams())
+        if ignore_eos:
+            stop = ()
+        else:
+            stop = self.spec.stop_token_ids if stop_token_ids is None else stop_token_ids
+        return generate(self, sampler, prompts, max_new_tokens=max_new_tokens, stop_token_ids=stop, max_batch=max_batch,
+                        on_token=on_token, sync=torch.cuda.synchronize)

@@ -1,0 +1,173 @@
+"""The generation loop above the step function.
+
+The reference generates for one sequence: reset, ``prefill`` (which yields the first token), then
+``decode`` until the stop token or ``max_new_tokens``; the stop token is part of the output; time is
+split into prefill and decode (examples/cli_common.cpp:438-530) and the metrics are
+``decode_tokens = generated - 1``, ``ttft = prefill_ms``, ``tpot = decode_ms / decode_tokens``,
+``prefill_tps``, ``decode_tps`` (examples/cli_common.cpp:418-436).  Here the same loop runs over
+batches of requests with unequal prompts: all prompts of a batch in one step, then one token for each
+sequence that is still running; a sequence that ends leaves the batch at once and its slot goes back;
+batches follow one another until every request is served.
+
+The loop only decides; the engine steps and the sampler chooses.  Both are handed in, so the decisions
+can be tested with stand-ins.
+"""
+from __future__ import annotations
+
+import time
+from dataclasses import dataclass, field
+
+from ..cache.pool import PAGE_TOKENS, pages_for
+from ..sampling import SequenceSampling
+from .engine import StepEntry
+
+
+@dataclass
+class GenerationResult:
+    """Of one request.  ``finish_reason``: "stop" (a stop token came, and is the last token), "length"
+    (max_new_tokens), "context" (the sequence filled the longest context the cache takes)."""
+    prompt_tokens: int
+    token_ids: list = field(default_factory=list)
+    finish_reason: str = ""
+    prefill_ms: float = 0.0
+    decode_ms: float = 0.0
+
+    @property
+    def hit_eos(self) -> bool:
+        return self.finish_reason == "stop"
+
+
+@dataclass
+class GenerationMetrics:
+    prompt_tokens: int = 0
+    generated_tokens: int = 0
+    decode_tokens: int = 0
+    ttft_ms: float = 0.0
+    tpot_ms: float = 0.0
+    prefill_tps: float = 0.0
+    decode_tps: float = 0.0
+    total_ms: float = 0.0
+
+
+def compute_metrics(results, prefill_ms: float, decode_ms: float) -> GenerationMetrics:
+    """The reference's definitions (examples/cli_common.cpp:418-436), summed over the requests of a run:
+    every request's first token comes from the prefill, the others from decode steps."""
+    m = GenerationMetrics()
+    m.prompt_tokens = sum(r.prompt_tokens for r in results)
+    m.generated_tokens = sum(len(r.token_ids) for r in results)
+    m.decode_tokens = sum(max(len(r.token_ids) - 1, 0) for r in results)
+    m.ttft_ms = prefill_ms
+    m.tpot_ms = decode_ms / m.decode_tokens if m.decode_tokens > 0 and decode_ms > 0 else 0.0
+    m.prefill_tps = 1000.0 * m.prompt_tokens / prefill_ms if prefill_ms > 0 else 0.0
+    m.decode_tps = 1000.0 * m.decode_tokens / decode_ms if decode_ms > 0 else 0.0
+    m.total_ms = prefill_ms + decode_ms
+    return m
+
+
+class RequestTooLong(ValueError):
+    pass
+
+
+def plan_batches(prompt_lengths, max_new_tokens: int, max_batch: int, cache_tokens: int, max_seq_tokens: int):
+    """Which requests run together: in the order given, as many as ``max_batch`` allows and as the cache
+    can hold when every sequence of the batch grows to its full length (pages of PAGE_TOKENS each).
+    Returns lists of request indices."""
+    if max_batch < 1:
+        raise ValueError("max_batch must be at least 1")
+    batches, current, held = [], [], 0
+    for i, n in enumerate(prompt_lengths):
+        if n < 1:
+            raise RequestTooLong(f"request {i}: the prompt is empty")
+        if n > max_seq_tokens:
+            raise RequestTooLong(f"request {i}: a prompt of {n} tokens exceeds the longest sequence the cache takes "
+                                 f"({max_seq_tokens})")
+        full = min(n + max_new_tokens, max_seq_tokens)
+        need = pages_for(full) * PAGE_TOKENS
+        if need > cache_tokens:
+            raise RequestTooLong(f"request {i}: {full} tokens do not fit a cache of {cache_tokens}")
+        if current and (len(current) >= max_batch or held + need > cache_tokens):
+            batches.append(current)
+            current, held = [], 0
+        current.append(i)
+        held += need
+    if current:
+        batches.append(current)
+    return batches
+
+
+def generate(engine, sampler, prompts, max_new_tokens: int = 2048, stop_token_ids=(), max_batch: int = 64,
+             on_token=None, timer=time.perf_counter, sync=None):
+    """Generate for every prompt (a list of token ids); results come in the order of the prompts.
+
+    ``engine``: ``open() -> slot``, ``close(slot)``, ``step(entries) -> logits [rows, vocab]``,
+    ``cache.max_tokens``, ``cache.max_seq_tokens``.  ``sampler``: ``sample(logits, states) -> ids`` (anything
+    with ``.tolist()``).  ``on_token(request index, token id)`` is called for every token as it comes.
+    ``sync()`` waits for the device before a time is taken.  Returns (results, metrics).
+    """
+    if max_new_tokens < 1:
+        raise ValueError("max_new_tokens must be >= 1")
+    prompts = [list(map(int, p)) for p in prompts]
+    stop = set(int(t) for t in stop_token_ids)
+    max_seq = engine.cache.max_seq_tokens
+    results = [GenerationResult(prompt_tokens=len(p)) for p in prompts]
+    batches = plan_batches([len(p) for p in prompts], max_new_tokens, max_batch, engine.cache.max_tokens, max_seq)
+    sync = sync or (lambda: None)
+    total_prefill = total_decode = 0.0
+
+    for batch in batches:
+        slots = {i: engine.open() for i in batch}
+        states = {i: SequenceSampling(stream=i) for i in batch}
+        try:
+            # ---- all prompts in one step; it yields each request's first token ----
+            sync()
+            t0 = timer()
+            logits = engine.step([StepEntry(slots[i], prompts[i], [len(prompts[i]) - 1]) for i in batch])
+            for i in batch:
+                states[i].accept(prompts[i])
+            tokens = sampler.sample(logits, [states[i] for i in batch]).tolist()
+            sync()
+            prefill_ms = (timer() - t0) * 1000.0
+            total_prefill += prefill_ms
+
+            def take(i, tok):
+                """Record a token; True if the sequence goes on."""
+                r = results[i]
+                r.token_ids.append(tok)
+                if on_token:
+                    on_token(i, tok)
+                if tok in stop:
+                    r.finish_reason = "stop"
+                elif len(r.token_ids) >= max_new_tokens:
+                    r.finish_reason = "length"
+                elif len(prompts[i]) + len(r.token_ids) > max_seq:
+                    # the next step would have to hold one token more than the cache takes
+                    r.finish_reason = "context"
+                if r.finish_reason:
+                    engine.close(slots.pop(i))
+                    return False
+                return True
+
+            live = []
+            for i, tok in zip(batch, tokens):
+                results[i].prefill_ms = prefill_ms
+                if take(i, int(tok)):
+                    live.append(i)
+
+            # ---- one token for each sequence that still runs ----
+            t1 = timer()
+            while live:
+                last = {i: results[i].token_ids[-1] for i in live}
+                logits = engine.step([StepEntry(slots[i], [last[i]], [0]) for i in live])
+                for i in live:
+                    states[i].accept([last[i]])
+                tokens = sampler.sample(logits, [states[i] for i in live]).tolist()
+                live = [i for i, tok in zip(live, tokens) if take(i, int(tok))]
+            sync()
+            decode_ms = (timer() - t1) * 1000.0
+            total_decode += decode_ms
+            for i in batch:
+                results[i].decode_ms = decode_ms
+        finally:
+            for slot in slots.values():      # only after a fault: every sequence that ended has left already
+                engine.close(slot)
+    return results, compute_metrics(results, total_prefill, total_decode)

@@ -1,0 +1,170 @@
+"""The cache's bookkeeping on the host: no slot or page lost, held twice or freed twice (no GPU)."""
+import random
+
+import pytest
+import torch
+
+from palm_infra_amd.cache import (PAGE_TOKENS, CacheFull, CacheMisuse, FreeList, KVNeed, ModelCache, PageTable,
+                                  StateNeed, pages_for)
+
+
+def test_free_list_hands_out_each_number_once_and_lowest_first():
+    f = FreeList(4, "slot")
+    assert [f.take() for _ in range(4)] == [0, 1, 2, 3]
+    with pytest.raises(CacheFull):
+        f.take()
+    f.give_back(2)
+    f.give_back(0)
+    with pytest.raises(CacheMisuse, match="not held"):
+        f.give_back(2)
+    with pytest.raises(CacheMisuse, match="does not exist"):
+        f.give_back(9)
+    assert f.take() == 0 and f.take() == 2          # what was given back is used again, lowest first
+    f.check()
+
+
+def test_take_many_takes_nothing_if_it_cannot_take_all():
+    f = FreeList(3, "page")
+    f.take()
+    with pytest.raises(CacheFull):
+        f.take_many(3)
+    assert f.free_count == 2
+    f.check()
+
+
+def _cache(needs=None, shares=None, max_tokens=64 * 12, max_seqs=None, max_positions=4096):
+    needs = needs if needs is not None else [[KVNeed(2, 16)], [KVNeed(2, 16)]]
+    shares = shares if shares is not None else [None] * len(needs)
+    return ModelCache(needs, shares, max_tokens, max_seqs, max_positions, torch.float32, "cpu")
+
+
+def test_pages_follow_lengths_and_come_back():
+    c = _cache()
+    a, b = c.open(), c.open()
+    c.reserve([(a, 70), (b, 1)])
+    c.commit([(a, 70), (b, 1)])
+    g = c.kv_groups[0]
+    assert g.table.slot_pages[a] == [0, 1] and g.table.slot_pages[b] == [2]
+    assert c.lengths[a] == 70 and c.lengths[b] == 1
+    for _ in range(58):                              # 70 -> 128: still two pages
+        c.reserve([(a, 1)]); c.commit([(a, 1)])
+    assert len(g.table.slot_pages[a]) == 2
+    c.reserve([(a, 1)]); c.commit([(a, 1)])          # 129: a third
+    assert g.table.slot_pages[a] == [0, 1, 3]
+    assert g.table_dev[a, :4].tolist() == [0, 1, 3, g.pad_page]
+    c.close(a)
+    assert g.table.pages.free_count == 12 - 1
+    c.check()
+    d = c.open()
+    assert d == a                                    # the slot is used again ...
+    c.reserve([(d, 10)])
+    assert g.table.slot_pages[d] == [0]              # ... and so is its first page, uncleared
+    with pytest.raises(CacheMisuse):
+        c.close(7)
+    c.close(d)
+    with pytest.raises(CacheMisuse):
+        c.close(d)
+    c.check()
+
+
+def test_a_step_that_does_not_fit_takes_nothing():
+    c = _cache(max_tokens=64 * 4)
+    a, b = c.open(), c.open()
+    c.reserve([(a, 64)]); c.commit([(a, 64)])
+    free = c.kv_groups[0].table.pages.free_count
+    with pytest.raises(CacheFull, match="more pages"):
+        c.reserve([(a, 65), (b, 100)])               # 2 + 2 pages wanted, 3 free
+    assert c.kv_groups[0].table.pages.free_count == free and c.lengths[a] == 64
+    with pytest.raises(CacheFull, match="longest sequence"):
+        c.reserve([(b, 64 * 4 + 1)])
+    with pytest.raises(CacheMisuse, match="not open"):
+        c.reserve([(3, 1)])
+    c.check()
+
+
+def test_longest_sequence_is_bounded_by_positions_and_by_the_cache():
+    assert _cache(max_tokens=64 * 12, max_positions=100).max_seq_tokens == 100
+    assert _cache(max_tokens=64 * 2, max_positions=4096).max_seq_tokens == 128
+    assert _cache(max_tokens=65).max_tokens == 128   # rounded up to whole pages
+
+
+def test_groups_have_storage_of_their_own():
+    needs = [[KVNeed(2, 16)], [KVNeed(1, 32, window=100)], [KVNeed(2, 16)], [KVNeed(1, 32, window=100), StateNeed("s", (3, 2))]]
+    c = _cache(needs)
+    assert len(c.kv_groups) == 2 and len(c.state_groups) == 1
+    full, win = c.kv_groups
+    assert full.k.shape == (2, 13, 2, PAGE_TOKENS, 16) and win.k.shape == (2, 13, 1, PAGE_TOKENS, 32)
+    assert full.k.data_ptr() != win.k.data_ptr() and full.table is not win.table
+    lc = c.layer_caches
+    assert lc[0].kv is full and lc[2].kv is full and (lc[0].kv_entry, lc[2].kv_entry) == (0, 1)
+    assert lc[1].kv is win and lc[3].kv is win and lc[3].states["s"].shape == (c.max_seqs + 1, 3, 2)
+    assert lc[0].k.data_ptr() != lc[2].k.data_ptr()
+
+
+def test_a_window_gives_pages_back_as_the_sequence_grows():
+    c = _cache([[KVNeed(1, 16, window=70)], [KVNeed(1, 16)]])
+    win, full = c.kv_groups
+    s = c.open()
+    c.reserve([(s, 200)]); c.commit([(s, 200)])
+    # the next query sits at 200 and reads keys 131..200: pages 0 and 1 (positions 0..127) are out of reach
+    assert win.table.slot_pages[s] == [-1, -1, 2, 3] and full.table.slot_pages[s] == [0, 1, 2, 3]
+    assert win.table_dev[s, :4].tolist() == [win.pad_page, win.pad_page, 2, 3]
+    assert win.table.pages.free_count == 12 - 2
+    c.reserve([(s, 1)]); c.commit([(s, 1)])          # 201: first key needed is 132, page 2 still is
+    assert win.table.slot_pages[s][2] == 2
+    c.check()
+    c.close(s)
+    assert win.table.pages.free_count == 12 and full.table.pages.free_count == 12
+
+
+def test_state_is_zero_for_a_new_sequence():
+    c = _cache([[StateNeed("h", (4,))]])
+    s = c.open()
+    c.state_groups[0].data[0, s] = 5.0
+    c.close(s)
+    assert c.open() == s
+    assert float(c.state_groups[0].data[0, s].abs().sum()) == 0.0
+
+
+def test_an_entry_can_read_another_entrys_cache():
+    c = _cache([[KVNeed(2, 16)], []], shares=[None, 0])
+    a, b = c.layer_caches
+    assert b.kv is a.kv and b.kv_entry == a.kv_entry and a.writes and not b.writes
+    assert c.kv_groups[0].k.shape[0] == 1
+
+
+def test_random_traffic_keeps_the_books():
+    rng = random.Random(0)
+    c = _cache([[KVNeed(2, 16)], [KVNeed(2, 16, window=90)]], max_tokens=64 * 40, max_seqs=9)
+    live = {}
+    for step in range(600):
+        op = rng.random()
+        if op < 0.25 and len(live) < 9:
+            live[c.open()] = 0
+        elif op < 0.4 and live:
+            s = rng.choice(list(live))
+            c.close(s)
+            del live[s]
+        elif live:
+            batch = rng.sample(list(live), rng.randint(1, len(live)))
+            growth = [(s, rng.choice([1, 1, 1, 5, 64, 130])) for s in batch]
+            try:
+                c.reserve(growth)
+            except CacheFull:
+                continue
+            c.commit(growth)
+            for s, n in growth:
+                live[s] += n
+        c.check()
+        for s, n in live.items():
+            assert c.lengths[s] == n
+            for g in c.kv_groups:
+                pages = g.table.slot_pages[s]
+                assert len(pages) >= pages_for(n)
+                first = 0 if g.need.window is None else max(0, n - g.need.window + 1) // PAGE_TOKENS
+                assert all(p >= 0 for p in pages[first:pages_for(n)])     # every page a query can reach is there
+                assert g.table_dev[s, :len(pages)].tolist() == [p if p >= 0 else g.pad_page for p in pages]
+    for s in list(live):
+        c.close(s)
+    c.check()
+    assert all(g.table.pages.free_count == g.n_pages for g in c.kv_groups) and c.slots.free_count == 9

@@ -1,0 +1,186 @@
+"""The engine against the plain implementation under every way of cutting and batching the same
+requests: each alone and whole; whole minus the last 32 tokens, which then come one by one; batches of
+unequal lengths whose shorter requests end earlier, one batch after another so that slots and pages are
+used again; long decoding; the first tokens of a sequence.  In float32 and in bfloat16."""
+import pytest
+import torch
+
+import plain_qwen3 as P
+import tiny
+
+pytestmark = pytest.mark.gpu
+
+CASES = [(name, dtype) for name in ("A", "B", "C") for dtype in ("float32", "bfloat16")]
+LENGTHS = {"A": [5, 17, 9, 64, 100, 33], "B": [1, 31, 12, 64, 65, 200], "C": [48, 7, 129, 2, 300, 70]}
+
+_engines = {}
+_refs = {}
+
+
+def engine_for(model_dirs, name, dtype):
+    from palm_infra_amd.engine import Engine
+    key = (name, dtype)
+    if key not in _engines:
+        _engines[key] = Engine.from_dir(model_dirs[name][dtype], dtype=dtype, max_tokens=64 * 24)
+    return _engines[key]
+
+
+def reference(model_dirs, name, dtype, ids):
+    """Plain logits [n, V] of one whole sequence, from the same stored weights."""
+    key = (name, dtype, tuple(ids))
+    if key not in _refs:
+        cfg, w = P.read_model(model_dirs[name][dtype])
+        _refs[key] = P.logits(cfg, w, ids)
+    return _refs[key]
+
+
+@pytest.mark.parametrize("name,dtype", CASES)
+def test_each_request_alone_and_whole(model_dirs, name, dtype):
+    from palm_infra_amd.engine import StepEntry
+    eng = engine_for(model_dirs, name, dtype)
+    for ids in tiny.prompts(name, LENGTHS[name]):
+        slot = eng.open()
+        got = eng.step([StepEntry(slot, ids, list(range(len(ids))))])
+        eng.close(slot)
+        tiny.assert_logits_close(got, reference(model_dirs, name, dtype, ids), dtype, f"{name} whole {len(ids)}")
+    eng.cache.check()
+
+
+@pytest.mark.parametrize("name,dtype", CASES)
+def test_last_32_tokens_one_by_one(model_dirs, name, dtype):
+    from palm_infra_amd.engine import StepEntry
+    eng = engine_for(model_dirs, name, dtype)
+    for ids in tiny.prompts(name, [n for n in LENGTHS[name] if n > 32], seed=1):
+        ref = reference(model_dirs, name, dtype, ids)
+        cut = len(ids) - 32
+        slot = eng.open()
+        got = [eng.step([StepEntry(slot, ids[:cut], list(range(cut)))])]
+        for t in range(cut, len(ids)):
+            got.append(eng.step([StepEntry(slot, [ids[t]], [0])]))
+            assert eng.length(slot) == t + 1
+        eng.close(slot)
+        tiny.assert_logits_close(torch.cat(got), ref, dtype, f"{name} {len(ids)} tokens, last 32 one by one")
+
+
+@pytest.mark.parametrize("name,dtype", CASES)
+def test_batches_of_unequal_lengths_one_after_another(model_dirs, name, dtype):
+    """Two batches through the same slots and pages.  In a batch all prompts go in one step minus their
+    last `tail` tokens, which come one a step; a request with no tokens left ends (its slot goes back at
+    once), so later steps are smaller."""
+    from palm_infra_amd.engine import StepEntry
+    eng = engine_for(model_dirs, name, dtype)
+    held_before = eng.cache.kv_groups[0].table.pages.held_count
+    for round_no, (seed, tails) in enumerate([(2, [3, 0, 9, 1, 20, 5]), (3, [1, 12, 0, 2, 7, 30])]):
+        reqs = tiny.prompts(name, LENGTHS[name] if round_no == 0 else LENGTHS[name][::-1], seed=seed)
+        tails = [min(t, len(r) - 1) for t, r in zip(tails, reqs)]
+        slots = [eng.open() for _ in reqs]
+        assert sorted(slots) == list(range(len(reqs)))                # the second batch gets the first one's slots
+        got = {i: [] for i in range(len(reqs))}
+        cuts = [len(r) - t for r, t in zip(reqs, tails)]
+        out = eng.step([StepEntry(s, r[:c], list(range(c))) for s, r, c in zip(slots, reqs, cuts)])
+        o = 0
+        for i, c in enumerate(cuts):
+            got[i].append(out[o:o + c])
+            o += c
+        live = list(range(len(reqs)))
+        fed = list(cuts)
+        while True:
+            for i in [i for i in live if fed[i] == len(reqs[i])]:
+                eng.close(slots[i])
+                live.remove(i)
+            if not live:
+                break
+            out = eng.step([StepEntry(slots[i], [reqs[i][fed[i]]], [0]) for i in live])
+            for r, i in enumerate(live):
+                got[i].append(out[r:r + 1])
+                fed[i] += 1
+        for i, r in enumerate(reqs):
+            tiny.assert_logits_close(torch.cat(got[i]), reference(model_dirs, name, dtype, r), dtype,
+                                     f"{name} batch {round_no} request {i} ({len(r)} tokens, {tails[i]} one by one)")
+        eng.cache.check()
+        assert eng.cache.kv_groups[0].table.pages.held_count == held_before
+
+
+@pytest.mark.parametrize("name,dtype", [("C", "float32"), ("C", "bfloat16"), ("B", "float32")])
+def test_long_decoding(model_dirs, name, dtype):
+    """A short prompt, then every further token one by one, across several pages."""
+    from palm_infra_amd.engine import StepEntry
+    eng = engine_for(model_dirs, name, dtype)
+    n = 250 if name == "B" else 420
+    ids = tiny.prompts(name, [n], seed=4)[0]
+    ref = reference(model_dirs, name, dtype, ids)
+    other = eng.open()                                                # a neighbour that decodes along, then leaves
+    eng.step([StepEntry(other, ids[5:40], [])])
+    slot = eng.open()
+    got = [eng.step([StepEntry(slot, ids[:3], [0, 1, 2])])]
+    for t in range(3, n):
+        entries = [StepEntry(slot, [ids[t]], [0])]
+        if t < 200:
+            entries.insert(0, StepEntry(other, [ids[t]], []))
+        elif t == 200:
+            eng.close(other)
+        got.append(eng.step(entries))
+    eng.close(slot)
+    tiny.assert_logits_close(torch.cat(got), ref, dtype, f"{name} long decoding")
+    eng.cache.check()
+
+
+@pytest.mark.parametrize("name,dtype", CASES)
+def test_first_tokens_of_a_sequence(model_dirs, name, dtype):
+    """Prompts of one and two tokens, and a sequence fed one token at a time from its first."""
+    from palm_infra_amd.engine import StepEntry
+    eng = engine_for(model_dirs, name, dtype)
+    ids = tiny.prompts(name, [6], seed=5)[0]
+    ref = reference(model_dirs, name, dtype, ids)
+    a, b, c = eng.open(), eng.open(), eng.open()
+    first = eng.step([StepEntry(a, ids[:1], [0]), StepEntry(b, ids[:2], [0, 1]), StepEntry(c, ids[:6], [5])])
+    tiny.assert_logits_close(first[0:1], ref[0:1], dtype, "one-token prompt")
+    tiny.assert_logits_close(first[1:3], ref[0:2], dtype, "two-token prompt")
+    tiny.assert_logits_close(first[3:4], ref[5:6], dtype, "last place only")
+    got = [first[0:1]]
+    for t in range(1, 6):
+        got.append(eng.step([StepEntry(a, [ids[t]], [0])]))
+    tiny.assert_logits_close(torch.cat(got), ref, dtype, "token by token from the first")
+    for s in (a, b, c):
+        eng.close(s)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_padding_and_companions_change_no_result(model_dirs, dtype):
+    """The same request alone, among longer and shorter companions, and in another slot."""
+    from palm_infra_amd.engine import StepEntry
+    eng = engine_for(model_dirs, "B", dtype)
+    reqs = tiny.prompts("B", [40, 3, 130, 64], seed=6)
+    s = eng.open()
+    alone = eng.step([StepEntry(s, reqs[0], list(range(40)))]).cpu()
+    eng.close(s)
+    slots = [eng.open() for _ in range(4)]
+    order = [2, 1, 0, 3]
+    out = eng.step([StepEntry(slots[j], reqs[j], list(range(len(reqs[j])))) for j in order]).cpu()
+    for sl in slots:
+        eng.close(sl)
+    together = out[130 + 3:130 + 3 + 40]
+    if dtype == "float32":
+        # every output element adds its products in the same order whatever else is in the batch
+        assert torch.equal(alone, together)
+    else:
+        tiny.assert_logits_close(together, alone.double(), dtype, "with companions")
+
+
+def test_a_refused_step_changes_nothing(model_dirs):
+    from palm_infra_amd.cache import CacheFull
+    from palm_infra_amd.engine import StepEntry, StepError
+    eng = engine_for(model_dirs, "A", "float32")
+    s = eng.open()
+    ids = tiny.prompts("A", [10], seed=7)[0]
+    eng.step([StepEntry(s, ids[:4], [])])
+    for bad, err in (([StepEntry(s, [256], [0])], StepError), ([StepEntry(s, [1], [1])], StepError),
+                     ([StepEntry(s, [], [])], StepError), ([StepEntry(s, [1], []), StepEntry(s, [2], [])], StepError),
+                     ([StepEntry(31, [1], [])], StepError), ([StepEntry(s, [1] * 200, [])], CacheFull), ([], StepError)):
+        with pytest.raises(err):
+            eng.step(bad)
+        assert eng.length(s) == 4
+    got = eng.step([StepEntry(s, ids[4:], list(range(6)))])           # max_position_embeddings is 128: 200 more do not fit
+    tiny.assert_logits_close(got, reference(model_dirs, "A", "float32", ids)[4:], "float32", "after refused steps")
+    eng.close(s)
+    eng.cache.check()

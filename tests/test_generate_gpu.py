@@ -1,0 +1,133 @@
+"""Generation through the entry points: greedy tokens equal the plain implementation's; temperature
+sampling is reproducible and a sequence's tokens do not depend on its batch companions."""
+import subprocess
+import sys
+from pathlib import Path
+
+import pytest
+import torch
+
+import plain_qwen3 as P
+import tiny
+
+pytestmark = pytest.mark.gpu
+ROOT = Path(__file__).resolve().parent.parent
+
+
+@pytest.fixture(scope="module")
+def engine_a(model_dirs):
+    import palm_infra_amd
+    return palm_infra_amd.load(model_dirs["A"]["float32"], dtype="float32", max_tokens=64 * 16)
+
+
+def test_greedy_generation_equals_the_plain_implementation(model_dirs, engine_a):
+    from palm_infra_amd.sampling import GREEDY
+    cfg, w = P.read_model(model_dirs["A"]["float32"])
+    prompts = tiny.prompts("A", [5, 17, 9], seed=10)                 # the workload of the first tiny configuration
+    results, metrics = engine_a.generate(prompts, GREEDY, max_new_tokens=8, ignore_eos=True)
+    for p, r in zip(prompts, results):
+        assert r.token_ids == P.greedy(cfg, w, p, 8) and r.finish_reason == "length"
+    assert metrics.prompt_tokens == 31 and metrics.generated_tokens == 24 and metrics.decode_tokens == 21
+    assert metrics.prefill_tps > 0 and metrics.decode_tps > 0
+    engine_a.cache.check()
+    assert engine_a.cache.slots.held_count == 0
+
+
+def test_stop_tokens_end_sequences_early_and_batches_follow(model_dirs, engine_a):
+    from palm_infra_amd.sampling import GREEDY
+    cfg, w = P.read_model(model_dirs["A"]["float32"])
+    prompts = tiny.prompts("A", [6, 3, 11, 4, 8], seed=11)
+    free_run = [P.greedy(cfg, w, p, 12) for p in prompts]
+    stop = free_run[0][3]                                            # a token the first request emits fourth
+    results, _ = engine_a.generate(prompts, GREEDY, max_new_tokens=12, stop_token_ids=[stop], max_batch=2)
+    for p, r, free in zip(prompts, results, free_run):
+        expect = P.greedy(cfg, w, p, 12, stop=(stop,))
+        assert r.token_ids == expect
+        assert r.finish_reason == ("stop" if expect[-1] == stop else "length")
+    assert results[0].hit_eos and len(results[0].token_ids) <= 4
+    # config.json's eos_token_id is the default stop token
+    eos = 7
+    results, _ = engine_a.generate(prompts, GREEDY, max_new_tokens=12)
+    for p, r in zip(prompts, results):
+        assert r.token_ids == P.greedy(cfg, w, p, 12, stop=(eos,))
+    assert engine_a.cache.slots.held_count == 0
+
+
+def test_bfloat16_greedy_follows_the_oracle_where_the_margin_is_clear(model_dirs):
+    """bfloat16 may pick another token where two logits are close; on the oracle's own path (teacher
+    forcing) its argmax must agree wherever the oracle's top-2 margin exceeds the rounding bound."""
+    from palm_infra_amd.engine import Engine, StepEntry
+    cfg, w = P.read_model(model_dirs["B"]["bfloat16"])
+    eng = Engine.from_dir(model_dirs["B"]["bfloat16"], dtype="bfloat16", max_tokens=64 * 8)
+    ids = tiny.prompts("B", [250], seed=12)[0]
+    ref = P.logits(cfg, w, ids)
+    s = eng.open()
+    got = eng.step([StepEntry(s, ids, list(range(250)))]).cpu().double()
+    eng.close(s)
+    top2 = ref.topk(2, dim=-1).values
+    clear = (top2[:, 0] - top2[:, 1]) > 2 * tiny.BFLOAT16_MAX_REL * float(ref.pow(2).mean().sqrt())  # both logits may move
+    assert int(clear.sum()) >= 5
+    assert torch.equal(got.argmax(-1)[clear], ref.argmax(-1)[clear])
+
+
+def test_temperature_sampling_is_reproducible_and_independent_of_companions(model_dirs):
+    from palm_infra_amd.engine import Engine
+    from palm_infra_amd.sampling import SamplingParams
+    eng = Engine.from_dir(model_dirs["B"]["float32"], dtype="float32", max_tokens=64 * 16)
+    prompts = tiny.prompts("B", [1, 31, 12, 64], seed=13)            # the workload of the second tiny configuration
+    sp = SamplingParams(temperature=0.7, top_k=0, top_p=0.0, seed=1)
+    a, _ = eng.generate(prompts, sp, max_new_tokens=16, ignore_eos=True)
+    b, _ = eng.generate(prompts, sp, max_new_tokens=16, ignore_eos=True)
+    assert [r.token_ids for r in a] == [r.token_ids for r in b]      # same seed, same stream
+    c, _ = eng.generate(prompts, SamplingParams(temperature=0.7, top_k=0, top_p=0.0, seed=2), max_new_tokens=16, ignore_eos=True)
+    assert [r.token_ids for r in a] != [r.token_ids for r in c]
+    # request 0 alone draws the same tokens as in the batch: its stream is its own
+    alone, _ = eng.generate(prompts[:1], sp, max_new_tokens=16, ignore_eos=True)
+    assert alone[0].token_ids == a[0].token_ids
+    one_by_one, _ = eng.generate(prompts, sp, max_new_tokens=16, ignore_eos=True, max_batch=1)
+    assert [r.token_ids for r in one_by_one] == [r.token_ids for r in a]
+    # every token drawn has positive probability under the plain distribution of its own context
+    cfg, w = P.read_model(model_dirs["B"]["float32"])
+    r = a[2]
+    ctx = list(prompts[2])
+    for tok in r.token_ids[:6]:
+        probs = P.probabilities(P.logits(cfg, w, ctx)[-1].numpy(), 0.7)
+        assert probs[tok] > 0
+        ctx.append(tok)
+
+
+def test_all_sampling_options_together(model_dirs):
+    from palm_infra_amd.engine import Engine
+    from palm_infra_amd.sampling import SamplingParams
+    eng = Engine.from_dir(model_dirs["A"]["bfloat16"], dtype="bfloat16", max_tokens=64 * 8)
+    sp = SamplingParams(temperature=0.9, top_k=20, top_p=0.8, min_p=0.02, repeat_penalty=1.3, repeat_last_n=8,
+                        presence_penalty=0.5, frequency_penalty=0.2, seed=3)
+    prompts = tiny.prompts("A", [4, 9], seed=14)
+    a, _ = eng.generate(prompts, sp, max_new_tokens=20, ignore_eos=True)
+    b, _ = eng.generate(prompts, sp, max_new_tokens=20, ignore_eos=True)
+    assert [r.token_ids for r in a] == [r.token_ids for r in b] and all(len(r.token_ids) == 20 for r in a)
+    # a strong penalty forbids an immediate repeat under greedy choice
+    greedy_pen = SamplingParams(temperature=0.0, repeat_penalty=1.0, presence_penalty=2.0, frequency_penalty=2.0, repeat_last_n=-1)
+    out, _ = eng.generate(prompts, greedy_pen, max_new_tokens=12, ignore_eos=True)
+    plain, _ = eng.generate(prompts, SamplingParams(temperature=0.0), max_new_tokens=12, ignore_eos=True)
+    assert [r.token_ids for r in out] != [r.token_ids for r in plain]
+
+
+def test_command_line_generates_and_reports(model_dirs):
+    cfg, w = P.read_model(model_dirs["A"]["float32"])
+    prompt = tiny.prompts("A", [6], seed=15)[0]
+    r = subprocess.run([str(ROOT / "bin" / "palm_chat"), "--package", str(model_dirs["A"]["float32"]), "--dtype", "float32",
+                        "--prompt-ids", ",".join(map(str, prompt)), "--max-new-tokens", "6", "--temperature", "0", "--n-ctx", "256"],
+                       capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert [int(t) for t in r.stdout.split()] == P.greedy(cfg, w, prompt, 6, stop=(7,))
+    b = subprocess.run([str(ROOT / "bin" / "palm_bench"), "--package", str(model_dirs["A"]["bfloat16"]), "--prompt-tokens", "20",
+                        "--batch", "3", "--max-new-tokens", "5", "--temperature", "0", "--n-ctx", "512", "--warmup", "1"],
+                       capture_output=True, text=True, timeout=120)
+    assert b.returncode == 0, b.stderr[-2000:]
+    kv = dict(line.split("=", 1) for line in b.stdout.strip().splitlines())
+    assert kv["prompt_tokens"] == "60" and kv["generated_tokens"] == "15" and kv["decode_tokens"] == "12" and kv["hit_eos"] == "0"
+    assert float(kv["decode_tps"]) > 0 and float(kv["prefill_tps"]) > 0
+    bad = subprocess.run([str(ROOT / "bin" / "palm_chat"), "--package", str(model_dirs["A"]["float32"]), "--temperature", "3"],
+                         capture_output=True, text=True, timeout=120)
+    assert bad.returncode == 1 and "temperature must be between 0 and 2" in bad.stderr

@@ -1,0 +1,136 @@
+"""The generation loop's decisions, with stand-ins for the engine and the sampler (no GPU)."""
+import pytest
+import torch
+
+from palm_infra_amd.engine.generate import RequestTooLong, compute_metrics, generate, plan_batches, GenerationResult
+
+
+class ScriptedEngine:
+    """Its "logits" put all weight on the token that a script names for (request, how many tokens it has
+    seen); it keeps the engine's books so the loop's use of slots can be checked."""
+
+    def __init__(self, script, vocab=50, max_tokens=64 * 64, max_seq_tokens=4096, n_slots=8):
+        self.script, self.vocab = script, vocab
+        self.cache = type("C", (), {"max_tokens": max_tokens, "max_seq_tokens": max_seq_tokens})()
+        self.free = list(range(n_slots - 1, -1, -1))
+        self.seen = {}            # slot -> tokens consumed
+        self.steps = []           # [(slot, n tokens), ...] of every step
+        self.closed = []
+
+    def open(self):
+        s = self.free.pop()
+        self.seen[s] = []
+        return s
+
+    def close(self, slot):
+        assert slot in self.seen, "closed twice"
+        del self.seen[slot]
+        self.closed.append(slot)
+        self.free.append(slot)
+        self.free.sort(reverse=True)
+
+    def step(self, entries):
+        self.steps.append([(e.slot, len(e.tokens)) for e in entries])
+        rows = []
+        for e in entries:
+            assert e.slot in self.seen
+            self.seen[e.slot].extend(e.tokens)
+            assert len(e.want) == 1 and e.want[0] == len(e.tokens) - 1
+            row = torch.zeros(self.vocab)
+            row[self.script(tuple(self.seen[e.slot]))] = 1.0
+            rows.append(row)
+        return torch.stack(rows)
+
+
+class ArgmaxSampler:
+    def __init__(self):
+        self.histories = []
+
+    def sample(self, logits, states):
+        self.histories.append([list(s.history) for s in states])
+        return logits.argmax(-1)
+
+
+def test_unequal_prompts_stop_tokens_and_early_endings():
+    # a prompt is [how many tokens to generate before the stop token, filler..., 0]; the stop token is 9
+    prompts = [[3, 1, 1, 0], [1, 0], [5, 7, 7, 7, 7, 7, 0]]
+
+    def script2(seen):
+        n_gen = len(seen) - (seen.index(0) + 1)
+        return 9 if n_gen >= seen[0] else 20 + n_gen
+    eng, smp = ScriptedEngine(script2), ArgmaxSampler()
+    seen_tokens = []
+    results, metrics = generate(eng, smp, prompts, max_new_tokens=5, stop_token_ids=[9],
+                                on_token=lambda i, t: seen_tokens.append((i, t)))
+    assert [r.token_ids for r in results] == [[20, 21, 22, 9], [20, 9], [20, 21, 22, 23, 24]]
+    assert [r.finish_reason for r in results] == ["stop", "stop", "length"]
+    assert results[0].hit_eos and not results[2].hit_eos
+    # one step with all prompts, then one token for each sequence that still runs
+    assert eng.steps[0] == [(0, 4), (1, 2), (2, 7)]
+    assert eng.steps[1:] == [[(0, 1), (1, 1), (2, 1)], [(0, 1), (2, 1)], [(0, 1), (2, 1)], [(2, 1)]]
+    assert sorted(eng.closed) == [0, 1, 2] and eng.closed[0] == 1           # the shortest left first
+    assert not eng.seen
+    # sampling history follows what the model has consumed (engine/engine.cpp:977, 1451)
+    assert smp.histories[0] == prompts and smp.histories[1][0] == prompts[0] + [20]
+    assert seen_tokens[:3] == [(0, 20), (1, 20), (2, 20)]
+    # the reference's metrics (examples/cli_common.cpp:418-436), summed
+    assert metrics.prompt_tokens == 13 and metrics.generated_tokens == 11 and metrics.decode_tokens == 8
+
+
+def test_stop_at_the_first_token_runs_no_decode_step():
+    eng = ScriptedEngine(lambda seen: 9)
+    results, _ = generate(eng, ArgmaxSampler(), [[1, 2], [3]], max_new_tokens=8, stop_token_ids=[9])
+    assert [r.token_ids for r in results] == [[9], [9]] and len(eng.steps) == 1 and not eng.seen
+
+
+def test_batches_follow_one_another_and_slots_are_used_again():
+    eng = ScriptedEngine(lambda seen: 30 + len(seen), n_slots=2)
+    prompts = [[1] * n for n in (3, 5, 2, 4, 6)]
+    results, _ = generate(eng, ArgmaxSampler(), prompts, max_new_tokens=2, max_batch=2)
+    assert [r.token_ids for r in results] == [[33, 34], [35, 36], [32, 33], [34, 35], [36, 37]]
+    firsts = [s for s in eng.steps if any(n > 1 for _, n in s)]
+    assert firsts == [[(0, 3), (1, 5)], [(0, 2), (1, 4)], [(0, 6)]]
+    assert not eng.seen
+
+
+def test_a_sequence_that_fills_its_context_ends():
+    eng = ScriptedEngine(lambda seen: 1, max_seq_tokens=6)
+    results, _ = generate(eng, ArgmaxSampler(), [[2, 2, 2, 2]], max_new_tokens=50)
+    # 4 prompt tokens; tokens 1 and 2 can still be fed (lengths 5, 6); the third cannot
+    assert results[0].finish_reason == "context" and len(results[0].token_ids) == 3
+    assert len(eng.steps) == 3 and not eng.seen
+
+
+def test_slots_come_back_when_a_step_fails():
+    class Failing(ScriptedEngine):
+        def step(self, entries):
+            if len(self.steps) == 2:
+                raise RuntimeError("boom")
+            return super().step(entries)
+    eng = Failing(lambda seen: 1)
+    with pytest.raises(RuntimeError, match="boom"):
+        generate(eng, ArgmaxSampler(), [[1], [2]], max_new_tokens=9)
+    assert not eng.seen and sorted(eng.closed) == [0, 1]
+
+
+def test_plan_batches():
+    # 64-token pages: 60+10 -> 2 pages, 10+10 -> 1 page
+    assert plan_batches([60, 10, 10, 10], 10, max_batch=8, cache_tokens=64 * 3, max_seq_tokens=4096) == [[0, 1], [2, 3]]
+    assert plan_batches([1, 1, 1, 1, 1], 1, max_batch=2, cache_tokens=64 * 100, max_seq_tokens=4096) == [[0, 1], [2, 3], [4]]
+    with pytest.raises(RequestTooLong, match="request 1"):
+        plan_batches([5, 200], 1, 4, 64 * 100, max_seq_tokens=128)
+    with pytest.raises(RequestTooLong, match="do not fit"):
+        plan_batches([5, 200], 100, 4, 64 * 2, max_seq_tokens=4096)
+    with pytest.raises(RequestTooLong, match="empty"):
+        plan_batches([0], 1, 4, 64, 64)
+    with pytest.raises(ValueError):
+        generate(ScriptedEngine(lambda s: 1), ArgmaxSampler(), [[1]], max_new_tokens=0)   # examples/cli_common.cpp:451-454
+
+
+def test_metrics_follow_the_reference_definitions():
+    rs = [GenerationResult(prompt_tokens=10, token_ids=[1, 2, 3]), GenerationResult(prompt_tokens=6, token_ids=[4])]
+    m = compute_metrics(rs, prefill_ms=8.0, decode_ms=4.0)
+    assert (m.prompt_tokens, m.generated_tokens, m.decode_tokens) == (16, 4, 2)
+    assert m.ttft_ms == 8.0 and m.tpot_ms == 2.0 and m.prefill_tps == 2000.0 and m.decode_tps == 500.0 and m.total_ms == 12.0
+    m0 = compute_metrics([GenerationResult(prompt_tokens=3, token_ids=[1])], 1.0, 0.0)
+    assert m0.decode_tokens == 0 and m0.tpot_ms == 0.0 and m0.decode_tps == 0.0

@@ -1,0 +1,392 @@
+"""Each kernel alone against its plain reference, at other sizes than the engine's tiny models use."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import plain_qwen3 as P
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+F32, BF16 = torch.float32, torch.bfloat16
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from palm_infra_amd.kernels import ops
+    return ops
+
+
+def rand(*shape, seed=0, scale=1.0, dtype=F32):
+    return (torch.randn(*shape, generator=torch.Generator().manual_seed(seed)) * scale).to(dtype)
+
+
+def tol(dtype):
+    return 2e-5 if dtype == F32 else 2e-2
+
+
+# ---- embedding, norm, swiglu, cast --------------------------------------------------------------
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_embed(ops, dtype):
+    table = rand(515, 80, seed=1, dtype=dtype)
+    ids = torch.tensor([0, 514, 7, 7, 300], dtype=torch.int32)
+    got = ops.embed(table.to(DEV), ids.to(DEV)).cpu()
+    assert got.dtype == F32 and torch.equal(got, table[ids.long()].float())
+    bad = ops.embed(table.to(DEV), torch.tensor([3, 515, -1], dtype=torch.int32).to(DEV)).cpu()
+    assert torch.equal(bad[0], table[3].float()) and torch.isnan(bad[1:]).all()      # visible, never a wrong row
+
+
+@pytest.mark.parametrize("width", [8, 17, 64, 2048, 5120])
+@pytest.mark.parametrize("eps", [1e-6, 1e-5])
+def test_rmsnorm_widths_of_the_reference_test(ops, width, eps):       # tests/test_norm.cpp:43-256
+    x, w = rand(5, width, seed=width), rand(width, seed=1) + 1.0
+    got = ops.rmsnorm(x.to(DEV), w.to(DEV), eps, F32).cpu()
+    assert torch.allclose(got.double(), P.rms_norm(x, w, eps), atol=1e-5 if width < 2048 else 1e-4)
+
+
+def test_rmsnorm_eps_inside_the_root_and_zero_rows(ops):
+    x = torch.full((2, 32), 1e-4)
+    x[1] = 0.0
+    got = ops.rmsnorm(x.to(DEV), torch.ones(32).to(DEV), 1e-6, F32).cpu()
+    assert torch.allclose(got[0], x[0] / math.sqrt(1e-8 + 1e-6), rtol=1e-5) and float(got[1].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("out_dtype,delta_dtype", [(F32, F32), (BF16, BF16), (BF16, F32)])
+def test_rmsnorm_adds_the_pending_branch_in_32_bit(ops, out_dtype, delta_dtype):
+    x, d, w = rand(7, 96, seed=2), rand(7, 96, seed=3, dtype=delta_dtype), rand(96, seed=4) + 1.0
+    xd = x.to(DEV)
+    got = ops.rmsnorm(xd, w.to(DEV), 1e-5, out_dtype, delta=d.to(DEV), update_x=True).cpu()
+    assert torch.equal(xd.cpu(), x + d.float())                        # the residual stream holds the exact 32-bit sum
+    assert torch.allclose(got.double(), P.rms_norm(x.double() + d.double(), w, 1e-5), atol=tol(out_dtype))
+    # row selection reads x + delta without touching x
+    xd2 = x.to(DEV)
+    rows = torch.tensor([6, 0, 3], dtype=torch.int32).to(DEV)
+    sel = ops.rmsnorm(xd2, w.to(DEV), 1e-5, F32, delta=d.to(DEV), rows=rows).cpu()
+    assert torch.equal(xd2.cpu(), x)
+    assert torch.allclose(sel.double(), P.rms_norm(x.double() + d.double(), w, 1e-5)[[6, 0, 3]], atol=2e-5)
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_swiglu(ops, dtype):
+    gu = rand(9, 2 * 176, seed=5, scale=3.0, dtype=dtype)
+    got = ops.swiglu(gu.to(DEV)).cpu()
+    g, u = gu[:, :176].double(), gu[:, 176:].double()
+    assert torch.allclose(got.double(), g / (1 + torch.exp(-g)) * u, atol=tol(dtype), rtol=tol(dtype))
+    swapped = u / (1 + torch.exp(-u)) * g
+    assert not torch.allclose(got.double(), swapped, atol=0.1)
+
+
+def test_cast_rounds_to_nearest_even(ops):
+    x = torch.tensor([1.0, 1.00390625, 1.01171875, -3.1415927, 1e-40, 65504.0, float("inf")])
+    assert torch.equal(ops.cast(x.to(DEV), BF16).cpu(), x.to(BF16))
+    assert torch.equal(ops.cast(x.to(BF16).to(DEV), F32).cpu(), x.to(BF16).float())
+
+
+# ---- linear -------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("M,N,K", [(1, 7, 5), (3, 130, 67), (65, 64, 16), (70, 515, 80), (129, 96, 224)])
+@pytest.mark.parametrize("ta,tw,tc", [(F32, F32, F32), (BF16, BF16, BF16), (BF16, F32, BF16), (BF16, BF16, F32)])
+def test_linear_exact(ops, M, N, K, ta, tw, tc):
+    a, w = rand(M, K, seed=M, dtype=ta), rand(N, K, seed=N, dtype=tw)
+    got = ops.linear_exact(a.to(DEV), w.to(DEV), tc).cpu()
+    ref = P.linear(a, w)
+    assert got.dtype == tc
+    assert torch.allclose(got.double(), ref, atol=1e-4 if tc == F32 else 0.1, rtol=1e-5 if tc == F32 else 1e-2)
+
+
+def test_linear_exact_result_of_a_row_does_not_depend_on_the_other_rows(ops):
+    a, w = rand(70, 80, seed=1), rand(130, 80, seed=2)
+    whole = ops.linear_exact(a.to(DEV), w.to(DEV)).cpu()
+    for r in (0, 33, 69):
+        alone = ops.linear_exact(a[r:r + 1].contiguous().to(DEV), w.to(DEV)).cpu()
+        assert torch.equal(alone[0], whole[r])
+
+
+def test_linear_refuses_what_does_not_fit(ops):
+    from palm_infra_amd.kernels import KernelError
+    with pytest.raises(KernelError, match="inner size"):
+        ops.linear_exact(rand(2, 5).to(DEV), rand(3, 6).to(DEV))
+    with pytest.raises(KernelError, match="GPU only"):
+        ops.linear_exact(rand(2, 5), rand(3, 5))
+    with pytest.raises(KernelError, match="contiguous"):
+        ops.linear_exact(rand(5, 2).t().to(DEV), rand(3, 5).to(DEV))
+
+
+# ---- rotation, q/k norm and the cache write -----------------------------------------------------
+
+def _paged(n_pages, nkv, hd, dtype):
+    return (torch.zeros(n_pages, nkv, 64, hd, dtype=dtype, device=DEV), torch.zeros(n_pages, nkv, 64, hd, dtype=dtype, device=DEV))
+
+
+@pytest.mark.parametrize("theta,half", [(10000.0, 8), (1000000.0, 24), (500000.0, 64)])
+def test_rope_table(ops, theta, half):
+    pos = [0, 1, 2, 63, 64, 1000, 40000]
+    i = np.arange(half, dtype=np.float32)
+    inv = (np.float32(1.0) / np.power(np.float32(theta), np.float32(2.0) * i / np.float32(2 * half))).astype(np.float32)
+    cos, sin = ops.rope_table(torch.tensor(pos, dtype=torch.int32).to(DEV), torch.from_numpy(inv).to(DEV))
+    rc, rs = P.rope_table(pos, 2 * half, theta)
+    # the angle is a float32 product on both sides; pow may differ in the last bit, which the position multiplies
+    assert torch.allclose(cos.cpu().double(), rc, atol=2e-3) and torch.allclose(sin.cpu().double(), rs, atol=2e-3)
+    assert torch.allclose(cos.cpu().double()[:5], rc[:5], atol=1e-5) and torch.allclose(sin.cpu().double()[:5], rs[:5], atol=1e-5)
+    assert float(cos[0, 0]) == 1.0 and float(sin[0, 0]) == 0.0         # tests/test_engine.cpp:90-91
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("nh,nkv,hd", [(5, 5, 48), (6, 2, 80), (3, 1, 128)])
+def test_qk_norm_rope_store(ops, dtype, nh, nkv, hd):
+    # two sequences in slots 2 and 0, the first continuing at position 60 (so it crosses a page border)
+    starts, counts, slots = [60, 0], [9, 5], [2, 0]
+    n = sum(counts)
+    pos = [s + j for s, c in zip(starts, counts) for j in range(c)]
+    tslot = [sl for sl, c in zip(slots, counts) for _ in range(c)]
+    qkv = rand(n, (nh + 2 * nkv) * hd, seed=hd, dtype=dtype)
+    qw, kw = rand(hd, seed=1) + 1.0, rand(hd, seed=2) + 1.0
+    eps, theta = 1e-5, 10000.0
+    table = torch.full((4, 3), 7, dtype=torch.int32)
+    table[2, :2] = torch.tensor([5, 1])
+    table[0, :1] = torch.tensor([3])
+    kc, vc = _paged(8, nkv, hd, dtype)
+    inv = torch.from_numpy((1.0 / np.power(np.float32(theta), 2.0 * np.arange(hd // 2, dtype=np.float32) / hd)).astype(np.float32))
+    cos, sin = ops.rope_table(torch.tensor(pos, dtype=torch.int32).to(DEV), inv.to(DEV))
+    q = ops.qk_norm_rope_store(qkv.to(DEV), nh, nkv, hd, torch.tensor(pos, dtype=torch.int32).to(DEV), q_norm_w=qw.to(DEV),
+                               k_norm_w=kw.to(DEV), eps=eps, cos=cos, sin=sin, rotary_dim=hd, pairing=0, k_cache=kc, v_cache=vc,
+                               block_table=table.to(DEV), tok_slot=torch.tensor(tslot, dtype=torch.int32).to(DEV)).cpu()
+    x = qkv.double()
+    rq = x[:, :nh * hd].reshape(n, nh, hd)
+    rk = x[:, nh * hd:(nh + nkv) * hd].reshape(n, nkv, hd)
+    rv = x[:, (nh + nkv) * hd:].reshape(n, nkv, hd)
+    c64, s64 = P.rope_table(pos, hd, theta)
+    rq = P.rope_half_split(P.rms_norm(rq, qw, eps), c64, s64)
+    rk = P.rope_half_split(P.rms_norm(rk, kw, eps), c64, s64)
+    t = 5e-5 if dtype == F32 else 4e-2
+    assert torch.allclose(q.double().reshape(n, nh, hd), rq, atol=t)
+    kc, vc = kc.cpu().double(), vc.cpu().double()
+    for i in range(n):
+        page = int(table[tslot[i], pos[i] // 64])
+        assert torch.allclose(kc[page, :, pos[i] % 64], rk[i], atol=t), i
+        assert torch.allclose(vc[page, :, pos[i] % 64], rv[i], atol=1e-12 if dtype == F32 else 0), i   # v is stored as it is
+    written = {(int(table[tslot[i], pos[i] // 64]), pos[i] % 64) for i in range(n)}
+    for page in range(8):
+        for r in range(64):
+            if (page, r) not in written:
+                assert float(kc[page, :, r].abs().max()) == 0.0 and float(vc[page, :, r].abs().max()) == 0.0
+
+
+def test_rotation_variants_interleaved_partial_and_none(ops):
+    n, nh, nkv, hd, rot = 4, 2, 1, 32, 16
+    pos = [3, 4, 5, 6]
+    qkv = rand(n, (nh + 2 * nkv) * hd, seed=9)
+    inv = torch.from_numpy((1.0 / np.power(np.float32(1e4), 2.0 * np.arange(rot // 2, dtype=np.float32) / rot)).astype(np.float32))
+    posd = torch.tensor(pos, dtype=torch.int32).to(DEV)
+    cos, sin = ops.rope_table(posd, inv.to(DEV))
+    x = qkv.double()[:, :nh * hd].reshape(n, nh, hd)
+    c, s = P.rope_table(pos, rot, 1e4)
+    # partial rotation, half-split: the tail passes (kernels/rope.cpp:26-29)
+    q = ops.qk_norm_rope_store(qkv.to(DEV), nh, nkv, hd, posd, cos=cos, sin=sin, rotary_dim=rot, pairing=0, write_cache=False).cpu()
+    assert torch.allclose(q.double().reshape(n, nh, hd), P.rope_half_split(x, c, s), atol=1e-5)
+    # interleaved pairs (2i, 2i+1) (kernels/rope.cpp:31-40)
+    q = ops.qk_norm_rope_store(qkv.to(DEV), nh, nkv, hd, posd, cos=cos, sin=sin, rotary_dim=rot, pairing=1, write_cache=False).cpu()
+    ref = x.clone()
+    ev, od = x[..., 0:rot:2], x[..., 1:rot:2]
+    ref[..., 0:rot:2] = ev * c[:, None] - od * s[:, None]
+    ref[..., 1:rot:2] = ev * s[:, None] + od * c[:, None]
+    assert torch.allclose(q.double().reshape(n, nh, hd), ref, atol=1e-5)
+    # no norm, no rotation: q comes through unchanged
+    q = ops.qk_norm_rope_store(qkv.to(DEV), nh, nkv, hd, posd, write_cache=False).cpu()
+    assert torch.equal(q.reshape(n, nh, hd), qkv[:, :nh * hd].reshape(n, nh, hd))
+
+
+# ---- attention ----------------------------------------------------------------------------------
+
+def _fill_cache(kc, vc, table, slot, k, v):
+    """k, v [len, nkv, hd] into the pages of `slot`."""
+    for p in range(k.shape[0]):
+        page = int(table[slot, p // 64])
+        kc[page, :, p % 64] = k[p].to(kc.dtype)
+        vc[page, :, p % 64] = v[p].to(vc.dtype)
+
+
+def _attention_case(ops, fn, dtype, nh, nkv, hd, lens_new, window, seed=0, scale=None):
+    """Sequences (total length, new tokens): queries are the last `new` positions."""
+    scale = scale if scale is not None else hd ** -0.5
+    B = len(lens_new)
+    n_pages = sum((L + 63) // 64 for L, _ in lens_new) + 2
+    perm = torch.randperm(n_pages - 1, generator=torch.Generator().manual_seed(seed)).tolist()
+    max_pages = max((L + 63) // 64 for L, _ in lens_new) + 1
+    slots = torch.randperm(B + 4, generator=torch.Generator().manual_seed(seed + 7)).tolist()[:B]      # distinct, not in order
+    table = torch.full((B + 4, max_pages), n_pages - 1, dtype=torch.int32)
+    kc = rand(n_pages, nkv, 64, hd, seed=seed + 50, dtype=dtype).to(DEV)      # stale values everywhere
+    vc = rand(n_pages, nkv, 64, hd, seed=seed + 51, dtype=dtype).to(DEV)
+    qs, refs, o = [], [], 0
+    for b, (L, new) in enumerate(lens_new):
+        npg = (L + 63) // 64
+        table[slots[b], :npg] = torch.tensor(perm[o:o + npg], dtype=torch.int32)
+        o += npg
+        k, v = rand(L, nkv, hd, seed=seed + 10 * b + 1, dtype=dtype), rand(L, nkv, hd, seed=seed + 10 * b + 2, dtype=dtype)
+        q = rand(L, nh, hd, seed=seed + 10 * b + 3, scale=2.0, dtype=dtype)
+        _fill_cache(kc, vc, table, slots[b], k.to(DEV), v.to(DEV))
+        refs.append(P.causal_attention(q, k, v, scale, window)[L - new:])
+        qs.append(q[L - new:])
+    qcat = torch.cat(qs).reshape(-1, nh * hd).contiguous()
+    i32 = lambda xs: torch.tensor(xs, dtype=torch.int32).to(DEV)
+    cu = [0]
+    for _, new in lens_new:
+        cu.append(cu[-1] + new)
+    got = fn(qcat.to(DEV), kc, vc, table.to(DEV), i32(slots), i32([L - new for L, new in lens_new]),
+             i32([new for _, new in lens_new]), i32(cu), max(new for _, new in lens_new), nh, nkv, hd, scale, window)
+    return got.cpu().double().reshape(-1, nh, hd), torch.cat(refs)
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("nh,nkv,hd", [(8, 4, 16), (5, 5, 48), (6, 1, 80), (4, 2, 128)])
+def test_attention_exact_prompts_decode_and_mixed_lengths(ops, dtype, nh, nkv, hd):
+    # tests/test_attention.cpp:186-217: GQA, past > 0, tails that do not fill a tile, 256 keys
+    cases = [[(20, 20)], [(256, 256)], [(300, 1)], [(1, 1)], [(64, 64), (65, 1), (130, 70), (7, 7)]]
+    for lens in cases:
+        got, ref = _attention_case(ops, ops.attention_exact, dtype, nh, nkv, hd, lens, None, seed=len(lens))
+        assert torch.allclose(got, ref, atol=1e-5 if dtype == F32 else 2e-2), lens
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_attention_exact_window(ops, dtype):
+    for window in (1, 5, 64, 100):
+        got, ref = _attention_case(ops, ops.attention_exact, dtype, 4, 2, 32, [(200, 200), (150, 1), (70, 3)], window, seed=window)
+        assert torch.allclose(got, ref, atol=1e-5 if dtype == F32 else 2e-2), window
+
+
+def _spike_case(ops, fn, dtype, L, spike_at, window=None):
+    """One key among L is made to dominate the last query; the output must be that key's value."""
+    nh, nkv, hd = 2, 1, 32
+    k = rand(L, nkv, hd, seed=1, scale=0.1, dtype=dtype)
+    v = rand(L, nkv, hd, seed=2, dtype=dtype)
+    q = rand(1, nh, hd, seed=3, scale=0.1, dtype=dtype)
+    k[spike_at, 0, :] = 0
+    k[spike_at, 0, 5] = 8.0
+    q[0, :, 5] = 8.0                         # score 64 * scale at the spike, ~0 elsewhere
+    table = torch.arange((L + 63) // 64 + 1, dtype=torch.int32).flip(0)[None, :].contiguous()
+    n_pages = table.shape[1]
+    kc, vc = _paged(n_pages, nkv, hd, dtype)
+    _fill_cache(kc, vc, table, 0, k.to(DEV), v.to(DEV))
+    i32 = lambda xs: torch.tensor(xs, dtype=torch.int32).to(DEV)
+    got = fn(q.reshape(1, nh * hd).to(DEV), kc, vc, table.to(DEV), i32([0]), i32([L - 1]), i32([1]), i32([0, 1]), 1, nh, nkv, hd,
+             1.0, window)
+    return got.cpu().float().reshape(nh, hd), v
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_a_far_key_among_hundreds_is_found(ops, dtype):
+    for L, at in ((700, 13), (700, 0), (700, 699), (513, 448), (64, 63), (65, 64)):
+        got, v = _spike_case(ops, ops.attention_exact, dtype, L, at)
+        assert torch.allclose(got, v[at, 0].float().expand(2, -1), atol=1e-2), (L, at)
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_the_edge_of_a_window(ops, dtype):
+    L, w = 300, 70
+    inside, outside = L - w, L - w - 1       # the last query sits at L-1 and reads keys L-w .. L-1
+    got, v = _spike_case(ops, ops.attention_exact, dtype, L, inside, window=w)
+    assert torch.allclose(got, v[inside, 0].float().expand(2, -1), atol=1e-2)
+    got, v = _spike_case(ops, ops.attention_exact, dtype, L, outside, window=w)
+    assert not torch.allclose(got, v[outside, 0].float().expand(2, -1), atol=0.2)   # the spike is out of reach
+
+
+# ---- sampling -----------------------------------------------------------------------------------
+
+def test_argmax_takes_the_first_maximum(ops):
+    lg = rand(6, 1000, seed=3)
+    lg[1, 17] = lg[1, 900] = 50.0
+    lg[2, :] = 0.0
+    lg[3, 999] = 60.0
+    lg[4, 0] = 60.0
+    got = ops.argmax(lg.to(DEV)).cpu().tolist()
+    assert got == [int(lg[0].argmax()), 17, 0, 999, 0, int(lg[5].argmax())]
+    assert ops.argmax(torch.tensor([[0.5, 3.0, 2.0]]).to(DEV)).item() == 1       # tests/test_sampler.cpp:26-27
+
+
+def _sample(ops, lg, u, **kw):
+    lg = torch.as_tensor(lg, dtype=F32).reshape(1, -1)
+    return ops.sample(lg.to(DEV), torch.tensor([u], dtype=F32).to(DEV), **kw).item()
+
+
+def test_sampling_vectors_of_the_reference(ops):
+    # tests/test_sampler.cpp:19-60
+    assert _sample(ops, [0.5, 3.0, 2.0], 0.7, temperature=0.0) == 1
+    assert _sample(ops, [0.5, 3.0, 2.0], 0.99, temperature=1.0, top_k=1) == 1
+    for u in (0.0, 0.5, 0.999):
+        assert _sample(ops, [4.0, 0.0, -1.0], u, temperature=1.0, min_p=0.5) == 0
+        assert _sample(ops, [4.0, 0.0, -1.0], u, temperature=1.0, top_p=0.5) == 0
+        assert _sample(ops, [4.0, 0.0, -1.0], u, temperature=1.0, top_k=2, top_p=0.5) == 0
+    # tests/test_sampler.cpp:170-181
+    lg = torch.tensor([[0.0, math.log(2.0), math.log(3.0)]])
+    _, probs = ops.sample(lg.to(DEV), torch.zeros(1).to(DEV), 1.0, 0, 1.0, 0.0, want_probs=True)
+    assert torch.allclose(probs.cpu(), torch.tensor([[1 / 6, 2 / 6, 3 / 6]]), atol=1e-5)
+
+
+@pytest.mark.parametrize("kw", [
+    dict(temperature=0.7), dict(temperature=1.3, min_p=0.05), dict(temperature=1.0, top_p=0.8), dict(temperature=0.9, top_p=0.3, min_p=0.01),
+    dict(temperature=0.8, top_k=50), dict(temperature=1.0, top_k=5, top_p=0.7), dict(temperature=1.5, top_k=1024, top_p=0.9, min_p=0.02),
+    dict(temperature=0.6, top_k=50, top_p=0.9),          # the reference's defaults
+])
+def test_the_distribution_drawn_from_is_the_plain_one(ops, kw):
+    V = 5003
+    lg = rand(3, V, seed=11, scale=2.0)
+    lg[1, 100] = lg[1, 4000] = lg[1, 7] = float(lg[1].max()) + 0.5       # ties at the top, to be taken by lower id first
+    lg[2, :] = torch.round(lg[2, :] * 2) / 2                              # many ties everywhere
+    full = dict(temperature=1.0, top_k=0, top_p=0.0, min_p=0.0)
+    full.update(kw)
+    _, probs = ops.sample(lg.to(DEV), torch.zeros(3).to(DEV), full["temperature"], full["top_k"], full["top_p"], full["min_p"], want_probs=True)
+    probs = probs.cpu().double().numpy()
+    for r in range(3):
+        ref = P.probabilities(lg[r].double().numpy(), **full)
+        kept, kept_ref = set(np.nonzero(probs[r])[0]), set(np.nonzero(ref)[0])
+        # a candidate exactly at a filter's threshold may fall on either side of a 32-bit sum; nothing else may differ
+        assert len(kept ^ kept_ref) <= 1, (r, sorted(kept ^ kept_ref))
+        if kept == kept_ref:
+            assert np.allclose(probs[r], ref, atol=1e-5), r
+
+
+def test_draws_walk_the_kept_set_and_follow_u(ops):
+    V = 3001
+    lg = rand(1, V, seed=5, scale=1.5)
+    # without top-k the walk is in index order
+    ref = P.probabilities(lg[0].double().numpy(), temperature=0.9, top_p=0.6)
+    cdf = np.cumsum(ref)
+    for u in (0.0, 0.1, 0.37, 0.5, 0.81, 0.999):
+        tok = ops.sample(lg.to(DEV), torch.tensor([u], dtype=F32).to(DEV), 0.9, 0, 0.6, 0.0).item()
+        assert ref[tok] > 0
+        lo = cdf[tok] - ref[tok]
+        assert lo - 1e-4 <= u <= cdf[tok] + 1e-4, (u, tok)
+    # with top-k the walk is over the sorted candidates, as the reference's (engine/sampler.cpp:180-187)
+    for u in (0.0, 0.2, 0.55, 0.93, 0.9999):
+        tok = ops.sample(lg.to(DEV), torch.tensor([u], dtype=F32).to(DEV), 0.9, 40, 0.95, 0.0).item()
+        assert tok == P.draw(lg[0].double().numpy(), u, temperature=0.9, top_k=40, top_p=0.95), u
+
+
+def test_rows_are_sampled_independently(ops):
+    lg = rand(4, 2000, seed=8)
+    u = torch.tensor([0.1, 0.5, 0.9, 0.3])
+    together = ops.sample(lg.to(DEV), u.to(DEV), 1.0, 20, 0.9, 0.0).cpu().tolist()
+    alone = [ops.sample(lg[r:r + 1].to(DEV), u[r:r + 1].to(DEV), 1.0, 20, 0.9, 0.0).item() for r in range(4)]
+    assert together == alone
+
+
+def test_penalties(ops):
+    lg = torch.tensor([[2.0, -2.0, 1.0, 0.5], [1.0, 1.0, 1.0, 1.0]])
+    d = lg.to(DEV)
+    i32 = lambda xs: torch.tensor(xs, dtype=torch.int32).to(DEV)
+    ops.apply_penalties(d, i32([0, 0, 1]), i32([0, 1, 3]), i32([1, 2, 4]), 2.0, 0.5, 0.25)
+    ref0 = P.apply_penalties(lg[0].numpy(), [0, 1, 1], repeat_penalty=2.0, repeat_last_n=-1, presence_penalty=0.5, frequency_penalty=0.25)
+    assert np.allclose(d.cpu().numpy()[0], ref0) and np.allclose(d.cpu().numpy()[1], [1, 1, 1, 1 / 2 - 0.5 - 1.0])
+
+
+def test_sampling_refuses_bad_options(ops):
+    from palm_infra_amd.kernels import KernelError
+    lg, u = rand(1, 5000).to(DEV), torch.zeros(1).to(DEV)
+    with pytest.raises(KernelError, match="temperature"):
+        ops.sample(lg, u, 3.0)
+    with pytest.raises(KernelError, match="at most 1024"):
+        ops.sample(lg, u, 1.0, top_k=2000)
+    with pytest.raises(KernelError, match="uniform"):
+        ops.sample(lg, None, 1.0)

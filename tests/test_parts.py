@@ -1,0 +1,218 @@
+"""Each part alone: built from its description and a few tensors, stepped with a hand-made context,
+compared with the plain function of the same part."""
+import pytest
+import torch
+
+import plain_qwen3 as P
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+F32, BF16 = torch.float32, torch.bfloat16
+
+
+class Tensors:
+    """Stands in for loaded weights: TensorRef -> tensor."""
+
+    def __init__(self):
+        self.by_names = {}
+
+    def add(self, ref, t):
+        self.by_names[ref.names] = t.to(DEV)
+        return ref
+
+    def get(self, ref):
+        return self.by_names[ref.names]
+
+
+def rand(*shape, seed=0, scale=1.0):
+    return torch.randn(*shape, generator=torch.Generator().manual_seed(seed)) * scale
+
+
+def build(spec, tensors, dtype):
+    from palm_infra_amd.parts import Builder
+    return Builder(tensors, dtype, DEV).build(spec)
+
+
+def tol(dtype):
+    return 3e-5 if dtype == F32 else 5e-2
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_norm_part(dtype):
+    from palm_infra_amd.config import PartSpec, tensor
+    T = Tensors()
+    w = rand(80, seed=1) + 1
+    spec = PartSpec("norm", "rms", {"width": 80, "eps": 3e-6}, {"weight": T.add(tensor("n.weight", (80,), "vector"), w)})
+    norm = build(spec, T, dtype)
+    x, d = rand(6, 80, seed=2), rand(6, 80, seed=3).to(dtype)
+    xd = x.to(DEV)
+    y = norm(xd, delta=d.to(DEV), update=True)
+    assert y.dtype == dtype and torch.equal(xd.cpu(), x + d.float())
+    assert torch.allclose(y.cpu().double(), P.rms_norm(x.double() + d.double(), w, 3e-6), atol=tol(dtype))
+    assert torch.allclose(norm(x.to(DEV), out_dtype=F32).cpu().double(), P.rms_norm(x, w, 3e-6), atol=3e-5)
+
+
+def test_position_part_makes_its_tables_once_per_step():
+    from palm_infra_amd.config import PartSpec
+    from palm_infra_amd.parts import make_context
+    rot = build(PartSpec("position", "rotary", {"rotary_dim": 48, "theta": 500000.0, "pairing": "half_split"}), Tensors(), F32)
+    ctx = make_context([0, 1], [10, 0], [[1, 2, 3], [4]], F32, DEV)
+    cos, sin = rot.tables(ctx)
+    rc, rs = P.rope_table([10, 11, 12, 0], 48, 500000.0)
+    assert torch.allclose(cos.cpu().double(), rc, atol=1e-6) and torch.allclose(sin.cpu().double(), rs, atol=1e-6)
+    assert rot.tables(ctx)[0] is cos
+    same = build(PartSpec("position", "rotary", {"rotary_dim": 48, "theta": 500000.0}), Tensors(), F32)
+    other = build(PartSpec("position", "rotary", {"rotary_dim": 48, "theta": 10000.0}), Tensors(), F32)
+    assert same.tables(ctx)[0] is cos and other.tables(ctx)[0] is not cos
+    assert build(PartSpec("position", "none"), Tensors(), F32).tables(ctx) is None
+    with pytest.raises(ValueError, match="pairing"):
+        build(PartSpec("position", "rotary", {"rotary_dim": 8, "theta": 1.0, "pairing": "spiral"}), Tensors(), F32)
+
+
+def attention_spec(T, H, nh, nkv, hd, eps, theta, window=None, qk_norm=True, position=True, seed=0):
+    from palm_infra_amd.config import PartSpec, joined, tensor
+    # without a q/k norm the scores' spread is set by these scales: kept near one so that bfloat16 rounding
+    # cannot flip which key leads
+    w = {"q": rand(nh * hd, H, seed=seed + 1, scale=0.1), "k": rand(nkv * hd, H, seed=seed + 2, scale=0.1),
+         "v": rand(nkv * hd, H, seed=seed + 3, scale=0.3), "o": rand(H, nh * hd, seed=seed + 4, scale=0.3),
+         "qn": rand(hd, seed=seed + 5) * 0.2 + 2.0, "kn": rand(hd, seed=seed + 6) * 0.2 + 1.0}
+    parts = {}
+    if qk_norm:
+        parts["q_norm"] = PartSpec("norm", "rms", {"width": hd, "eps": eps}, {"weight": T.add(tensor("qn", (hd,), "vector"), w["qn"])})
+        parts["k_norm"] = PartSpec("norm", "rms", {"width": hd, "eps": eps}, {"weight": T.add(tensor("kn", (hd,), "vector"), w["kn"])})
+    if position:
+        parts["position"] = PartSpec("position", "rotary", {"rotary_dim": hd, "theta": theta, "pairing": "half_split"})
+    spec = PartSpec("mixer", "attention", {"hidden_size": H, "num_heads": nh, "num_kv_heads": nkv, "head_dim": hd,
+                                           "scale": hd ** -0.5, "window": window},
+                    {"qkv": T.add(joined(("q", "k", "v"), ((nh * hd, H), (nkv * hd, H), (nkv * hd, H))), torch.cat([w["q"], w["k"], w["v"]])),
+                     "out": T.add(tensor("o", (H, nh * hd)), w["o"])}, parts)
+    return spec, w
+
+
+def plain_attention(h, w, nh, nkv, hd, eps, theta, window, qk_norm, position):
+    n = h.shape[0]
+    q = P.linear(h, w["q"]).reshape(n, nh, hd)
+    k = P.linear(h, w["k"]).reshape(n, nkv, hd)
+    v = P.linear(h, w["v"]).reshape(n, nkv, hd)
+    if qk_norm:
+        q, k = P.rms_norm(q, w["qn"], eps), P.rms_norm(k, w["kn"], eps)
+    if position:
+        cos, sin = P.rope_table(list(range(n)), hd, theta)
+        q, k = P.rope_half_split(q, cos, sin), P.rope_half_split(k, cos, sin)
+    return P.linear(P.causal_attention(q, k, v, hd ** -0.5, window).reshape(n, nh * hd), w["o"])
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("kw", [dict(), dict(window=40), dict(qk_norm=False), dict(position=False), dict(qk_norm=False, position=False)])
+def test_attention_part_in_pieces_against_whole_sequences(dtype, kw):
+    """Plain attention without rotation or norm is one of the cases; each switch is a parameter of the part."""
+    from palm_infra_amd.cache import ModelCache
+    from palm_infra_amd.parts import cache_needs, make_context
+    H, nh, nkv, hd, eps, theta = 72, 6, 3, 48, 1e-5, 10000.0
+    window, qk_norm, position = kw.get("window"), kw.get("qk_norm", True), kw.get("position", True)
+    T = Tensors()
+    spec, w = attention_spec(T, H, nh, nkv, hd, eps, theta, window, qk_norm, position)
+    att = build(spec, T, dtype)
+    needs = cache_needs(spec)
+    assert needs[0].num_kv_heads == nkv and needs[0].head_dim == hd and needs[0].window == window
+    cache = ModelCache([needs], [None], 64 * 8, None, 4096, dtype, DEV)
+    seqs = [rand(150, H, seed=11), rand(70, H, seed=12)]
+    slots = [cache.open(), cache.open()]
+    outs = [[], []]
+    done = [0, 0]
+    for pieces in ([100, 64], [1, 0], [49, 6]):            # a prompt each, one token for the first only, the rest
+        live = [b for b in range(2) if pieces[b] > 0]
+        growth = [(slots[b], pieces[b]) for b in live]
+        cache.reserve(growth)
+        ctx = make_context([slots[b] for b in live], [done[b] for b in live], [[0] * pieces[b] for b in live], dtype, DEV)
+        ctx.layer_cache = cache.layer_caches[0]
+        h = torch.cat([seqs[b][done[b]:done[b] + pieces[b]] for b in live]).to(dtype).to(DEV)
+        out = att.forward(h, ctx).cpu()
+        cache.commit(growth)
+        o = 0
+        for b in live:
+            outs[b].append(out[o:o + pieces[b]])
+            o += pieces[b]
+            done[b] += pieces[b]
+    for b in range(2):
+        ref = plain_attention(seqs[b].to(dtype), w_as(w, dtype), nh, nkv, hd, eps, theta, window, qk_norm, position)
+        got = torch.cat(outs[b]).double()
+        scale = float(ref.abs().max())
+        assert torch.allclose(got, ref, atol=tol(dtype) * max(scale, 1.0)), (b, float((got - ref).abs().max()), scale)
+
+
+def w_as(w, dtype):
+    """The weights as the part holds them: matrices in the run's precision, norm vectors in float32."""
+    return {k: (v if k in ("qn", "kn") else v.to(dtype)) for k, v in w.items()}
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_feed_forward_part(dtype):
+    from palm_infra_amd.config import PartSpec, joined, tensor
+    H, I = 80, 176
+    T = Tensors()
+    wg, wu, wd = rand(I, H, seed=1, scale=0.2), rand(I, H, seed=2, scale=0.2), rand(H, I, seed=3, scale=0.2)
+    spec = PartSpec("feed_forward", "gated_silu", {"hidden_size": H, "intermediate_size": I},
+                    {"gate_up": T.add(joined(("g", "u"), ((I, H), (I, H))), torch.cat([wg, wu]).to(dtype)),
+                     "down": T.add(tensor("d", (H, I)), wd.to(dtype))})
+    ff = build(spec, T, dtype)
+    h = rand(9, H, seed=4).to(dtype)
+    got = ff.forward(h.to(DEV), None).cpu().double()
+    ref = P.swiglu_mlp(h, wg.to(dtype), wu.to(dtype), wd.to(dtype))
+    assert torch.allclose(got, ref, atol=tol(dtype) * float(ref.abs().max()))
+    # one expert of a routed feed-forward is this feed-forward: nothing else to reduce to here
+    with pytest.raises(ValueError, match="do not fit"):
+        build(PartSpec("feed_forward", "gated_silu", {"hidden_size": H, "intermediate_size": I + 1}, spec.tensors), T, dtype)
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_embedding_and_head_parts(dtype):
+    from palm_infra_amd.config import PartSpec, tensor
+    V, H = 515, 80
+    T = Tensors()
+    table = rand(V, H, seed=1).to(dtype)
+    ref_t = T.add(tensor("emb", (V, H), "table"), table)
+    emb = build(PartSpec("embedding", "token_table", {"vocab_size": V, "hidden_size": H}, {"table": ref_t}), T, dtype)
+    ids = torch.tensor([0, 514, 3], dtype=torch.int32)
+    assert torch.equal(emb.forward(ids.to(DEV)).cpu(), table[ids.long()].float())
+    head = build(PartSpec("head", "linear", {"vocab_size": V, "hidden_size": H}, {"weight": ref_t}), T, dtype)   # tied
+    h = rand(4, H, seed=2).to(dtype)
+    lg = head.forward(h.to(DEV)).cpu()
+    assert lg.dtype == F32 and torch.allclose(lg.double(), P.linear(h, table), atol=1e-4 if dtype == F32 else 2e-2)
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_block_part_is_a_plain_decoder_layer(dtype, model_dirs):
+    """One layer of tiny model C, built as a block from the model's description and run alone."""
+    import tiny
+    from palm_infra_amd.cache import ModelCache
+    from palm_infra_amd.config import config_from_dir
+    from palm_infra_amd.parts import Builder, cache_needs, make_context
+    from palm_infra_amd.weights import ModelFiles, load_weights
+    name = "float32" if dtype == F32 else "bfloat16"
+    d = model_dirs["C"][name]
+    files = ModelFiles(d)
+    spec = config_from_dir(d).spec(files.names())
+    weights = load_weights(spec, files, dtype, DEV)
+    block = Builder(weights, dtype, DEV).build(spec.layers[1])
+    cache = ModelCache([cache_needs(spec.layers[1])], [None], 64 * 4, None, 2048, dtype, DEV)
+    slot = cache.open()
+    cfg, w = P.read_model(d)
+    S = P.sizes(cfg)
+    x0 = rand(70, S["H"], seed=5)
+    pend = rand(70, S["H"], seed=6).to(dtype)
+    cache.reserve([(slot, 70)])
+    ctx = make_context([slot], [0], [[0] * 70], dtype, DEV)
+    ctx.layer_cache = cache.layer_caches[0]
+    xd = x0.to(DEV)
+    x_out, pending = block.forward(xd, pend.to(DEV), ctx)
+    assert x_out is xd and x_out.dtype == F32                    # the residual stream stays 32-bit and in place
+    got = x_out.cpu().double() + pending.cpu().double()
+    ref = P.decoder_layer(x0.double() + pend.double(), w, 1, S, list(range(70)))
+    assert torch.allclose(got, ref, atol=tol(dtype) * float(ref.abs().max()))
+
+
+def test_unknown_kind_names_the_registered_ones():
+    from palm_infra_amd.config import PartSpec
+    with pytest.raises(KeyError, match="attention"):
+        build(PartSpec("mixer", "convolution"), Tensors(), F32)

@@ -1,0 +1,229 @@
+"""New kinds of parts, defined here and registered from outside the framework, are built and stepped
+without a change to its files: a mixer with state of its own, layers of two kinds in one model, a run
+order that names a layer twice and lets an entry read another entry's cache."""
+import dataclasses
+
+import pytest
+import torch
+
+import plain_qwen3 as P
+import tiny
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def register_toy_mixer():
+    from palm_infra_amd.cache import StateNeed
+    from palm_infra_amd.parts import register_part
+
+    @register_part("mixer", "toy_decay")
+    class DecayMixer:
+        """s_t = decay * s_{t-1} + h_t W_in^T; out_t = s_t W_out^T.  The state s (one vector for each sequence)
+        lives in the cache's per-sequence state; a prompt is a scan, a single token one update."""
+
+        def __init__(self, spec, builder):
+            self.w_in, self.w_out = builder.tensor(spec, "w_in"), builder.tensor(spec, "w_out")
+            self.decay, self.width = float(spec.params["decay"]), int(spec.params["state_size"])
+            self.dtype = builder.dtype
+
+        @staticmethod
+        def cache_needs(spec):
+            return [StateNeed("decay_state", (int(spec.params["state_size"]),))]
+
+        def forward(self, h, ctx):
+            state = ctx.layer_cache.states["decay_state"]          # [slots + 1, state_size], float32
+            u = h.float() @ self.w_in.float().T
+            out = torch.empty_like(u)
+            for b, (slot, n) in enumerate(zip(ctx.host["slots"], ctx.host["counts"])):
+                s = state[slot].clone()
+                for j in range(n):
+                    r = ctx.host["cu"][b] + j
+                    s = self.decay * s + u[r]
+                    out[r] = s
+                state[slot] = s
+            return (out @ self.w_out.float().T).to(self.dtype)
+    return DecayMixer
+
+
+def toy_spec(base_spec, decay=0.8, state_size=24):
+    """Tiny model A with its second layer's attention replaced by the toy mixer."""
+    from palm_infra_amd.config import PartSpec, tensor
+    H = base_spec.hidden_size
+    layer = base_spec.layers[1]
+    toy = PartSpec("mixer", "toy_decay", {"decay": decay, "state_size": state_size},
+                   {"w_in": tensor("toy.w_in", (state_size, H)), "w_out": tensor("toy.w_out", (H, state_size))})
+    parts = dict(layer.parts)
+    parts["mixer"] = toy
+    return dataclasses.replace(base_spec, layers=(base_spec.layers[0], dataclasses.replace(layer, parts=parts)))
+
+
+class ExtraWeights:
+    def __init__(self, weights, extra):
+        self.weights, self.extra = weights, extra
+
+    def get(self, ref):
+        return self.extra[ref.names] if ref.names in self.extra else self.weights.get(ref)
+
+    def nbytes(self):
+        return self.weights.nbytes()
+
+
+def plain_toy_logits(cfg, w, ids, w_in, w_out, decay):
+    S = P.sizes(cfg)
+    pos = list(range(len(ids)))
+    x = P.embedding(w["model.embed_tokens.weight"], ids)
+    x = P.decoder_layer(x, w, 0, S, pos)
+    p = "model.layers.1."
+    h = P.rms_norm(x, w[p + "input_layernorm.weight"], S["eps"])
+    u = h @ w_in.double().T
+    s = torch.zeros(w_in.shape[0], dtype=torch.float64)
+    mixed = []
+    for t in range(len(ids)):
+        s = decay * s + u[t]
+        mixed.append(s)
+    x = x + torch.stack(mixed) @ w_out.double().T
+    h = P.rms_norm(x, w[p + "post_attention_layernorm.weight"], S["eps"])
+    x = x + P.swiglu_mlp(h, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+    return P.linear(P.rms_norm(x, w["model.norm.weight"], S["eps"]), P.head_weight(w))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_mixer_with_state_of_its_own(model_dirs, dtype):
+    from palm_infra_amd.config import config_from_dir
+    from palm_infra_amd.engine import Engine, StepEntry
+    from palm_infra_amd.weights import ModelFiles, load_weights
+    register_toy_mixer()
+    d = model_dirs["A"][dtype]
+    tdt = torch.float32 if dtype == "float32" else torch.bfloat16
+    config = config_from_dir(d)
+    files = ModelFiles(d)
+    base = config.spec(files.names())
+    spec = toy_spec(base)
+    g = torch.Generator().manual_seed(3)
+    w_in = (torch.randn(24, 64, generator=g) * 0.2).to(tdt)
+    w_out = (torch.randn(64, 24, generator=g) * 0.2).to(tdt)
+    weights = ExtraWeights(load_weights(base, files, tdt, DEV), {("toy.w_in",): w_in.to(DEV), ("toy.w_out",): w_out.to(DEV)})
+    eng = Engine(config, spec, weights, tdt, max_tokens=64 * 8)
+    # the cache has one key/value group (layer 0) and one state group (layer 1)
+    assert [g_.n_entries for g_ in eng.cache.kv_groups] == [1] and len(eng.cache.state_groups) == 1
+    assert eng.cache.layer_caches[1].kv is None and "decay_state" in eng.cache.layer_caches[1].states
+
+    cfg, w = P.read_model(d)
+    reqs = tiny.prompts("A", [30, 9, 50], seed=20)
+    refs = [plain_toy_logits(cfg, w, r, w_in, w_out, 0.8) for r in reqs]
+    for round_no in range(2):                 # twice through the same slots: the state must start from zero again
+        slots = [eng.open() for _ in reqs]
+        cuts = [20, 9, 1]
+        out = eng.step([StepEntry(s, r[:c], list(range(c))) for s, r, c in zip(slots, reqs, cuts)])
+        got = {i: [] for i in range(3)}
+        o = 0
+        for i, c in enumerate(cuts):
+            got[i].append(out[o:o + c]); o += c
+        fed = list(cuts)
+        while any(fed[i] < len(reqs[i]) for i in range(3)):
+            live = [i for i in range(3) if fed[i] < len(reqs[i])]
+            out = eng.step([StepEntry(slots[i], [reqs[i][fed[i]]], [0]) for i in live])
+            for r_, i in enumerate(live):
+                got[i].append(out[r_:r_ + 1]); fed[i] += 1
+        for i in range(3):
+            tiny.assert_logits_close(torch.cat(got[i]), refs[i], dtype, f"toy mixer round {round_no} request {i}")
+            eng.close(slots[i])
+    eng.cache.check()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_run_order_names_a_layer_twice_and_shares_a_cache(model_dirs, dtype):
+    """Order: layer 0, layer 1, layer 0 again (weights shared, cache of its own), layer 1 again reading
+    the keys and values its first run wrote."""
+    from palm_infra_amd.config import LayerCall, config_from_dir
+    from palm_infra_amd.engine import Engine, StepEntry
+    from palm_infra_amd.weights import ModelFiles, load_weights
+    d = model_dirs["A"][dtype]
+    tdt = torch.float32 if dtype == "float32" else torch.bfloat16
+    config = config_from_dir(d)
+    files = ModelFiles(d)
+    base = config.spec(files.names())
+    spec = dataclasses.replace(base, order=(LayerCall(0), LayerCall(1), LayerCall(0), LayerCall(1, cache_of=1)))
+    eng = Engine(config, spec, load_weights(base, files, tdt, DEV), tdt, max_tokens=64 * 4)
+    assert eng.cache.kv_groups[0].n_entries == 3                   # three stores for four runs
+
+    cfg, w = P.read_model(d)
+    S = P.sizes(cfg)
+    ids = tiny.prompts("A", [40], seed=21)[0]
+    pos = list(range(40))
+    x = P.embedding(w["model.embed_tokens.weight"], ids)
+    x = P.decoder_layer(x, w, 0, S, pos)
+    # layer 1, keeping its k and v
+    p = "model.layers.1.self_attn."
+    h1 = P.rms_norm(x, w["model.layers.1.input_layernorm.weight"], S["eps"])
+    k1 = P.rms_norm(P.linear(h1, w[p + "k_proj.weight"]).reshape(40, S["nkv"], S["hd"]), w[p + "k_norm.weight"], S["eps"])
+    cos, sin = P.rope_table(pos, S["hd"], S["theta"])
+    k1 = P.rope_half_split(k1, cos, sin)
+    v1 = P.linear(h1, w[p + "v_proj.weight"]).reshape(40, S["nkv"], S["hd"])
+    x = P.decoder_layer(x, w, 1, S, pos)
+    x = P.decoder_layer(x, w, 0, S, pos)
+    # layer 1 again: its own queries over the first run's keys and values
+    h = P.rms_norm(x, w["model.layers.1.input_layernorm.weight"], S["eps"])
+    q = P.rope_half_split(P.rms_norm(P.linear(h, w[p + "q_proj.weight"]).reshape(40, S["nh"], S["hd"]), w[p + "q_norm.weight"], S["eps"]), cos, sin)
+    a = P.linear(P.causal_attention(q, k1, v1, S["hd"] ** -0.5).reshape(40, -1), w[p + "o_proj.weight"])
+    x = x + a
+    h = P.rms_norm(x, w["model.layers.1.post_attention_layernorm.weight"], S["eps"])
+    x = x + P.swiglu_mlp(h, w["model.layers.1.mlp.gate_proj.weight"], w["model.layers.1.mlp.up_proj.weight"], w["model.layers.1.mlp.down_proj.weight"])
+    ref = P.linear(P.rms_norm(x, w["model.norm.weight"], S["eps"]), P.head_weight(w))
+
+    s = eng.open()
+    got = [eng.step([StepEntry(s, ids[:25], list(range(25)))])]
+    for t in range(25, 40):
+        got.append(eng.step([StepEntry(s, [ids[t]], [0])]))
+    eng.close(s)
+    tiny.assert_logits_close(torch.cat(got), ref, dtype, "layers run twice, shared cache")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_layers_with_and_without_a_window_in_one_model(model_dirs, dtype):
+    """Layer 0 keeps all keys, layer 1 a window of 37: two groups with storage of their own; prompts longer
+    than the window, cut into pieces, then single tokens."""
+    from palm_infra_amd.config import PartSpec, config_from_dir
+    from palm_infra_amd.engine import Engine, StepEntry
+    from palm_infra_amd.weights import ModelFiles, load_weights
+    d = model_dirs["C"][dtype]
+    tdt = torch.float32 if dtype == "float32" else torch.bfloat16
+    config = config_from_dir(d)
+    files = ModelFiles(d)
+    base = config.spec(files.names())
+    layer = base.layers[1]
+    mixer = layer.parts["mixer"]
+    parts = dict(layer.parts)
+    parts["mixer"] = dataclasses.replace(mixer, params=dict(mixer.params, window=37))
+    spec = dataclasses.replace(base, layers=(base.layers[0], dataclasses.replace(layer, parts=parts)))
+    eng = Engine(config, spec, load_weights(base, files, tdt, DEV), tdt, max_tokens=64 * 12)
+    assert sorted(str(g.need.window) for g in eng.cache.kv_groups) == ["37", "None"]
+    eng.step_tokens_per_seq = 50                                     # force long prompts through in pieces
+
+    cfg, w = P.read_model(d)
+    S = P.sizes(cfg)
+
+    def plain(ids):
+        pos = list(range(len(ids)))
+        x = P.embedding(w["model.embed_tokens.weight"], ids)
+        x = P.decoder_layer(x, w, 0, S, pos)
+        x = P.decoder_layer(x, w, 1, S, pos, window=37)
+        return P.linear(P.rms_norm(x, w["model.norm.weight"], S["eps"]), P.head_weight(w))
+
+    reqs = tiny.prompts("C", [180, 60], seed=22)
+    slots = [eng.open(), eng.open()]
+    out = eng.step([StepEntry(slots[0], reqs[0][:160], list(range(160))), StepEntry(slots[1], reqs[1][:55], list(range(55)))])
+    got = [[out[:160]], [out[160:]]]
+    fed = [160, 55]
+    while any(f < len(r) for f, r in zip(fed, reqs)):
+        live = [i for i in range(2) if fed[i] < len(reqs[i])]
+        out = eng.step([StepEntry(slots[i], [reqs[i][fed[i]]], [0]) for i in live])
+        for r_, i in enumerate(live):
+            got[i].append(out[r_:r_ + 1]); fed[i] += 1
+    win = [g for g in eng.cache.kv_groups if g.need.window][0]
+    assert win.table.slot_pages[slots[0]][:2] == [-1, -1]            # pages below the window went back
+    for i in range(2):
+        tiny.assert_logits_close(torch.cat(got[i]), plain(reqs[i]), dtype, f"window model request {i}")
+        eng.close(slots[i])
+    eng.cache.check()

@@ -1,0 +1,159 @@
+"""Safetensors files, the loader's errors and the random-weights mode (no GPU)."""
+import json
+import struct
+
+import pytest
+import torch
+
+import plain_qwen3 as P
+import tiny
+from palm_infra_amd.config import config_from_dict, config_from_dir
+from palm_infra_amd.weights import (ModelFiles, SafetensorsError, SafetensorsFile, WeightError, load_weights,
+                                    random_tensors, write_random_model, write_safetensors)
+
+
+def test_round_trip_is_bit_exact(tmp_path):
+    g = torch.Generator().manual_seed(0)
+    tensors = {"a": torch.randn(3, 5, generator=g), "b": torch.randn(7, generator=g).to(torch.bfloat16),
+               "c": torch.randn(2, 2, generator=g).to(torch.float16), "d": torch.arange(6, dtype=torch.int32).reshape(2, 3)}
+    write_safetensors(tmp_path / "m.safetensors", tensors)
+    f = SafetensorsFile(tmp_path / "m.safetensors")
+    for k, t in tensors.items():
+        got = f.tensor(k)
+        assert got.dtype == t.dtype and got.shape == t.shape
+        assert torch.equal(got.view(torch.uint8) if t.dtype != torch.int32 else got, t.view(torch.uint8) if t.dtype != torch.int32 else t)
+    # and the oracle's own reader agrees
+    write_safetensors(tmp_path / "f.safetensors", {k: t for k, t in tensors.items() if t.is_floating_point()})
+    mine = P.read_safetensors(tmp_path / "f.safetensors")
+    assert torch.equal(mine["b"], tensors["b"].double())
+
+
+def _raw_file(path, header: dict, payload: bytes, hlen=None):
+    raw = json.dumps(header).encode()
+    path.write_bytes(struct.pack("<Q", len(raw) if hlen is None else hlen) + raw + payload)
+
+
+def test_bad_files_are_refused(tmp_path):
+    # the checks of models/safetensors_stream.py:71-118
+    p = tmp_path / "x.safetensors"
+    _raw_file(p, {"t": {"dtype": "F32", "shape": [2, 2], "data_offsets": [0, 12]}}, b"\0" * 12)
+    with pytest.raises(SafetensorsError, match="needs 16"):
+        SafetensorsFile(p)
+    _raw_file(p, {"t": {"dtype": "F32", "shape": [2], "data_offsets": [0, 8]}}, b"\0" * 4)
+    with pytest.raises(SafetensorsError, match="outside the file"):
+        SafetensorsFile(p)
+    _raw_file(p, {"t": {"dtype": "F8_E4M3", "shape": [2], "data_offsets": [0, 2]}}, b"\0" * 2)
+    with pytest.raises(SafetensorsError, match="not supported"):
+        SafetensorsFile(p)
+    _raw_file(p, {}, b"", hlen=1 << 40)
+    with pytest.raises(SafetensorsError, match="exceeds"):
+        SafetensorsFile(p)
+    _raw_file(p, {}, b"", hlen=500)
+    with pytest.raises(SafetensorsError, match="cut off"):
+        SafetensorsFile(p)
+    with pytest.raises(FileNotFoundError, match="No safetensors"):
+        ModelFiles(tmp_path / "nowhere")
+
+
+def test_one_error_lists_missing_unexpected_and_misshapen(tmp_path):
+    tensors = tiny.sharpened_tensors("A", "float32")
+    del tensors["model.layers.1.self_attn.k_proj.weight"]
+    del tensors["model.norm.weight"]
+    tensors["model.layers.0.mlp.down_proj.weight"] = torch.zeros(64, 100)
+    tensors["model.layers.0.self_attn.q_norm.weight"] = torch.zeros(32)
+    tensors["model.layers.7.mlp.up_proj.weight"] = torch.zeros(2, 2)
+    tensors["rotary.inv_freq"] = torch.zeros(8)
+    (tmp_path / "config.json").write_text(json.dumps(tiny.CONFIGS["A"]))
+    write_safetensors(tmp_path / "model.safetensors", tensors)
+    cfg = config_from_dir(tmp_path)
+    files = ModelFiles(tmp_path)
+    with pytest.raises(WeightError) as e:
+        load_weights(cfg.spec(files.names()), files, torch.float32, "cpu")
+    err = e.value
+    assert sorted(err.missing) == ["model.layers.1.self_attn.k_proj.weight", "model.norm.weight"]
+    assert sorted(err.unexpected) == ["model.layers.7.mlp.up_proj.weight", "rotary.inv_freq"]
+    assert sorted(n for n, _, _ in err.wrong_shape) == ["model.layers.0.mlp.down_proj.weight", "model.layers.0.self_attn.q_norm.weight"]
+    text = str(err)
+    for word in ("missing", "unexpected", "wrong shapes", "k_proj", "inv_freq", "expected [64, 128], file has [64, 100]"):
+        assert word in text, word
+
+
+def test_tied_config_with_a_stored_head_is_reported(tmp_path):
+    tensors = tiny.sharpened_tensors("A", "float32")
+    tensors["lm_head.weight"] = torch.zeros(256, 64)
+    (tmp_path / "config.json").write_text(json.dumps(tiny.CONFIGS["A"]))      # tie_word_embeddings: true
+    write_safetensors(tmp_path / "model.safetensors", tensors)
+    files = ModelFiles(tmp_path)
+    with pytest.raises(WeightError) as e:
+        load_weights(config_from_dir(tmp_path).spec(files.names()), files, torch.float32, "cpu")
+    assert e.value.unexpected == ["lm_head.weight"]
+
+
+def test_what_is_kept_in_which_precision(tmp_path):
+    cfg = config_from_dict(tiny.CONFIGS["B"])
+    d = tiny.write_model("B", tmp_path / "bf", "bfloat16")
+    files = ModelFiles(d)
+    spec = cfg.spec(files.names())
+    w = load_weights(spec, files, torch.bfloat16, "cpu")
+    mixer = spec.layers[0].parts["mixer"]
+    assert w.get(mixer.tensors["qkv"]).dtype == torch.bfloat16
+    assert w.get(mixer.tensors["qkv"]).shape == (8 * 32 + 2 * 32, 96)
+    assert w.get(mixer.parts["q_norm"].tensors["weight"]).dtype == torch.float32      # vectors are widened
+    assert w.get(spec.embedding.tensors["table"]).dtype == torch.bfloat16
+    w32 = load_weights(spec, files, torch.float32, "cpu")
+    assert w32.get(mixer.tensors["qkv"]).dtype == torch.float32
+    # a tensor stored in 32-bit stays so in the bfloat16 mode
+    d32 = tiny.write_model("B", tmp_path / "f32", "float32")
+    f32 = ModelFiles(d32)
+    wmix = load_weights(spec, f32, torch.bfloat16, "cpu")
+    assert wmix.get(mixer.tensors["qkv"]).dtype == torch.float32
+    # the joined matrix is q rows, k rows, v rows
+    q = f32.tensor("model.layers.0.self_attn.q_proj.weight")
+    v = f32.tensor("model.layers.0.self_attn.v_proj.weight")
+    joined = wmix.get(mixer.tensors["qkv"])
+    assert torch.equal(joined[:256], q) and torch.equal(joined[-32:], v)
+
+
+def test_tied_head_is_the_embedding_itself(tmp_path):
+    d = tiny.write_model("A", tmp_path / "a", "float32")
+    files = ModelFiles(d)
+    spec = config_from_dir(d).spec(files.names())
+    w = load_weights(spec, files, torch.float32, "cpu")
+    assert w.get(spec.head.tensors["weight"]).data_ptr() == w.get(spec.embedding.tensors["table"]).data_ptr()
+
+
+def test_sharded_checkpoint_with_index(tmp_path):
+    tensors = tiny.sharpened_tensors("A", "float32")
+    names = list(tensors)
+    half = len(names) // 2
+    write_safetensors(tmp_path / "model-00001-of-00002.safetensors", {n: tensors[n] for n in names[:half]})
+    write_safetensors(tmp_path / "model-00002-of-00002.safetensors", {n: tensors[n] for n in names[half:]})
+    index = {"weight_map": {n: ("model-00001-of-00002.safetensors" if i < half else "model-00002-of-00002.safetensors")
+                            for i, n in enumerate(names)}}
+    (tmp_path / "model.safetensors.index.json").write_text(json.dumps(index))
+    files = ModelFiles(tmp_path)
+    assert sorted(files.names()) == sorted(names)
+    assert torch.equal(files.tensor(names[-1]), tensors[names[-1]])
+    (tmp_path / "model.safetensors.index.json").unlink()       # the glob patterns of models/qwen3.py:39-54
+    assert sorted(ModelFiles(tmp_path).names()) == sorted(names)
+
+
+def test_random_weights_mode_writes_a_loadable_folder(tmp_path):
+    cfg = config_from_dict(tiny.CONFIGS["B"])
+    d1 = write_random_model(cfg, 5, tmp_path / "one")
+    d2 = write_random_model(tiny.CONFIGS["B"], 5, tmp_path / "two")
+    d3 = write_random_model(cfg, 6, tmp_path / "three")
+    assert (d1 / "config.json").is_file() and (d1 / "model.safetensors").is_file()
+    assert config_from_dir(d1) == cfg
+    a, b, c = (ModelFiles(d) for d in (d1, d2, d3))
+    n = "model.layers.2.mlp.up_proj.weight"
+    assert a.dtype_name(n) == "BF16"
+    assert torch.equal(a.tensor(n).float(), b.tensor(n).float())            # the seed decides
+    assert not torch.equal(a.tensor(n).float(), c.tensor(n).float())
+    load_weights(cfg.spec(a.names()), a, torch.bfloat16, "cpu")
+    t = random_tensors(cfg.spec(), 5, "float32")
+    assert abs(float(t[n].std()) - 0.02) < 2e-3 and abs(float(t["model.norm.weight"].mean()) - 1.0) < 2e-2
+    # a tensor depends on the seed and its name only: a model with fewer layers starts the same
+    small = config_from_dict(dict(tiny.CONFIGS["B"], num_hidden_layers=1))
+    assert torch.equal(random_tensors(small.spec(), 5, "float32")["model.layers.0.mlp.up_proj.weight"],
+                       t["model.layers.0.mlp.up_proj.weight"])
