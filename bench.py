@@ -1,0 +1,189 @@
+"""Measures generation with random weights of Qwen3-8B's layer sizes on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One JSON line: ``value`` is decoded tokens a second at batch 8 with 2,048-token contexts (a step is one
+decode step of the whole batch: the model's forward pass from the cache, greedy choice on the device and
+the copy of the chosen tokens to the host, as the generation loop does it).  The same line holds the
+prefill of 2,048 tokens, the decode step's fraction of the HBM roofline, and decode at batch 1 and 64.
+
+The protocol is the reference's (examples/bench.cpp:564-590, docs/performance.md:127-131): synthetic
+token ids, no stop token, warm-up before the timed run, decode timed from an existing context.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+# MI355X, published: HBM3E 8 TB/s; dense matrix cores 2.5 PFLOP/s for bfloat16
+PEAK_HBM_GBS = 8000.0
+PEAK_FLOPS = {"bf16": 2.5e15, "fp16": 2.5e15, "fp8": 5.0e15, "fp32": 157.3e12}
+
+# BASELINE.json configs[2]: Qwen3-8B sizes
+QWEN3_8B = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_size=151936, hidden_size=4096,
+                num_hidden_layers=36, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
+                intermediate_size=12288, rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=False,
+                max_position_embeddings=40960)
+CONTEXT = 2048          # tokens every sequence holds when decoding starts
+PREFILL_TOKENS = 2048
+BATCH = 8
+FULL_LAYERS = 36
+
+
+def layer_params(c) -> int:
+    q, kv = c["num_attention_heads"] * c["head_dim"], c["num_key_value_heads"] * c["head_dim"]
+    H, I = c["hidden_size"], c["intermediate_size"]
+    return (q + 2 * kv) * H + H * q + 3 * H * I
+
+
+def decode_bytes(c, batch: int, context: float, itemsize: int = 2) -> float:
+    """What one decode step has to read: every weight it uses once (layers and head; the embedding only
+    its batch rows) and the keys and values of the live requests."""
+    L = c["num_hidden_layers"]
+    weights = (L * layer_params(c) + c["vocab_size"] * c["hidden_size"]) * itemsize
+    kv = 2 * c["num_key_value_heads"] * c["head_dim"] * itemsize * L * context * batch
+    return weights + kv
+
+
+def prefill_flops(c, tokens: int) -> float:
+    """Linear layers for every token, causal attention (half of the square), the head for one row."""
+    L = c["num_hidden_layers"]
+    linear = 2.0 * tokens * L * layer_params(c)
+    attention = L * 4.0 * c["num_attention_heads"] * c["head_dim"] * tokens * tokens / 2.0
+    return linear + attention + 2.0 * c["hidden_size"] * c["vocab_size"]
+
+
+def random_ids(n: int, vocab: int, seed: int) -> list:
+    import torch
+    return torch.randint(0, vocab, (n,), generator=torch.Generator().manual_seed(seed)).tolist()
+
+
+def fill_contexts(engine, batch: int, context: int, vocab: int, group: int = 8):
+    """Open `batch` sequences and put `context` tokens into each, a few sequences a step."""
+    from palm_infra_amd.engine import StepEntry
+    slots = [engine.open() for _ in range(batch)]
+    for g in range(0, batch, group):
+        engine.step([StepEntry(s, random_ids(context, vocab, 100 + g + j), []) for j, s in enumerate(slots[g:g + group])])
+    return slots
+
+
+def time_decode(engine, sampler, slots, steps: int, warmup: int, vocab: int):
+    """ms per decode step over `steps` steps after `warmup`, tokens chosen greedily and fed back."""
+    import torch
+    from palm_infra_amd.engine import StepEntry
+    from palm_infra_amd.sampling import SequenceSampling
+    states = [SequenceSampling(i) for i in range(len(slots))]
+    tokens = [random_ids(1, vocab, 7 + i)[0] for i in range(len(slots))]
+
+    def one():
+        nonlocal tokens
+        logits = engine.step([StepEntry(s, [t], [0]) for s, t in zip(slots, tokens)])
+        tokens = sampler.sample(logits, states).tolist()
+
+    for _ in range(warmup):
+        one()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        one()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1000.0 / steps
+
+
+def time_prefill(engine, tokens: int, vocab: int, repeats: int = 3) -> float:
+    """Best ms of `repeats` for one fresh sequence of `tokens` tokens, logits at the last place."""
+    import torch
+    from palm_infra_amd.engine import StepEntry
+    best = float("inf")
+    for r in range(repeats + 1):            # the first run warms up
+        ids = random_ids(tokens, vocab, 500 + r)
+        slot = engine.open()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        engine.step([StepEntry(slot, ids, [tokens - 1])])
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 1000.0
+        engine.close(slot)
+        if r > 0:
+            best = min(best, ms)
+    return best
+
+
+def main(argv=None) -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128, help="timed decode steps (the workload's 128)")
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=FULL_LAYERS, help="fewer layers than the model has, for a quick look")
+    ap.add_argument("--batch", type=int, default=BATCH)
+    ap.add_argument("--no-points", action="store_true", help="skip batch 1 and batch 64")
+    args = ap.parse_args(argv)
+    if args.gpus != 1:
+        print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not measured")
+        return 2
+
+    import torch
+    from palm_infra_amd.engine import Engine
+    from palm_infra_amd.sampling import GREEDY, DeviceSampler
+
+    cfg = dict(QWEN3_8B, num_hidden_layers=args.layers)
+    vocab = cfg["vocab_size"]
+    room = CONTEXT + args.warmup + args.steps + 64
+    biggest = max(args.batch, 1 if args.no_points else 64)
+    t_load = time.perf_counter()
+    engine = Engine.from_config(cfg, seed=0, dtype="bfloat16", max_tokens=biggest * room + PREFILL_TOKENS + 64)
+    torch.cuda.synchronize()
+    load_s = time.perf_counter() - t_load
+    sampler = DeviceSampler(GREEDY)
+
+    prefill_ms = time_prefill(engine, PREFILL_TOKENS, vocab)
+    pf = prefill_flops(cfg, PREFILL_TOKENS)
+
+    def decode_at(batch: int, steps: int, warmup: int) -> float:
+        slots = fill_contexts(engine, batch, CONTEXT, vocab)
+        ms = time_decode(engine, sampler, slots, steps, warmup, vocab)
+        for s in slots:
+            engine.close(s)
+        return ms
+
+    ms_step = decode_at(args.batch, args.steps, args.warmup)
+    value = args.batch * 1000.0 / ms_step
+    points = {}
+    if not args.no_points:
+        points["decode_b1"] = round(1 * 1000.0 / decode_at(1, args.steps, args.warmup), 2)
+        points["decode_b64"] = round(64 * 1000.0 / decode_at(64, max(16, args.steps // 4), args.warmup), 2)
+
+    mid_context = CONTEXT + args.warmup + args.steps / 2.0
+    bytes_step = decode_bytes(cfg, args.batch, mid_context)
+    achieved = bytes_step / (ms_step * 1e-3) / 1e9
+    record = {
+        "metric": "decode tok/s at batch 8, 2048-token contexts (Qwen3-8B sizes, bf16)",
+        "value": round(value, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic: random weights, uniform random token ids, no stop token",
+        "config": {"model": "Qwen3-8B sizes, random weights", "global_batch": args.batch, "seq_len": CONTEXT,
+                   "parallelism": "single GPU", "layers": args.layers, "layers_of_model": FULL_LAYERS,
+                   "hidden_size": cfg["hidden_size"], "heads": cfg["num_attention_heads"],
+                   "kv_heads": cfg["num_key_value_heads"], "head_dim": cfg["head_dim"],
+                   "intermediate_size": cfg["intermediate_size"], "vocab_size": vocab, "rope_theta": cfg["rope_theta"],
+                   "rms_norm_eps": cfg["rms_norm_eps"], "tied_head": False, "cache_context": 4096,
+                   "prefill_tokens": PREFILL_TOKENS, "decode_steps": args.steps, "load_s": round(load_s, 1)},
+        "prefill": {"value": round(PREFILL_TOKENS * 1000.0 / prefill_ms, 1), "tokens": PREFILL_TOKENS,
+                    "ms": round(prefill_ms, 3), "frac": round(pf / (prefill_ms * 1e-3) / PEAK_FLOPS["bf16"], 4)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": round(achieved / PEAK_HBM_GBS, 4)},
+        "points": points,
+    }
+    print(json.dumps(record), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -8,7 +8,7 @@ other kinds of layers, fixed-size state buffers without a length that ``reset()`
 
 * Layers whose mixers ask for the same kind of storage (same kv heads, head size and window) form a
   *group*.  A group has storage of its own: ``k`` and ``v`` of shape
-  ``[layers of the group, pages + 1, kv_heads, PAGE_TOKENS, head_dim]`` and one page table (the pages
+  ``[layers of the group, pages + 1, kv_heads, PAGE_TOKENS, head_dim]`` (``v`` with the last two swapped) and one page table (the pages
   of every slot), shared by the group's layers.  The last page is never handed out: rows that pad a
   batch write there.
 * State groups are ``[layers of the group, slots + 1, *shape]``, zeroed when a slot is opened.
@@ -45,9 +45,12 @@ class KVGroup:
         self.need, self.n_entries, self.n_pages = need, n_entries, n_pages
         self.table = PageTable(n_pages, n_slots, max_pages_per_slot, need.window)
         self.pad_page = n_pages
-        shape = (n_entries, n_pages + 1, need.num_kv_heads, PAGE_TOKENS, need.head_dim)
-        self.k = torch.zeros(shape, dtype=dtype, device=device)
-        self.v = torch.zeros(shape, dtype=dtype, device=device)
+        # values are kept transposed (positions innermost): both products of attention then sum over an
+        # index that is contiguous in memory
+        self.k = torch.zeros((n_entries, n_pages + 1, need.num_kv_heads, PAGE_TOKENS, need.head_dim), dtype=dtype,
+                             device=device)
+        self.v = torch.zeros((n_entries, n_pages + 1, need.num_kv_heads, need.head_dim, PAGE_TOKENS), dtype=dtype,
+                             device=device)
         self.table_host = torch.full((n_slots + 1, max_pages_per_slot), self.pad_page, dtype=torch.int32)
         self.table_dev = self.table_host.to(device)
 

@@ -1,0 +1,280 @@
+// Causal grouped-query attention over the paged cache on the matrix cores, bfloat16, compiled for one
+// head size (PALM_HEAD_DIM, a multiple of 16).  Same semantics as the exact kernel
+// (models/qwen3.py:336-341; kernels/attention.cpp:84-217, 937-962): head h reads kv head h / (nh / nkv),
+// keys j <= p of the query's own sequence (j > p - window with a window), softmax in 32-bit with the
+// running maximum, o = sum_j p_j v_j.
+//
+// Cache layouts: K [pages, nkv, 64 keys, hd] (a key's row is contiguous); V is kept transposed,
+// [pages, nkv, hd, 64 keys], so that for both products the summed index is contiguous in memory.
+//
+// Formulation (transposed, so that no operand has to be shuffled between the two products):
+//   S^T[key, query] = sum_d K[key, d] Q[query, d]        A = K rows, B = Q rows
+//   O^T[d, query]   = sum_key V^T[d, key] P^T[key, query]  A = V^T rows, B = P^T = the registers S^T left
+// A 16x16 result tile leaves lane (q, g) with rows 4g..4g+3 of column q.  Two S^T tiles therefore give a
+// lane eight keys of one query, which is exactly a B operand of the second product if the tiles' rows are
+// chosen as keys {8g'+0..3} and {8g'+4..7} of a run of 32 keys: then the eight keys of lane group g are
+// keys 8g..8g+7, one 16-byte read of a V^T row.  All softmax statistics are per column, i.e. per lane.
+//
+// decode:  one wave per (sequence, kv head, slice of the key range); the G = nh / nkv query heads of the
+//          kv head are the columns.  Partial (max, sum, output) go to a workspace and a second kernel
+//          merges the slices.  The kernel is bound by reading K and V once.
+// prefill: one block of four waves per (sequence, kv head, 16 query positions); wave w owns the columns
+//          of query head w of the group (more heads: more passes).
+#include "mfma.h"
+
+#ifndef PALM_HEAD_DIM
+#error "compile with -DPALM_HEAD_DIM=<head size>"
+#endif
+
+constexpr int HD = PALM_HEAD_DIM;
+static_assert(HD % 16 == 0 && HD >= 16 && HD <= 256, "head size must be a multiple of 16, at most 256");
+constexpr int CHUNKS = HD / 8;               // 16-byte chunks in a row of K or Q
+constexpr int KSTEPS = (CHUNKS + 3) / 4;     // MFMA steps over d (32 values each; the last may be half empty)
+constexpr int DTILES = HD / 16;              // 16-row tiles of O^T
+constexpr float LOG2E = 1.4426950408889634f;
+
+PALM_DEFINE_LAST_ERROR()
+PALM_API int palm_attention_head_dim() { return HD; }
+
+struct Columns {          // softmax state of this lane's query column, and its share of the output
+    float m, l;
+    f32x4 o[DTILES];
+};
+
+// The key that row r of S^T tile `t` (0..3) of a page stands for: tiles 2h and 2h+1 cover keys 32h..32h+31.
+__device__ inline int tile_key(int t, int r) { return (t / 2) * 32 + (r / 4) * 8 + (t % 2) * 4 + (r % 4); }
+
+// One page: scores of its 64 keys against the columns' queries, online softmax, and the weighted values.
+// kp: K of this page and kv head [64, HD]; vp: V^T [HD, 64].  Keys outside [lo, hi] (in-page indices) are
+// masked.  qv: the B operand of the first product (this lane's query, chunks g, g+4, ..).
+__device__ inline void attend_page(const bf16_t* __restrict__ kp, const bf16_t* __restrict__ vp,
+                                   const bf16x8 (&qv)[KSTEPS], int lo, int hi, float scale_log2, Columns& c,
+                                   int r, int g) {
+    f32x4 s[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        const bf16_t* krow = kp + (size_t)tile_key(t, r) * HD;
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < KSTEPS; ++j) {
+            const int chunk = j * 4 + g;
+            const bf16x8 kv = chunk < CHUNKS ? load_bf16x8(krow + chunk * 8) : zero_bf16x8();
+            acc = mfma_16x16x32(kv, qv[j], acc);
+        }
+        s[t] = acc;
+    }
+    // this lane holds, for its query, keys tile_key(t, 4g + i)
+    float mx = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int key = tile_key(t, 4 * g + i);
+            const float v = (key >= lo && key <= hi) ? s[t][i] * scale_log2 : -INFINITY;
+            s[t][i] = v;
+            mx = fmaxf(mx, v);
+        }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+    const float m_new = fmaxf(c.m, mx);
+    // A column can reach a page of its tile in which it sees no key yet (a window's lower edge, a page
+    // border inside a tile of queries): its maximum is still -inf then; subtracting 0 instead keeps
+    // every exponential at exp2(-inf) = 0 rather than NaN.
+    const float m_sub = m_new == -INFINITY ? 0.f : m_new;
+    const float alpha = exp2f(c.m - m_sub);             // c.m = -inf before the first visible key: 0
+    float sum = 0.f;
+    bf16x8 pv[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float p = exp2f(s[2 * h + e / 4][e % 4] - m_sub);
+            sum += p;
+            pv[h][e] = (__bf16)p;
+        }
+    c.l = c.l * alpha + sum;                            // this lane's share; the groups are added at the end
+    c.m = m_new;
+#pragma unroll
+    for (int dt = 0; dt < DTILES; ++dt) {
+        f32x4 acc = c.o[dt] * alpha;
+        const bf16_t* vrow = vp + (size_t)(dt * 16 + r) * PAGE_TOKENS;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) acc = mfma_16x16x32(load_bf16x8(vrow + h * 32 + g * 8), pv[h], acc);
+        c.o[dt] = acc;
+    }
+}
+
+__device__ inline void load_query(const bf16_t* qrow, bool valid, int g, bf16x8 (&qv)[KSTEPS]) {
+#pragma unroll
+    for (int j = 0; j < KSTEPS; ++j) {
+        const int chunk = j * 4 + g;
+        qv[j] = (valid && chunk < CHUNKS) ? load_bf16x8(qrow + chunk * 8) : zero_bf16x8();
+    }
+}
+
+// ---- decode ---------------------------------------------------------------------------------------
+// grid (slices, nkv * query groups, sequences), one wave each.  Workspace per (sequence, head, slice):
+// m, l, then HD floats of the unnormalised output.
+__global__ __launch_bounds__(WAVE) void attention_decode_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+    const int* __restrict__ block_table, int max_pages, const int* __restrict__ seq_slot,
+    const int* __restrict__ seq_start, int nh, int nkv, float scale_log2, int window, int n_slices,
+    float* __restrict__ work, bf16_t* __restrict__ out) {
+    const int slice = blockIdx.x, b = blockIdx.z;
+    const int G = nh / nkv, groups = (G + 15) / 16;
+    const int kvh = blockIdx.y / groups, qg = blockIdx.y % groups;
+    const int lane = threadIdx.x, r = lane % 16, g = lane / 16;
+    const int pos = seq_start[b];                       // the query's position; keys 0..pos are in the cache
+    const int first = window > 0 ? max(0, pos - window + 1) : 0;
+    const int page_lo = first / PAGE_TOKENS, n_pages = pos / PAGE_TOKENS - page_lo + 1;
+    const int per = (n_pages + n_slices - 1) / n_slices;
+    const int p0 = page_lo + slice * per, p1 = min(p0 + per, page_lo + n_pages);
+    const int head = kvh * G + qg * 16 + r;             // this lane's query head (column r)
+    const bool valid = qg * 16 + r < G;
+
+    bf16x8 qv[KSTEPS];
+    load_query(q + ((size_t)b * nh + (valid ? head : 0)) * HD, valid, g, qv);
+    Columns c;
+    c.m = -INFINITY;
+    c.l = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < DTILES; ++dt) c.o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    const int* pages = block_table + (size_t)seq_slot[b] * max_pages;
+    for (int p = p0; p < p1; ++p) {
+        const size_t base = ((size_t)pages[p] * nkv + kvh) * PAGE_TOKENS * HD;
+        attend_page(k_cache + base, v_cache + base, qv, first - p * PAGE_TOKENS, pos - p * PAGE_TOKENS, scale_log2, c, r, g);
+    }
+    float l = c.l;
+    l += __shfl_xor(l, 16, WAVE);
+    l += __shfl_xor(l, 32, WAVE);
+    if (!valid) return;
+    if (n_slices == 1) {
+        const float inv = 1.0f / l;
+        bf16_t* o = out + ((size_t)b * nh + head) * HD;
+#pragma unroll
+        for (int dt = 0; dt < DTILES; ++dt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) o[dt * 16 + 4 * g + i] = f32_to_bf16(c.o[dt][i] * inv);
+        return;
+    }
+    float* w = work + (((size_t)b * nh + head) * n_slices + slice) * (HD + 2);
+    if (g == 0) { w[0] = c.m; w[1] = l; }               // an empty slice leaves m = -inf, l = 0
+#pragma unroll
+    for (int dt = 0; dt < DTILES; ++dt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) w[2 + dt * 16 + 4 * g + i] = c.o[dt][i];
+}
+
+// one block per (sequence, head): merge the slices in a fixed order
+__global__ void attention_merge_kernel(const float* __restrict__ work, int n_slices, bf16_t* __restrict__ out) {
+    const float* w = work + (size_t)blockIdx.x * n_slices * (HD + 2);
+    float m = -INFINITY;
+    for (int s = 0; s < n_slices; ++s) m = fmaxf(m, w[s * (HD + 2)]);
+    float l = 0.f;
+    for (int s = 0; s < n_slices; ++s) l += w[s * (HD + 2) + 1] * exp2f(w[s * (HD + 2)] - m);
+    for (int d = threadIdx.x; d < HD; d += blockDim.x) {
+        float o = 0.f;
+        for (int s = 0; s < n_slices; ++s) o += w[s * (HD + 2) + 2 + d] * exp2f(w[s * (HD + 2)] - m);
+        out[(size_t)blockIdx.x * HD + d] = f32_to_bf16(o / l);
+    }
+}
+
+PALM_API int palm_attention_decode_workspace_floats(int n_seqs, int nh, int n_slices) {
+    return n_seqs * nh * n_slices * (HD + 2);
+}
+
+PALM_API int palm_attention_decode(hipStream_t stream, const void* q, const void* k_cache, const void* v_cache,
+                                   const int* block_table, int max_pages, const int* seq_slot, const int* seq_start,
+                                   int n_seqs, int nh, int nkv, int hd, float scale, int window, int n_slices,
+                                   float* work, void* out) {
+    PALM_CHECK(hd == HD, "attention_decode: this library was built for head size %d, not %d", HD, hd);
+    PALM_CHECK(n_seqs >= 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attention_decode: seqs=%d heads=%d kv=%d", n_seqs, nh, nkv);
+    PALM_CHECK(n_slices >= 1 && n_slices <= 65535, "attention_decode: %d slices", n_slices);
+    PALM_CHECK(n_slices == 1 || work, "attention_decode: more than one slice needs a workspace");
+    PALM_CHECK(window >= 0 && max_pages > 0, "attention_decode: window=%d max_pages=%d", window, max_pages);
+    if (n_seqs == 0) return 0;
+    const int groups = (nh / nkv + 15) / 16;
+    PALM_CHECK(nkv * groups <= 65535 && n_seqs <= 65535, "attention_decode: grid too large");
+    dim3 grid(n_slices, nkv * groups, n_seqs);
+    attention_decode_kernel<<<grid, WAVE, 0, stream>>>((const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache,
+                                                      block_table, max_pages, seq_slot, seq_start, nh, nkv, scale * LOG2E,
+                                                      window, n_slices, work, (bf16_t*)out);
+    PALM_LAUNCHED();
+    if (n_slices > 1) {
+        attention_merge_kernel<<<n_seqs * nh, HD <= 64 ? 64 : 128, 0, stream>>>(work, n_slices, (bf16_t*)out);
+        PALM_LAUNCHED();
+    }
+    return 0;
+}
+
+// ---- prefill --------------------------------------------------------------------------------------
+// grid (query tiles of 16 positions, nkv, sequences); four waves; wave w takes query heads w, w + 4, ..
+// of the kv head's group, so the waves of a block read the same pages of K and V.
+__global__ __launch_bounds__(4 * WAVE) void attention_prefill_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+    const int* __restrict__ block_table, int max_pages, const int* __restrict__ seq_slot,
+    const int* __restrict__ seq_start, const int* __restrict__ seq_new, const int* __restrict__ cu_new, int nh,
+    int nkv, float scale_log2, int window, bf16_t* __restrict__ out) {
+    const int b = blockIdx.z, kvh = blockIdx.y;
+    const int q0 = blockIdx.x * 16;
+    const int n_new = seq_new[b];
+    if (q0 >= n_new) return;
+    const int G = nh / nkv;
+    const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE, r = lane % 16, g = lane / 16;
+    const int start = seq_start[b];
+    const bool valid = q0 + r < n_new;                  // column r is query position q0 + r of the step
+    const int pos = start + min(q0 + r, n_new - 1);     // its position in the sequence
+    const int row = cu_new[b] + min(q0 + r, n_new - 1);
+    // the tile's key range: from the first key of its first query to the last query's own position
+    const int tile_last = start + min(q0 + 15, n_new - 1);
+    const int tile_first = window > 0 ? max(0, start + q0 - window + 1) : 0;
+    const int my_first = window > 0 ? max(0, pos - window + 1) : 0;
+    const int* pages = block_table + (size_t)seq_slot[b] * max_pages;
+
+    for (int hq = wave; hq < G; hq += 4) {
+        const int head = kvh * G + hq;
+        bf16x8 qv[KSTEPS];
+        load_query(q + ((size_t)row * nh + head) * HD, true, g, qv);
+        Columns c;
+        c.m = -INFINITY;
+        c.l = 0.f;
+#pragma unroll
+        for (int dt = 0; dt < DTILES; ++dt) c.o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int p = tile_first / PAGE_TOKENS; p <= tile_last / PAGE_TOKENS; ++p) {
+            const size_t base = ((size_t)pages[p] * nkv + kvh) * PAGE_TOKENS * HD;
+            // a column whose own range misses this page entirely still needs a finite maximum: its scores are
+            // all -inf then and the page adds nothing, which the guard below keeps free of NaN
+            attend_page(k_cache + base, v_cache + base, qv, my_first - p * PAGE_TOKENS, pos - p * PAGE_TOKENS, scale_log2, c, r, g);
+        }
+        float l = c.l;
+        l += __shfl_xor(l, 16, WAVE);
+        l += __shfl_xor(l, 32, WAVE);
+        if (valid) {
+            const float inv = 1.0f / l;
+            bf16_t* o = out + ((size_t)row * nh + head) * HD;
+#pragma unroll
+            for (int dt = 0; dt < DTILES; ++dt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) o[dt * 16 + 4 * g + i] = f32_to_bf16(c.o[dt][i] * inv);
+        }
+    }
+}
+
+PALM_API int palm_attention_prefill(hipStream_t stream, const void* q, const void* k_cache, const void* v_cache,
+                                    const int* block_table, int max_pages, const int* seq_slot, const int* seq_start,
+                                    const int* seq_new, const int* cu_new, int n_seqs, int max_new, int nh, int nkv,
+                                    int hd, float scale, int window, void* out) {
+    PALM_CHECK(hd == HD, "attention_prefill: this library was built for head size %d, not %d", HD, hd);
+    PALM_CHECK(n_seqs >= 0 && max_new >= 0 && nh > 0 && nkv > 0 && nh % nkv == 0,
+               "attention_prefill: seqs=%d max_new=%d heads=%d kv=%d", n_seqs, max_new, nh, nkv);
+    PALM_CHECK(window >= 0 && max_pages > 0, "attention_prefill: window=%d max_pages=%d", window, max_pages);
+    if (n_seqs == 0 || max_new == 0) return 0;
+    PALM_CHECK(nkv <= 65535 && n_seqs <= 65535, "attention_prefill: grid too large");
+    dim3 grid((max_new + 15) / 16, nkv, n_seqs);
+    attention_prefill_kernel<<<grid, 4 * WAVE, 0, stream>>>((const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache,
+                                                           block_table, max_pages, seq_slot, seq_start, seq_new, cu_new, nh,
+                                                           nkv, scale * LOG2E, window, (bf16_t*)out);
+    PALM_LAUNCHED();
+    return 0;
+}

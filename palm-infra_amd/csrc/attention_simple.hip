@@ -6,6 +6,7 @@
 // head h reads kv head h / (nh / nkv); s_j = scale * q . k_j for the keys j <= p of the query's own
 // sequence (and j > p - window if there is a window); softmax with the running maximum subtracted;
 // o = sum_j p_j v_j.  The keys of the step's own tokens are already in the cache when this runs.
+// K is [pages, nkv, 64, hd]; V is kept transposed, [pages, nkv, hd, 64].
 //
 // One block of four waves per (query, head).  A wave takes every fourth page of the key range; inside
 // a page each lane scores one key, the wave keeps a running (max, sum, output) and the four partial
@@ -67,11 +68,10 @@ __global__ __launch_bounds__(ATT_WAVES * WAVE) void attention_simple_kernel(
         const int j_last = min(pos, pg * PAGE_TOKENS + PAGE_TOKENS - 1) - pg * PAGE_TOKENS;
         for (int jj = j_first; jj <= j_last; ++jj) {
             const float pj = __shfl(p, jj, WAVE);   // jj is the same in every lane
-            const T* vr = vp + (size_t)jj * hd;
 #pragma unroll
             for (int i = 0; i < ATT_ACC; ++i) {
                 const int d = lane + i * WAVE;
-                if (d < hd) acc[i] = fmaf(pj, to_float(vr[d]), acc[i]);
+                if (d < hd) acc[i] = fmaf(pj, to_float(vp[(size_t)d * PAGE_TOKENS + jj]), acc[i]);
             }
         }
     }

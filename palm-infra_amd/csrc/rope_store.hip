@@ -9,8 +9,9 @@
 // tokens, made once per step by the part that owns the position encoding.
 //
 // Layouts: qkv [n_tokens, (nh + 2 nkv) * hd] as the projection writes it (q heads, k heads, v heads);
-// q_out [n_tokens, nh * hd]; cache [pages, nkv, PAGE_TOKENS, hd]; page of position p of a slot is
-// block_table[slot * max_pages + p / PAGE_TOKENS].
+// q_out [n_tokens, nh * hd]; key cache [pages, nkv, PAGE_TOKENS, hd]; value cache transposed,
+// [pages, nkv, hd, PAGE_TOKENS] (the attention kernels sum over keys, which must be contiguous for the
+// matrix cores); page of position p of a slot is block_table[slot * max_pages + p / PAGE_TOKENS].
 #include "common.h"
 
 constexpr int MAX_HEAD_DIM = 512;
@@ -60,14 +61,20 @@ __global__ __launch_bounds__(WAVE) void qk_norm_rope_store_kernel(
         __syncthreads();
     }
 
+    if (kind == 2) {
+        const int g = head - nh - nkv;
+        const int page = block_table[(size_t)tok_slot[t] * max_pages + pos / PAGE_TOKENS];
+        T* dst = v_cache + ((size_t)page * nkv + g) * hd * PAGE_TOKENS + pos % PAGE_TOKENS;
+        for (int d = lane; d < hd; d += WAVE) dst[(size_t)d * PAGE_TOKENS] = from_float<T>(vals[d]);
+        return;
+    }
     T* dst;
     if (kind == 0) {
         dst = q_out + ((size_t)t * nh + head) * hd;
     } else {
-        const int g = kind == 1 ? head - nh : head - nh - nkv;
+        const int g = head - nh;
         const int page = block_table[(size_t)tok_slot[t] * max_pages + pos / PAGE_TOKENS];
-        T* base = kind == 1 ? k_cache : v_cache;
-        dst = base + (((size_t)page * nkv + g) * PAGE_TOKENS + pos % PAGE_TOKENS) * hd;
+        dst = k_cache + (((size_t)page * nkv + g) * PAGE_TOKENS + pos % PAGE_TOKENS) * hd;
     }
     for (int d = lane; d < hd; d += WAVE) dst[d] = from_float<T>(vals[d]);
 }

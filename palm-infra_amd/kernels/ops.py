@@ -31,6 +31,7 @@ _SIGNATURES = {
     "palm_rope_table": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int],
     "palm_attention_simple": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                               c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
+    "palm_linear_thin": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int],
     "palm_argmax": [c_void_p, c_void_p, c_int, c_int, c_void_p],
     "palm_apply_penalties": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_float, c_float, c_float],
     "palm_sample": [c_void_p, c_void_p, c_int, c_int, c_void_p, c_float, c_int, c_float, c_float, c_void_p, c_void_p],
@@ -174,7 +175,8 @@ def linear_exact(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None
 def _check_cache(what, k_cache, v_cache, block_table, nkv, hd):
     _need(k_cache.dim() == 4 and k_cache.shape[1:] == (nkv, PAGE_TOKENS, hd),
           f"{what}: key cache {tuple(k_cache.shape)} is not [pages, {nkv}, {PAGE_TOKENS}, {hd}]")
-    _need(v_cache.shape == k_cache.shape and v_cache.dtype == k_cache.dtype, f"{what}: value cache differs from key cache")
+    _need(v_cache.shape == (k_cache.shape[0], nkv, hd, PAGE_TOKENS) and v_cache.dtype == k_cache.dtype,
+          f"{what}: value cache {tuple(v_cache.shape)} is not [pages, {nkv}, {hd}, {PAGE_TOKENS}] (values are kept transposed)")
     _need(block_table.dim() == 2, f"{what}: page table {tuple(block_table.shape)} is not [slots, pages]")
 
 
@@ -291,12 +293,114 @@ def linear_library(a: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     return torch.matmul(a, w.t())
 
 
-def linear_thin(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
-    """bfloat16 operands, few rows: the weight is streamed once."""
-    return linear_exact(a, w, out_dtype)
+def thin_serves(a: torch.Tensor, w: torch.Tensor) -> bool:
+    """The matrix-core kernel for thin products takes bfloat16 operands whose rows start on 16 bytes."""
+    return a.dtype == BF16 and w.dtype == BF16 and a.shape[1] % 8 == 0
+
+
+def linear_thin(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, gated: bool = False) -> torch.Tensor:
+    """bfloat16 a [M, K] . w [N, K]^T on the matrix cores, the weight streamed once per 64 rows of a;
+    result [M, N] in bfloat16 or float32.  With ``gated`` w is [gate rows | up rows] and the result is
+    silu(a gate^T) * (a up^T), [M, N/2]."""
+    if not thin_serves(a, w):
+        out = linear_exact(a, w, out_dtype)
+        return swiglu(out) if gated else out
+    _dev("linear_thin", a, w)
+    _need(a.dim() == 2 and w.dim() == 2 and a.shape[1] == w.shape[1],
+          f"linear: a {tuple(a.shape)} and w {tuple(w.shape)} do not share the inner size")
+    M, K = a.shape
+    N = w.shape[0]
+    _need(not gated or N % 2 == 0, f"linear_thin: a gated product needs an even number of weight rows, got {N}")
+    out = torch.empty((M, N // 2 if gated else N), dtype=out_dtype, device=a.device)
+    library.call(core(), "palm_linear_thin", _stream(), _p(a), _p(w), _p(out), _code(out, "linear_thin out"), M, N, K,
+                 1 if gated else 0)
+    return out
+
+
+# ---- attention on the matrix cores (one library for each head size) ---------------------------------
+
+_ATTENTION_SIGNATURES = {
+    "palm_attention_decode": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int,
+                              c_int, c_int, c_float, c_int, c_int, c_void_p, c_void_p],
+    "palm_attention_prefill": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
+                               c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
+}
+_attention_libs: dict = {}
+MFMA_HEAD_DIMS = tuple(range(16, 257, 16))
+DECODE_WAVES_WANTED = 2048        # slices of the key range are made until about this many waves run
+
+
+def attention_lib(hd: int):
+    if hd not in _attention_libs:
+        if hd not in MFMA_HEAD_DIMS:
+            raise KernelError(f"the matrix-core attention kernels take head sizes in steps of 16 up to 256, not {hd}")
+        lib = library.load(f"attention_hd{hd}")
+        for name, argtypes in _ATTENTION_SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.argtypes, fn.restype = argtypes, c_int
+        if lib.palm_attention_head_dim() != hd:
+            raise KernelError(f"library attention_hd{hd} was built for head size {lib.palm_attention_head_dim()}")
+        _attention_libs[hd] = lib
+    return _attention_libs[hd]
+
+
+def mfma_attention_serves(q: torch.Tensor, hd: int) -> bool:
+    return q.dtype == BF16 and hd in MFMA_HEAD_DIMS
+
+
+def decode_slices(n_seqs: int, nh: int, nkv: int, max_keys: int) -> int:
+    """Into how many slices each sequence's key range is cut, so that the launch fills the chip."""
+    waves = n_seqs * nkv * ((nh // nkv + 15) // 16)
+    pages = max(1, (max_keys + PAGE_TOKENS - 1) // PAGE_TOKENS)
+    return max(1, min(pages, (DECODE_WAVES_WANTED + waves - 1) // waves))
+
+
+def _attention_checks(what, q, k_cache, v_cache, block_table, nh, nkv, hd, *index):
+    _dev(what, q, k_cache, v_cache, block_table, *index)
+    _i32(what, block_table, *index)
+    _need(q.dim() == 2 and q.shape[1] == nh * hd and q.dtype == BF16, f"{what}: q {tuple(q.shape)} {q.dtype} is not bfloat16 [n, {nh}*{hd}]")
+    _need(nh % nkv == 0, f"{what}: {nh} heads are not a multiple of {nkv} kv heads")
+    _check_cache(what, k_cache, v_cache, block_table, nkv, hd)
+    _need(k_cache.dtype == BF16, f"{what}: the cache is {k_cache.dtype}, not bfloat16")
+
+
+def attention_decode(q, k_cache, v_cache, block_table, seq_slot, seq_start, nh: int, nkv: int, hd: int, scale: float,
+                     window: int | None, n_slices: int) -> torch.Tensor:
+    """One query for each sequence (row b of q, at position seq_start[b]) over keys 0..seq_start[b]."""
+    _attention_checks("attention_decode", q, k_cache, v_cache, block_table, nh, nkv, hd, seq_slot, seq_start)
+    B = seq_slot.shape[0]
+    _need(q.shape[0] == B and seq_start.shape == (B,), "attention_decode: one query, slot and start for each sequence")
+    out = torch.empty_like(q)
+    work = torch.empty((B * nh * n_slices * (hd + 2),), dtype=F32, device=q.device) if n_slices > 1 else None
+    library.call(attention_lib(hd), "palm_attention_decode", _stream(), _p(q), _p(k_cache), _p(v_cache), _p(block_table),
+                 block_table.shape[1], _p(seq_slot), _p(seq_start), B, nh, nkv, hd, float(scale), int(window or 0),
+                 int(n_slices), _p(work), _p(out))
+    return out
+
+
+def attention_prefill(q, k_cache, v_cache, block_table, seq_slot, seq_start, seq_new, cu_new, max_new: int, nh: int,
+                      nkv: int, hd: int, scale: float, window: int | None) -> torch.Tensor:
+    """The step's queries (several for each sequence) over the cache, on the matrix cores."""
+    _attention_checks("attention_prefill", q, k_cache, v_cache, block_table, nh, nkv, hd, seq_slot, seq_start, seq_new, cu_new)
+    B = seq_slot.shape[0]
+    _need(seq_start.shape == (B,) and seq_new.shape == (B,) and cu_new.shape == (B + 1,),
+          "attention_prefill: per-sequence arrays differ in length")
+    out = torch.empty_like(q)
+    library.call(attention_lib(hd), "palm_attention_prefill", _stream(), _p(q), _p(k_cache), _p(v_cache), _p(block_table),
+                 block_table.shape[1], _p(seq_slot), _p(seq_start), _p(seq_new), _p(cu_new), B, int(max_new), nh, nkv, hd,
+                 float(scale), int(window or 0), _p(out))
+    return out
 
 
 def attention(q, k_cache, v_cache, block_table, ctx, nh: int, nkv: int, hd: int, scale: float, window: int | None):
     """The step's queries over the cache; picks the kernel by element type, head size and step shape."""
+    if mfma_attention_serves(q, hd):
+        if ctx.is_decode:
+            keys = min(ctx.max_total, window) if window else ctx.max_total
+            n_slices = ctx.decode_slices or decode_slices(ctx.n_seqs, nh, nkv, keys)
+            return attention_decode(q, k_cache, v_cache, block_table, ctx.seq_slot, ctx.seq_start, nh, nkv, hd, scale,
+                                    window, n_slices)
+        return attention_prefill(q, k_cache, v_cache, block_table, ctx.seq_slot, ctx.seq_start, ctx.seq_new, ctx.cu_new,
+                                 ctx.max_new, nh, nkv, hd, scale, window)
     return attention_exact(q, k_cache, v_cache, block_table, ctx.seq_slot, ctx.seq_start, ctx.seq_new, ctx.cu_new,
                            ctx.max_new, nh, nkv, hd, scale, window)

@@ -87,6 +87,7 @@ class StepContext:
     seq_new: torch.Tensor        # int32 [B]
     cu_new: torch.Tensor         # int32 [B + 1]
     is_decode: bool = False      # every sequence brings exactly one token
+    decode_slices: int = 0       # if set: into how many slices decode attention cuts a key range (else chosen per call)
     layer_cache: object = None   # the LayerCache of the run-order entry that is running
     memo: dict = field(default_factory=dict)   # what parts make once per step (rotation tables)
     host: dict = field(default_factory=dict)   # the same facts as Python lists, for parts that plan on the host

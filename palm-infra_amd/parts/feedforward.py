@@ -4,7 +4,6 @@ from __future__ import annotations
 
 import torch
 
-from ..kernels import ops
 from .base import register_part
 from .linear import Linear
 
@@ -21,4 +20,4 @@ class GatedSiluFeedForward:
                              f"do not fit hidden {self.hidden}, intermediate {self.inter}")
 
     def forward(self, h: torch.Tensor, ctx) -> torch.Tensor:
-        return self.down(ops.swiglu(self.gate_up(h)))
+        return self.down(self.gate_up.gated(h))

@@ -30,3 +30,10 @@ class Linear:
                 return ops.linear_thin(x, w, out_dtype)
             return ops.linear_library(x, w)
         return ops.linear_exact(x, w, out_dtype)
+
+    def gated(self, x: torch.Tensor) -> torch.Tensor:
+        """silu(x G^T) * (x U^T) for a weight that is [G rows | U rows]: in one kernel when the product is thin,
+        else the product and then the activation."""
+        if x.shape[0] <= THIN_ROWS and ops.thin_serves(x, self.weight):
+            return ops.linear_thin(x, self.weight, x.dtype, gated=True)
+        return ops.swiglu(self(x))

@@ -94,6 +94,7 @@ def test_groups_have_storage_of_their_own():
     assert len(c.kv_groups) == 2 and len(c.state_groups) == 1
     full, win = c.kv_groups
     assert full.k.shape == (2, 13, 2, PAGE_TOKENS, 16) and win.k.shape == (2, 13, 1, PAGE_TOKENS, 32)
+    assert full.v.shape == (2, 13, 2, 16, PAGE_TOKENS)                  # values are kept transposed
     assert full.k.data_ptr() != win.k.data_ptr() and full.table is not win.table
     lc = c.layer_caches
     assert lc[0].kv is full and lc[2].kv is full and (lc[0].kv_entry, lc[2].kv_entry) == (0, 1)

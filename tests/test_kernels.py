@@ -117,7 +117,8 @@ def test_linear_refuses_what_does_not_fit(ops):
 # ---- rotation, q/k norm and the cache write -----------------------------------------------------
 
 def _paged(n_pages, nkv, hd, dtype):
-    return (torch.zeros(n_pages, nkv, 64, hd, dtype=dtype, device=DEV), torch.zeros(n_pages, nkv, 64, hd, dtype=dtype, device=DEV))
+    """Empty key and value caches; values are kept transposed, [pages, nkv, hd, 64]."""
+    return (torch.zeros(n_pages, nkv, 64, hd, dtype=dtype, device=DEV), torch.zeros(n_pages, nkv, hd, 64, dtype=dtype, device=DEV))
 
 
 @pytest.mark.parametrize("theta,half", [(10000.0, 8), (1000000.0, 24), (500000.0, 64)])
@@ -166,12 +167,12 @@ def test_qk_norm_rope_store(ops, dtype, nh, nkv, hd):
     for i in range(n):
         page = int(table[tslot[i], pos[i] // 64])
         assert torch.allclose(kc[page, :, pos[i] % 64], rk[i], atol=t), i
-        assert torch.allclose(vc[page, :, pos[i] % 64], rv[i], atol=1e-12 if dtype == F32 else 0), i   # v is stored as it is
+        assert torch.allclose(vc[page, :, :, pos[i] % 64], rv[i], atol=1e-12 if dtype == F32 else 0), i   # v is stored as it is
     written = {(int(table[tslot[i], pos[i] // 64]), pos[i] % 64) for i in range(n)}
     for page in range(8):
         for r in range(64):
             if (page, r) not in written:
-                assert float(kc[page, :, r].abs().max()) == 0.0 and float(vc[page, :, r].abs().max()) == 0.0
+                assert float(kc[page, :, r].abs().max()) == 0.0 and float(vc[page, :, :, r].abs().max()) == 0.0
 
 
 def test_rotation_variants_interleaved_partial_and_none(ops):
@@ -205,7 +206,7 @@ def _fill_cache(kc, vc, table, slot, k, v):
     for p in range(k.shape[0]):
         page = int(table[slot, p // 64])
         kc[page, :, p % 64] = k[p].to(kc.dtype)
-        vc[page, :, p % 64] = v[p].to(vc.dtype)
+        vc[page, :, :, p % 64] = v[p].to(vc.dtype)
 
 
 def _attention_case(ops, fn, dtype, nh, nkv, hd, lens_new, window, seed=0, scale=None):
@@ -218,7 +219,7 @@ def _attention_case(ops, fn, dtype, nh, nkv, hd, lens_new, window, seed=0, scale
     slots = torch.randperm(B + 4, generator=torch.Generator().manual_seed(seed + 7)).tolist()[:B]      # distinct, not in order
     table = torch.full((B + 4, max_pages), n_pages - 1, dtype=torch.int32)
     kc = rand(n_pages, nkv, 64, hd, seed=seed + 50, dtype=dtype).to(DEV)      # stale values everywhere
-    vc = rand(n_pages, nkv, 64, hd, seed=seed + 51, dtype=dtype).to(DEV)
+    vc = rand(n_pages, nkv, hd, 64, seed=seed + 51, dtype=dtype).to(DEV)
     qs, refs, o = [], [], 0
     for b, (L, new) in enumerate(lens_new):
         npg = (L + 63) // 64

@@ -1,0 +1,152 @@
+"""The matrix-core kernels alone against their plain references: the thin linear product (with and
+without the gated epilogue) and the bfloat16 attention kernels, at sizes other than the tiny models'."""
+import pytest
+import torch
+
+import plain_qwen3 as P
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+F32, BF16 = torch.float32, torch.bfloat16
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from palm_infra_amd.kernels import ops
+    return ops
+
+
+def rand(*shape, seed=0, scale=1.0, dtype=BF16):
+    return (torch.randn(*shape, generator=torch.Generator().manual_seed(seed)) * scale).to(dtype)
+
+
+@pytest.mark.parametrize("M", [1, 8, 16, 17, 33, 64, 70, 150])
+@pytest.mark.parametrize("N,K", [(7, 8), (130, 64), (515, 80), (1000, 224), (96, 4096), (4096, 1536), (300, 12288)])
+def test_linear_thin_against_the_plain_product(ops, M, N, K):
+    a, w = rand(M, K, seed=M + K), rand(N, K, seed=N, scale=0.5)
+    ref = P.linear(a, w)
+    got32 = ops.linear_thin(a.to(DEV), w.to(DEV), F32).cpu()
+    # exact products of bfloat16 values, added in 32-bit: only the order of the sum differs
+    assert torch.allclose(got32.double(), ref, atol=2e-4 * (K ** 0.5), rtol=1e-5), float((got32.double() - ref).abs().max())
+    got16 = ops.linear_thin(a.to(DEV), w.to(DEV), BF16).cpu()
+    assert torch.equal(got16, got32.to(BF16))                          # one rounding at the end
+
+
+def test_linear_thin_orientation(ops):
+    """One weight row and one token stand out: the product must land at [token, feature], not transposed,
+    and every k must be used exactly once."""
+    M, N, K = 5, 40, 256
+    a, w = torch.zeros(M, K, dtype=BF16), torch.zeros(N, K, dtype=BF16)
+    a[3] = torch.arange(K).to(BF16) % 7
+    w[29] = 1.0
+    w[11, 100] = 2.0
+    got = ops.linear_thin(a.to(DEV), w.to(DEV), F32).cpu()
+    ref = torch.zeros(M, N)
+    ref[3, 29] = float((torch.arange(K) % 7).sum())
+    ref[3, 11] = 2.0 * (100 % 7)
+    assert torch.equal(got, ref)
+
+
+@pytest.mark.parametrize("M", [1, 8, 20, 64])
+@pytest.mark.parametrize("I,K", [(5, 16), (176, 80), (224, 96), (1536, 512)])
+def test_linear_thin_gated(ops, M, I, K):
+    a, w = rand(M, K, seed=M), rand(2 * I, K, seed=I, scale=0.3)
+    g, u = P.linear(a, w[:I]), P.linear(a, w[I:])
+    ref = g / (1 + torch.exp(-g)) * u
+    got = ops.linear_thin(a.to(DEV), w.to(DEV), F32, gated=True).cpu()
+    assert got.shape == (M, I)
+    assert torch.allclose(got.double(), ref, atol=1e-3, rtol=1e-4), float((got.double() - ref).abs().max())
+    swapped = u / (1 + torch.exp(-u)) * g
+    assert not torch.allclose(got.double(), swapped, atol=1e-2) or I * M < 8
+    got16 = ops.linear_thin(a.to(DEV), w.to(DEV), BF16, gated=True).cpu()
+    assert torch.equal(got16, got.to(BF16))
+
+
+def test_linear_thin_is_the_same_bits_every_time_and_for_every_companion(ops):
+    a, w = rand(40, 1024, seed=1), rand(200, 1024, seed=2)
+    ad, wd = a.to(DEV), w.to(DEV)
+    first = ops.linear_thin(ad, wd, F32).cpu()
+    for _ in range(3):
+        assert torch.equal(ops.linear_thin(ad, wd, F32).cpu(), first)
+    # a row's result does not depend on which rows are computed with it (within one kernel shape)
+    assert torch.equal(ops.linear_thin(a[32:40].contiguous().to(DEV), wd, F32).cpu(),
+                       ops.linear_thin(a[25:40].contiguous().to(DEV), wd, F32).cpu()[7:])
+
+
+def test_linear_thin_falls_back_when_rows_do_not_start_on_16_bytes(ops):
+    a, w = rand(3, 12, seed=1), rand(9, 12, seed=2)          # K = 12: the exact kernel takes it
+    assert torch.allclose(ops.linear_thin(a.to(DEV), w.to(DEV), F32).cpu().double(), P.linear(a, w), atol=1e-4)
+    a32 = rand(3, 16, seed=1, dtype=F32)
+    assert torch.allclose(ops.linear_thin(a32.to(DEV), rand(9, 16, seed=2, dtype=F32).to(DEV), F32).cpu().double(),
+                          P.linear(a32, rand(9, 16, seed=2, dtype=F32)), atol=1e-4)
+
+
+# ---- attention on the matrix cores ------------------------------------------------------------------
+
+from test_kernels import _attention_case, _spike_case  # noqa: E402  (the cases and the cache filling are shared)
+
+
+def decode_fn(ops, n_slices):
+    def fn(q, kc, vc, table, slots, starts, news, cu, max_new, nh, nkv, hd, scale, window):
+        assert max_new == 1
+        return ops.attention_decode(q, kc, vc, table, slots, starts, nh, nkv, hd, scale, window, n_slices)
+    return fn
+
+
+HEADS = [(8, 4, 16), (5, 5, 48), (6, 1, 80), (4, 2, 128), (32, 8, 128), (40, 2, 32), (3, 3, 256)]
+
+
+@pytest.mark.parametrize("nh,nkv,hd", HEADS)
+def test_attention_prefill_mfma(ops, nh, nkv, hd):
+    # whole prompts, a prompt's continuation (past > 0), single tokens among prompts, tails that fill no tile
+    cases = [[(20, 20)], [(256, 256)], [(1, 1)], [(300, 44)], [(64, 64), (65, 1), (130, 70), (7, 7), (200, 17)]]
+    for lens in cases:
+        got, ref = _attention_case(ops, ops.attention_prefill, BF16, nh, nkv, hd, lens, None, seed=len(lens) + hd)
+        assert torch.allclose(got, ref, atol=2e-2), (lens, float((got - ref).abs().max()))
+
+
+@pytest.mark.parametrize("nh,nkv,hd", HEADS)
+@pytest.mark.parametrize("n_slices", [1, 3, 8])
+def test_attention_decode_mfma(ops, nh, nkv, hd, n_slices):
+    for lens in ([(300, 1)], [(1, 1)], [(64, 1), (65, 1), (700, 1), (7, 1), (128, 1)]):
+        got, ref = _attention_case(ops, decode_fn(ops, n_slices), BF16, nh, nkv, hd, lens, None, seed=len(lens) + hd)
+        assert torch.allclose(got, ref, atol=2e-2), (lens, float((got - ref).abs().max()))
+
+
+@pytest.mark.parametrize("window", [1, 5, 64, 100, 1000])
+def test_attention_mfma_window(ops, window):
+    got, ref = _attention_case(ops, ops.attention_prefill, BF16, 4, 2, 32, [(200, 200), (150, 1), (70, 3), (90, 30)], window, seed=window)
+    assert torch.allclose(got, ref, atol=2e-2), float((got - ref).abs().max())
+    for n_slices in (1, 4):
+        got, ref = _attention_case(ops, decode_fn(ops, n_slices), BF16, 4, 2, 32, [(200, 1), (150, 1), (3, 1)], window, seed=window)
+        assert torch.allclose(got, ref, atol=2e-2), (n_slices, float((got - ref).abs().max()))
+
+
+def test_attention_mfma_finds_a_far_key_and_respects_the_window_edge(ops):
+    for fn in (ops.attention_prefill, decode_fn(ops, 1), decode_fn(ops, 5)):
+        for L, at in ((700, 13), (700, 0), (700, 699), (513, 448), (64, 63), (65, 64), (129, 31)):
+            got, v = _spike_case(ops, fn, BF16, L, at)
+            assert torch.allclose(got, v[at, 0].float().expand(2, -1), atol=1e-2), (L, at)
+        L, w = 300, 70
+        got, v = _spike_case(ops, fn, BF16, L, L - w, window=w)
+        assert torch.allclose(got, v[L - w, 0].float().expand(2, -1), atol=1e-2)
+        got, v = _spike_case(ops, fn, BF16, L, L - w - 1, window=w)
+        assert not torch.allclose(got, v[L - w - 1, 0].float().expand(2, -1), atol=0.2)
+
+
+def test_attention_mfma_agrees_with_the_exact_kernel_on_the_same_cache(ops):
+    """Both read the same cache (keys as rows, values transposed): the layouts cannot drift apart."""
+    got_m, ref = _attention_case(ops, ops.attention_prefill, BF16, 8, 2, 64, [(190, 190), (64, 5)], None, seed=3)
+    got_e, _ = _attention_case(ops, ops.attention_exact, BF16, 8, 2, 64, [(190, 190), (64, 5)], None, seed=3)
+    assert torch.allclose(got_m, got_e, atol=2e-2) and torch.allclose(got_e, ref, atol=2e-2)
+
+
+def test_attention_mfma_refuses_what_it_was_not_built_for(ops):
+    from palm_infra_amd.kernels import KernelError
+    with pytest.raises(KernelError, match="steps of 16"):
+        ops.attention_lib(24)
+    q = torch.zeros(1, 2 * 32, dtype=F32, device=DEV)
+    kc, vc = torch.zeros(2, 1, 64, 32, dtype=F32, device=DEV), torch.zeros(2, 1, 32, 64, dtype=F32, device=DEV)
+    i32 = lambda xs: torch.tensor(xs, dtype=torch.int32).to(DEV)
+    with pytest.raises(KernelError, match="bfloat16"):
+        ops.attention_decode(q, kc, vc, i32([[0, 1]]), i32([0]), i32([3]), 2, 1, 32, 1.0, None, 1)
