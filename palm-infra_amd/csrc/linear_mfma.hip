@@ -6,11 +6,12 @@
 //
 // Work split.  A block owns a strip of 16 weight rows (16 output features) and all of K; its waves take
 // every NW-th "super-step" of 128 k-values and their partial tiles are added in LDS in a fixed order (no
-// atomics: the same input gives the same bits).  In a super-step lane (r, g) of a wave reads 64 contiguous
-// bytes of weight row r (k = k0 + 32 g ..), so a row is read in runs of 256 bytes, and the same k-values of
-// activation row r for each block of 16 tokens; four MFMA 16x16x32 consume them.  Several super-steps are
-// loaded before any is used, which is what keeps enough bytes in flight to fill the memory pipe with only
-// one or two blocks on a compute unit.
+// atomics: the same input gives the same bits).  In a super-step lane (r, g) of a wave makes four 16-byte
+// reads of weight row r, at k = k0 + 32 j + 8 g for j = 0..3, so that each read instruction takes 64
+// contiguous bytes of every row (the four lanes of a row side by side) and the four together a run of 256
+// bytes; it reads the same k-values of activation row r for each block of 16 tokens, and four MFMA 16x16x32
+// consume them.  Several super-steps are loaded before any is used, which is what keeps enough bytes in
+// flight to fill the memory pipe with only one or two blocks on a compute unit.
 #include "mfma.h"
 
 enum ThinEpilogue : int { EPI_STORE = 0, EPI_SWIGLU = 1 };
@@ -36,10 +37,10 @@ __global__ __launch_bounds__(NW * WAVE) void linear_thin_kernel(const bf16_t* __
     } else {
         wrow = min(strip * 16 + r, N - 1);
     }
-    const bf16_t* wp = W + (size_t)wrow * K + g * 32;
+    const bf16_t* wp = W + (size_t)wrow * K + g * 8;
     const bf16_t* xp[MB];
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) xp[mb] = A + (size_t)min(tok0 + mb * 16 + r, M - 1) * K + g * 32;
+    for (int mb = 0; mb < MB; ++mb) xp[mb] = A + (size_t)min(tok0 + mb * 16 + r, M - 1) * K + g * 8;
 
     f32x4 acc[MB];
 #pragma unroll
@@ -54,10 +55,10 @@ __global__ __launch_bounds__(NW * WAVE) void linear_thin_kernel(const bf16_t* __
             const int k0 = (ss + u * NW) * SUPER_K;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const bool ok = k0 + g * 32 + j * 8 < K;            // K is a multiple of 8: a chunk is whole or absent
-                wv[u][j] = ok ? load_bf16x8(wp + k0 + j * 8) : zero_bf16x8();
+                const bool ok = k0 + j * 32 + g * 8 < K;            // K is a multiple of 8: a chunk is whole or absent
+                wv[u][j] = ok ? load_bf16x8(wp + k0 + j * 32) : zero_bf16x8();
 #pragma unroll
-                for (int mb = 0; mb < MB; ++mb) xv[u][mb][j] = ok ? load_bf16x8(xp[mb] + k0 + j * 8) : zero_bf16x8();
+                for (int mb = 0; mb < MB; ++mb) xv[u][mb][j] = ok ? load_bf16x8(xp[mb] + k0 + j * 32) : zero_bf16x8();
             }
         }
 #pragma unroll

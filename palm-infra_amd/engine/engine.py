@@ -149,7 +149,79 @@ class Engine:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
         return torch.stack(rows)
 
+    # ---- decode steps as HIP graphs -----------------------------------------------------------
+    # A decode step is some hundred small kernels; launched one by one the host is the bottleneck.  For a
+    # batch of single tokens the whole forward pass is recorded once into a HIP graph and replayed with
+    # new contents in the same buffers.  A graph is keyed by the batch size, rounded up (rows that pad it
+    # belong to a slot of their own and write into a page that is never read), and by the longest sequence,
+    # rounded up to a power of two (it only sizes how attention cuts the key range).
+    GRAPH_MAX_BATCH = 64
+
+    @staticmethod
+    def _batch_bucket(n: int) -> int:
+        return n if n <= 8 else (n + 7) // 8 * 8
+
+    @staticmethod
+    def _length_bucket(n: int) -> int:
+        b = 256
+        while b < n:
+            b *= 2
+        return b
+
+    def _graph_serves(self, entries) -> bool:
+        return (self.graphs_enabled and self.model.capturable and len(entries) <= self.GRAPH_MAX_BATCH
+                and all(len(e.tokens) == 1 for e in entries))
+
+    def _run_decode_graph(self, entries) -> torch.Tensor:
+        from ..parts import StepContext
+        cache = self.cache
+        growth = [(e.slot, 1) for e in entries]
+        cache.reserve(growth)
+        starts = [cache.lengths[e.slot] for e in entries]
+        B = len(entries)
+        Bb = self._batch_bucket(B)
+        key = (Bb, self._length_bucket(max(starts) + 1))
+        pad = Bb - B
+        slots = [e.slot for e in entries] + [cache.pad_slot] * pad
+        meta = ([int(e.tokens[0]) for e in entries] + [0] * pad + starts + [0] * pad + slots     # ids, positions, slots
+                + starts + [0] * pad + [1] * Bb + list(range(Bb + 1)))                           # starts, counts, offsets
+        state = self._decode_graphs.get(key)
+        if state is None:
+            buf = torch.zeros((len(meta),), dtype=torch.int32, device=self.device)
+            v = [buf[i * Bb:(i + 1) * Bb] for i in range(5)]
+            ctx = StepContext(n_tokens=Bb, n_seqs=Bb, max_new=1, max_total=key[1], dtype=self.dtype, token_ids=v[0],
+                              positions=v[1], tok_slot=v[2], seq_slot=v[2], seq_start=v[3], seq_new=v[4],
+                              cu_new=buf[5 * Bb:], is_decode=True)
+            rows = torch.arange(Bb, dtype=torch.int32).to(self.device)
+            state = self._decode_graphs[key] = {"buf": buf, "ctx": ctx, "rows": rows, "graph": None, "logits": None,
+                                                "calls": 0}
+        state["buf"].copy_(torch.tensor(meta, dtype=torch.int32))
+        ctx = state["ctx"]
+        ctx.host = {"slots": slots, "starts": starts + [0] * pad, "counts": [1] * Bb, "cu": list(range(Bb + 1))}
+        if state["graph"] is None and state["calls"] == 0:
+            # the first step of a shape runs as it is (and loads or builds whatever it needs)
+            ctx.memo = {}
+            logits = self.model.forward(ctx, cache, state["rows"])
+        else:
+            if state["graph"] is None:
+                ctx.memo = {}
+                torch.cuda.synchronize()
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph):
+                    state["logits"] = self.model.forward(ctx, cache, state["rows"])
+                state["graph"] = graph
+            state["graph"].replay()
+            logits = state["logits"].clone()        # the graph's own buffer is overwritten by the next replay
+        state["calls"] += 1
+        cache.commit(growth)
+        wanted = [b for b, e in enumerate(entries) if e.want]
+        if len(wanted) == B:
+            return logits[:B]
+        return logits[torch.tensor(wanted, dtype=torch.long, device=self.device)] if wanted else logits[:0]
+
     def _run(self, entries) -> torch.Tensor:
+        if self._graph_serves(entries):
+            return self._run_decode_graph(entries)
         cache = self.cache
         growth = [(e.slot, len(e.tokens)) for e in entries]
         cache.reserve(growth)

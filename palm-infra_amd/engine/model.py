@@ -23,6 +23,13 @@ class DecoderModel:
         self.order = spec.order
         self.weights = weights
 
+    @property
+    def capturable(self) -> bool:
+        """Whether a decode step of this model may be recorded into a HIP graph: every part says of itself
+        that it launches the same kernels whatever the step holds (a part that plans on the host does not)."""
+        parts = [self.embedding, *self.layers, self.final_norm, self.head]
+        return all(getattr(p, "capturable", False) for p in parts)
+
     def cache_plan(self):
         """For each entry of the run order: what it keeps per sequence, and whose cache it reads."""
         needs, shares = [], []

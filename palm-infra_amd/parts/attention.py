@@ -20,6 +20,8 @@ from .position import PAIRINGS
 
 @register_part("mixer", "attention")
 class Attention:
+    capturable = True
+
     def __init__(self, spec, builder):
         p = spec.params
         self.hidden = int(p["hidden_size"])

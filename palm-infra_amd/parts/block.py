@@ -17,6 +17,11 @@ class PreNormBlock:
         self.feed_forward_norm = builder.build(spec.parts["feed_forward_norm"])
         self.feed_forward = builder.build(spec.parts["feed_forward"])
 
+    @property
+    def capturable(self) -> bool:
+        return all(getattr(p, "capturable", False) for p in (self.mixer_norm, self.mixer, self.feed_forward_norm,
+                                                              self.feed_forward))
+
     @staticmethod
     def cache_needs(spec):
         return cache_needs(spec.parts["mixer"])

@@ -10,6 +10,8 @@ from .linear import Linear
 
 @register_part("embedding", "token_table")
 class TokenEmbedding:
+    capturable = True
+
     """x[t, :] = E[id_t, :] widened to float32 (engine/engine.cpp:332-357).  Unlike the reference, an id
     outside the table is not mapped to row 0: the step refuses it before anything runs."""
 
@@ -25,6 +27,8 @@ class TokenEmbedding:
 
 @register_part("head", "linear")
 class LinearHead:
+    capturable = True
+
     """logits = h W^T in float32; W is lm_head.weight, or the embedding table when the head is tied
     (models/qwen3.py:89-95, 162-165; engine/engine.cpp:403-485)."""
 

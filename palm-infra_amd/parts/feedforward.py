@@ -10,6 +10,8 @@ from .linear import Linear
 
 @register_part("feed_forward", "gated_silu")
 class GatedSiluFeedForward:
+    capturable = True
+
     def __init__(self, spec, builder):
         self.hidden = int(spec.params["hidden_size"])
         self.inter = int(spec.params["intermediate_size"])

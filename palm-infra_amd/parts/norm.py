@@ -11,6 +11,8 @@ from .base import register_part
 
 @register_part("norm", "rms")
 class RMSNorm:
+    capturable = True      # launches the same kernels whatever the step holds: may be recorded into a HIP graph
+
     def __init__(self, spec, builder):
         self.width = int(spec.params["width"])
         self.eps = float(spec.params["eps"])

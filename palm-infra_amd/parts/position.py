@@ -22,6 +22,8 @@ PAIRINGS = {"half_split": 0, "interleaved": 1}
 
 @register_part("position", "rotary")
 class Rotary:
+    capturable = True
+
     def __init__(self, spec, builder):
         self.rotary_dim = int(spec.params["rotary_dim"])
         self.theta = float(spec.params["theta"])
@@ -44,6 +46,7 @@ class Rotary:
 
 @register_part("position", "none")
 class NoPosition:
+    capturable = True
     rotary_dim, pairing = 0, "half_split"
 
     def __init__(self, spec, builder):

@@ -1,0 +1,80 @@
+"""Decode steps replayed from HIP graphs give what the same steps give when launched one by one: over many
+replays, with other work and synchronisations between them, with batches that shrink and are padded, and
+with slots and pages used again."""
+import pytest
+import torch
+
+import tiny
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("name,dtype", [("A", "float32"), ("B", "bfloat16"), ("C", "bfloat16")])
+def test_replays_equal_plain_launches(model_dirs, name, dtype):
+    from palm_infra_amd.engine import Engine, StepEntry
+    g = Engine.from_dir(model_dirs[name][dtype], dtype=dtype, max_tokens=64 * 40, graphs=True)
+    e = Engine.from_dir(model_dirs[name][dtype], dtype=dtype, max_tokens=64 * 40, graphs=False)
+    assert g.model.capturable
+    n_req = 11
+    reqs = tiny.prompts(name, [3 + 7 * i for i in range(n_req)], seed=30)
+    decoded = tiny.prompts(name, [60] * n_req, seed=31)
+    for round_no in range(2):                                   # the second round reuses slots, pages and graphs
+        sg = [g.open() for _ in reqs]
+        se = [e.open() for _ in reqs]
+        a = g.step([StepEntry(s, r, [len(r) - 1]) for s, r in zip(sg, reqs)])
+        b = e.step([StepEntry(s, r, [len(r) - 1]) for s, r in zip(se, reqs)])
+        assert torch.equal(a, b)                                # prompts never go through a graph
+        live = list(range(n_req))
+        for t in range(50):
+            if t in (5, 9, 20, 21, 33, 40):                     # sequences end: 11 -> 10 -> 9 (a padded 16) -> .. -> 5
+                gone = live.pop(t % len(live))
+                g.close(sg[gone]); e.close(se[gone])
+            a = g.step([StepEntry(sg[i], [decoded[i][t]], [0]) for i in live])
+            b = e.step([StepEntry(se[i], [decoded[i][t]], [0]) for i in live])
+            if t % 7 == 3:                                      # other work and a synchronisation between replays
+                torch.cuda.synchronize()
+                extra = g.open()
+                g.step([StepEntry(extra, reqs[2], [0])])
+                g.close(extra)
+            if dtype == "float32":
+                assert torch.equal(a, b), (round_no, t)         # padding and recording change no bit
+            else:
+                # the recorded step cuts a key range into slices sized for a rounded-up length: another order of sums
+                tiny.assert_logits_close(a, b.double().cpu(), dtype, f"{name} round {round_no} step {t}")
+                assert float((a - b).abs().max()) < 0.05 * float(b.abs().max())
+        for i in live:
+            g.close(sg[i]); e.close(se[i])
+        g.cache.check(); e.cache.check()
+    keys = sorted(g._decode_graphs)
+    assert len(keys) >= 4 and all(st["graph"] is not None for k, st in g._decode_graphs.items() if st["calls"] > 1)
+    assert not e._decode_graphs
+
+
+def test_a_wanted_subset_and_an_empty_one(model_dirs):
+    from palm_infra_amd.engine import Engine, StepEntry
+    g = Engine.from_dir(model_dirs["A"]["bfloat16"], dtype="bfloat16", max_tokens=64 * 8)
+    reqs = tiny.prompts("A", [5, 6, 7], seed=32)
+    slots = [g.open() for _ in reqs]
+    g.step([StepEntry(s, r, []) for s, r in zip(slots, reqs)])
+    for t in range(4):
+        full = g.step([StepEntry(s, [t + 1], [0]) for s in slots])
+        assert full.shape == (3, 256)
+    some = g.step([StepEntry(slots[0], [9], []), StepEntry(slots[1], [9], [0]), StepEntry(slots[2], [9], [])])
+    none = g.step([StepEntry(s, [3], []) for s in slots])
+    assert some.shape == (1, 256) and none.shape == (0, 256)
+    assert [g.length(s) for s in slots] == [11, 12, 13]
+
+
+def test_a_model_with_a_part_that_plans_on_the_host_is_not_recorded(model_dirs):
+    import test_toy_parts as toy
+    from palm_infra_amd.config import config_from_dir
+    from palm_infra_amd.engine import Engine
+    from palm_infra_amd.weights import ModelFiles, load_weights
+    toy.register_toy_mixer()
+    d = model_dirs["A"]["float32"]
+    config, files = config_from_dir(d), ModelFiles(d)
+    base = config.spec(files.names())
+    w = toy.ExtraWeights(load_weights(base, files, torch.float32, "cuda:0"),
+                         {("toy.w_in",): torch.zeros(24, 64, device="cuda:0"), ("toy.w_out",): torch.zeros(64, 24, device="cuda:0")})
+    eng = Engine(config, toy.toy_spec(base), w, torch.float32, max_tokens=256)
+    assert not eng.model.capturable
