@@ -44,23 +44,48 @@ struct Columns {          // softmax state of this lane's query column, and its 
 // The key that row r of S^T tile `t` (0..3) of a page stands for: tiles 2h and 2h+1 cover keys 32h..32h+31.
 __device__ inline int tile_key(int t, int r) { return (t / 2) * 32 + (r / 4) * 8 + (t % 2) * 4 + (r % 4); }
 
-// One page: scores of its 64 keys against the columns' queries, online softmax, and the weighted values.
-// kp: K of this page and kv head [64, HD]; vp: V^T [HD, 64].  Keys outside [lo, hi] (in-page indices) are
-// masked.  qv: the B operand of the first product (this lane's query, chunks g, g+4, ..).
-__device__ inline void attend_page(const bf16_t* __restrict__ kp, const bf16_t* __restrict__ vp,
-                                   const bf16x8 (&qv)[KSTEPS], int lo, int hi, float scale_log2, Columns& c,
-                                   int r, int g) {
-    f32x4 s[4];
+// The operands of one page, read ahead of their use: K fragments for the first product, V^T fragments for
+// the second.  Every read is unconditional (an absent chunk reads chunk 0 and is zeroed by a select), so the
+// compiler can issue them all before the first wait; a read behind a branch would be waited for one by one.
+struct PageOperands {
+    bf16x8 k[4][KSTEPS];
+    bf16x8 v[DTILES][2];
+};
+
+__device__ inline void load_keys(const bf16_t* __restrict__ kp, int r, int g, PageOperands& ops) {
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
         const bf16_t* krow = kp + (size_t)tile_key(t, r) * HD;
-        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int j = 0; j < KSTEPS; ++j) {
             const int chunk = j * 4 + g;
-            const bf16x8 kv = chunk < CHUNKS ? load_bf16x8(krow + chunk * 8) : zero_bf16x8();
-            acc = mfma_16x16x32(kv, qv[j], acc);
+            const bool ok = (CHUNKS % 4 == 0) || chunk < CHUNKS;
+            const bf16x8 v = load_bf16x8(krow + (ok ? chunk : 0) * 8);
+            ops.k[t][j] = ok ? v : zero_bf16x8();
         }
+    }
+}
+
+__device__ inline void load_values(const bf16_t* __restrict__ vp, int r, int g, PageOperands& ops) {
+#pragma unroll
+    for (int dt = 0; dt < DTILES; ++dt) {
+        const bf16_t* vrow = vp + (size_t)(dt * 16 + r) * PAGE_TOKENS;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) ops.v[dt][h] = load_bf16x8(vrow + h * 32 + g * 8);
+    }
+}
+
+// Scores of a page's 64 keys against the columns' queries and the online softmax; leaves the page's
+// weights as the B operands of the second product.  Keys outside [lo, hi] (in-page indices) are masked.
+// qv: the B operand of the first product (this lane's query, chunks g, g+4, ..).
+__device__ inline float score_page(const PageOperands& ops, const bf16x8 (&qv)[KSTEPS], int lo, int hi,
+                                   float scale_log2, Columns& c, int g, bf16x8 (&pv)[2]) {
+    f32x4 s[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < KSTEPS; ++j) acc = mfma_16x16x32(ops.k[t][j], qv[j], acc);
         s[t] = acc;
     }
     // this lane holds, for its query, keys tile_key(t, 4g + i)
@@ -83,7 +108,6 @@ __device__ inline void attend_page(const bf16_t* __restrict__ kp, const bf16_t* 
     const float m_sub = m_new == -INFINITY ? 0.f : m_new;
     const float alpha = exp2f(c.m - m_sub);             // c.m = -inf before the first visible key: 0
     float sum = 0.f;
-    bf16x8 pv[2];
 #pragma unroll
     for (int h = 0; h < 2; ++h)
 #pragma unroll
@@ -94,13 +118,40 @@ __device__ inline void attend_page(const bf16_t* __restrict__ kp, const bf16_t* 
         }
     c.l = c.l * alpha + sum;                            // this lane's share; the groups are added at the end
     c.m = m_new;
+    return alpha;
+}
+
+__device__ inline void weigh_values(const PageOperands& ops, const bf16x8 (&pv)[2], float alpha, Columns& c) {
 #pragma unroll
     for (int dt = 0; dt < DTILES; ++dt) {
         f32x4 acc = c.o[dt] * alpha;
-        const bf16_t* vrow = vp + (size_t)(dt * 16 + r) * PAGE_TOKENS;
 #pragma unroll
-        for (int h = 0; h < 2; ++h) acc = mfma_16x16x32(load_bf16x8(vrow + h * 32 + g * 8), pv[h], acc);
+        for (int h = 0; h < 2; ++h) acc = mfma_16x16x32(ops.v[dt][h], pv[h], acc);
         c.o[dt] = acc;
+    }
+}
+
+// All pages p0 <= p < p1 of one sequence and kv head.  The reads of the next page are issued as soon as the
+// registers of the current one are free: K after the scores, V after the weighted sum, so that a page's
+// latency hides behind the previous page's arithmetic.  first/pos: the column's own key range.
+__device__ inline void attend_pages(const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+                                    const int* __restrict__ pages, int nkv, int kvh, int p0, int p1,
+                                    const bf16x8 (&qv)[KSTEPS], int first, int pos, float scale_log2, Columns& c,
+                                    int r, int g) {
+    if (p0 >= p1) return;
+    PageOperands ops;
+    size_t base = ((size_t)pages[p0] * nkv + kvh) * PAGE_TOKENS * HD;
+    load_keys(k_cache + base, r, g, ops);
+    load_values(v_cache + base, r, g, ops);
+    for (int p = p0; p < p1; ++p) {
+        const bool more = p + 1 < p1;
+        const size_t next = more ? ((size_t)pages[p + 1] * nkv + kvh) * PAGE_TOKENS * HD : base;
+        bf16x8 pv[2];
+        const float alpha = score_page(ops, qv, first - p * PAGE_TOKENS, pos - p * PAGE_TOKENS, scale_log2, c, g, pv);
+        if (more) load_keys(k_cache + next, r, g, ops);
+        weigh_values(ops, pv, alpha, c);
+        if (more) load_values(v_cache + next, r, g, ops);
+        base = next;
     }
 }
 
@@ -108,7 +159,9 @@ __device__ inline void load_query(const bf16_t* qrow, bool valid, int g, bf16x8 
 #pragma unroll
     for (int j = 0; j < KSTEPS; ++j) {
         const int chunk = j * 4 + g;
-        qv[j] = (valid && chunk < CHUNKS) ? load_bf16x8(qrow + chunk * 8) : zero_bf16x8();
+        const bool ok = valid && ((CHUNKS % 4 == 0) || chunk < CHUNKS);
+        const bf16x8 v = load_bf16x8(qrow + (chunk < CHUNKS ? chunk : 0) * 8);     // qrow is always a real row
+        qv[j] = ok ? v : zero_bf16x8();
     }
 }
 
@@ -141,10 +194,7 @@ __global__ __launch_bounds__(WAVE) void attention_decode_kernel(
     for (int dt = 0; dt < DTILES; ++dt) c.o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     const int* pages = block_table + (size_t)seq_slot[b] * max_pages;
-    for (int p = p0; p < p1; ++p) {
-        const size_t base = ((size_t)pages[p] * nkv + kvh) * PAGE_TOKENS * HD;
-        attend_page(k_cache + base, v_cache + base, qv, first - p * PAGE_TOKENS, pos - p * PAGE_TOKENS, scale_log2, c, r, g);
-    }
+    attend_pages(k_cache, v_cache, pages, nkv, kvh, p0, p1, qv, first, pos, scale_log2, c, r, g);
     float l = c.l;
     l += __shfl_xor(l, 16, WAVE);
     l += __shfl_xor(l, 32, WAVE);
@@ -166,17 +216,46 @@ __global__ __launch_bounds__(WAVE) void attention_decode_kernel(
         for (int i = 0; i < 4; ++i) w[2 + dt * 16 + 4 * g + i] = c.o[dt][i];
 }
 
-// one block per (sequence, head): merge the slices in a fixed order
-__global__ void attention_merge_kernel(const float* __restrict__ work, int n_slices, bf16_t* __restrict__ out) {
+// One wave per (sequence, head): merge the slices in a fixed order.  Lane s first reads slice s's maximum
+// and sum (all at once), the wave agrees on the overall maximum and on each slice's weight, then lane d sums
+// output element d over the slices, eight reads in flight at a time.
+__global__ __launch_bounds__(WAVE) void attention_merge_kernel(const float* __restrict__ work, int n_slices,
+                                                               bf16_t* __restrict__ out) {
     const float* w = work + (size_t)blockIdx.x * n_slices * (HD + 2);
+    const int lane = threadIdx.x;
     float m = -INFINITY;
-    for (int s = 0; s < n_slices; ++s) m = fmaxf(m, w[s * (HD + 2)]);
+    for (int s = lane; s < n_slices; s += WAVE) m = fmaxf(m, w[(size_t)s * (HD + 2)]);
+    m = wave_max(m);
     float l = 0.f;
-    for (int s = 0; s < n_slices; ++s) l += w[s * (HD + 2) + 1] * exp2f(w[s * (HD + 2)] - m);
-    for (int d = threadIdx.x; d < HD; d += blockDim.x) {
-        float o = 0.f;
-        for (int s = 0; s < n_slices; ++s) o += w[s * (HD + 2) + 2 + d] * exp2f(w[s * (HD + 2)] - m);
-        out[(size_t)blockIdx.x * HD + d] = f32_to_bf16(o / l);
+    for (int s = lane; s < n_slices; s += WAVE) l += w[(size_t)s * (HD + 2) + 1] * exp2f(w[(size_t)s * (HD + 2)] - m);
+    l = wave_sum(l);
+    constexpr int PER = (HD + WAVE - 1) / WAVE;
+    float o[PER];
+#pragma unroll
+    for (int i = 0; i < PER; ++i) o[i] = 0.f;
+    for (int s0 = 0; s0 < n_slices; s0 += 8) {
+        float ms[8], v[8][PER];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int s = min(s0 + u, n_slices - 1);
+            ms[u] = w[(size_t)s * (HD + 2)];
+#pragma unroll
+            for (int i = 0; i < PER; ++i) {
+                const int d = min(lane + i * WAVE, HD - 1);
+                v[u][i] = w[(size_t)s * (HD + 2) + 2 + d];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const float wt = s0 + u < n_slices ? exp2f(ms[u] - m) : 0.f;
+#pragma unroll
+            for (int i = 0; i < PER; ++i) o[i] += v[u][i] * wt;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        const int d = lane + i * WAVE;
+        if (d < HD) out[(size_t)blockIdx.x * HD + d] = f32_to_bf16(o[i] / l);
     }
 }
 
@@ -202,7 +281,7 @@ PALM_API int palm_attention_decode(hipStream_t stream, const void* q, const void
                                                       window, n_slices, work, (bf16_t*)out);
     PALM_LAUNCHED();
     if (n_slices > 1) {
-        attention_merge_kernel<<<n_seqs * nh, HD <= 64 ? 64 : 128, 0, stream>>>(work, n_slices, (bf16_t*)out);
+        attention_merge_kernel<<<n_seqs * nh, WAVE, 0, stream>>>(work, n_slices, (bf16_t*)out);
         PALM_LAUNCHED();
     }
     return 0;
@@ -241,12 +320,9 @@ __global__ __launch_bounds__(4 * WAVE) void attention_prefill_kernel(
         c.l = 0.f;
 #pragma unroll
         for (int dt = 0; dt < DTILES; ++dt) c.o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
-        for (int p = tile_first / PAGE_TOKENS; p <= tile_last / PAGE_TOKENS; ++p) {
-            const size_t base = ((size_t)pages[p] * nkv + kvh) * PAGE_TOKENS * HD;
-            // a column whose own range misses this page entirely still needs a finite maximum: its scores are
-            // all -inf then and the page adds nothing, which the guard below keeps free of NaN
-            attend_page(k_cache + base, v_cache + base, qv, my_first - p * PAGE_TOKENS, pos - p * PAGE_TOKENS, scale_log2, c, r, g);
-        }
+        // a column whose own range misses a page of the tile entirely adds nothing there (see score_page)
+        attend_pages(k_cache, v_cache, pages, nkv, kvh, tile_first / PAGE_TOKENS, tile_last / PAGE_TOKENS + 1, qv, my_first,
+                     pos, scale_log2, c, r, g);
         float l = c.l;
         l += __shfl_xor(l, 16, WAVE);
         l += __shfl_xor(l, 32, WAVE);

@@ -66,6 +66,85 @@ __global__ void rmsnorm_kernel(TX* __restrict__ x, const TD* __restrict__ delta,
     }
 }
 
+// The same, for widths that are a multiple of four and fit the block's registers: every thread reads its
+// elements once, four at a time, all reads issued before the first is used (a decode step's rows are few and
+// the kernel's time is the latency of its reads, so reads that wait for each other are what must be avoided).
+__device__ inline void load4(const float* p, float (&v)[4]) {
+    const float4 t = *reinterpret_cast<const float4*>(p);
+    v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+}
+__device__ inline void load4(const bf16_t* p, float (&v)[4]) {
+    const uint2 t = *reinterpret_cast<const uint2*>(p);
+    v[0] = __uint_as_float(t.x << 16); v[1] = __uint_as_float(t.x & 0xffff0000u);
+    v[2] = __uint_as_float(t.y << 16); v[3] = __uint_as_float(t.y & 0xffff0000u);
+}
+__device__ inline void store4(float* p, const float (&v)[4]) { *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]); }
+__device__ inline void store4(bf16_t* p, const float (&v)[4]) {
+    uint2 t;
+    t.x = (uint32_t)f32_to_bf16(v[0]).bits | ((uint32_t)f32_to_bf16(v[1]).bits << 16);
+    t.y = (uint32_t)f32_to_bf16(v[2]).bits | ((uint32_t)f32_to_bf16(v[3]).bits << 16);
+    *reinterpret_cast<uint2*>(p) = t;
+}
+
+template <typename TX, typename TD, typename TO, int ITERS>
+__global__ void rmsnorm_fast_kernel(TX* __restrict__ x, const TD* __restrict__ delta, const float* __restrict__ w,
+                                    const int* __restrict__ rows, TO* __restrict__ out, int width, float eps,
+                                    int update_x) {
+    __shared__ float scratch[16];
+    const int r = blockIdx.x;
+    const size_t src = rows ? (size_t)rows[r] : (size_t)r;
+    TX* xr = x + src * width;
+    const TD* dr = delta ? delta + src * width : nullptr;
+    float v[ITERS][4], d[ITERS][4], wt[ITERS][4];
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+        const int i = (it * blockDim.x + threadIdx.x) * 4;
+        const int at = i < width ? i : 0;                   // a thread beyond the row reads its start and adds nothing
+        load4(xr + at, v[it]);
+        load4(w + at, wt[it]);
+        if (dr) load4(dr + at, d[it]);
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+        const bool in = (it * blockDim.x + threadIdx.x) * 4 < width;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            if (dr) v[it][e] += d[it][e];
+            if (in) ss += v[it][e] * v[it][e];
+        }
+    }
+    ss = block_sum(ss, scratch);
+    const float inv = 1.0f / sqrtf(ss / (float)width + eps);
+    TO* o = out + (size_t)r * width;
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+        const int i = (it * blockDim.x + threadIdx.x) * 4;
+        if (i >= width) continue;
+        if (update_x) store4(xr + i, v[it]);
+        float y[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) y[e] = v[it][e] * inv * wt[it][e];
+        store4(o + i, y);
+    }
+}
+
+template <typename TX, typename TD, typename TO>
+static bool launch_rmsnorm_fast(hipStream_t stream, void* x, const void* delta, const float* weight, float eps,
+                                const int* rows, int n_out_rows, int width, void* out, int update_x) {
+    if (width % 4 != 0 || width > 32768) return false;
+    const int quads = width / 4;
+    const int iters = quads <= 256 ? 1 : (quads <= 512 ? 2 : (quads <= 1024 ? 4 : 8));
+    int threads = (quads + iters - 1) / iters;
+    threads = (threads + WAVE - 1) / WAVE * WAVE;
+    if (threads > 1024) return false;
+#define PALM_NORM_CASE(IT) case IT: rmsnorm_fast_kernel<TX, TD, TO, IT><<<n_out_rows, threads, 0, stream>>>( \
+        (TX*)x, (const TD*)delta, weight, rows, (TO*)out, width, eps, update_x); break;
+    switch (iters) { PALM_NORM_CASE(1) PALM_NORM_CASE(2) PALM_NORM_CASE(4) PALM_NORM_CASE(8) }
+#undef PALM_NORM_CASE
+    return true;
+}
+
 PALM_API int palm_rmsnorm(hipStream_t stream, void* x, int x_dtype, const void* delta, int delta_dtype,
                           const float* weight, float eps, const int* rows, int n_out_rows, int width,
                           void* out, int out_dtype, int update_x) {
@@ -73,6 +152,12 @@ PALM_API int palm_rmsnorm(hipStream_t stream, void* x, int x_dtype, const void* 
     PALM_CHECK(!(update_x && rows), "rmsnorm: the residual cannot be updated through a row selection");
     PALM_CHECK(!(update_x && !delta), "rmsnorm: update_x without a delta has nothing to add");
     if (n_out_rows == 0) return 0;
+    {
+        bool done = false;
+        PALM_DTYPE_SWITCH(x_dtype, TX, PALM_DTYPE_SWITCH(delta_dtype, TD, PALM_DTYPE_SWITCH(out_dtype, TO,
+            done = launch_rmsnorm_fast<TX, TD, TO>(stream, x, delta, weight, eps, rows, n_out_rows, width, out, update_x))));
+        if (done) { PALM_LAUNCHED(); return 0; }
+    }
     const int threads = width >= 1024 ? 256 : (width >= 256 ? 128 : 64);
     PALM_DTYPE_SWITCH(x_dtype, TX, PALM_DTYPE_SWITCH(delta_dtype, TD, PALM_DTYPE_SWITCH(out_dtype, TO,
         rmsnorm_kernel<TX, TD, TO><<<n_out_rows, threads, 0, stream>>>(

@@ -327,7 +327,7 @@ _ATTENTION_SIGNATURES = {
 }
 _attention_libs: dict = {}
 MFMA_HEAD_DIMS = tuple(range(16, 257, 16))
-DECODE_WAVES_WANTED = 2048        # slices of the key range are made until about this many waves run
+DECODE_WAVES_WANTED = 768         # slices of the key range are made until about this many waves run (measured best)
 
 
 def attention_lib(hd: int):
