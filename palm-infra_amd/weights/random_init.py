@@ -54,3 +54,23 @@ def write_random_model(config, seed: int, out_dir, dtype: str = "bfloat16") -> P
     write_safetensors(out_dir / "model.safetensors", random_tensors(config.spec(), seed, dtype),
                       metadata={"format": "pt", "seed": seed})
     return out_dir
+
+
+def main(argv=None) -> int:
+    """``python -m palm_infra_amd.weights.random_init --config config.json --seed 0 --out DIR``"""
+    import argparse
+    ap = argparse.ArgumentParser(prog="palm_random_model",
+                                 description="Write a model folder (config.json, model.safetensors) with random weights.")
+    ap.add_argument("--config", required=True, help="a config.json of a registered architecture")
+    ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--out", required=True, help="folder to write")
+    ap.add_argument("--dtype", default="bfloat16", choices=sorted(_STORE), help="how the tensors are stored")
+    args = ap.parse_args(argv)
+    raw = json.loads(Path(args.config).read_text())
+    out = write_random_model(raw, args.seed, args.out, args.dtype)
+    print(out)
+    return 0
+
+
+if __name__ == "__main__":
+    raise SystemExit(main())
