@@ -288,51 +288,217 @@ PALM_API int palm_attention_decode(hipStream_t stream, const void* q, const void
 }
 
 // ---- prefill --------------------------------------------------------------------------------------
-// grid (query tiles of 16 positions, nkv, sequences); four waves; wave w takes query heads w, w + 4, ..
-// of the kv head's group, so the waves of a block read the same pages of K and V.
-__global__ __launch_bounds__(4 * WAVE) void attention_prefill_kernel(
+// A block of four waves serves one kv head, up to eight query heads of its group (more heads: more blocks)
+// and a tile of QB query positions, QB = 16 * max(1, 8 / heads): at most eight "units" of 16 columns
+// (head, 16 positions), two for each wave.  A page of K and of V^T is read from memory once for the block,
+// into LDS; every wave takes its MFMA operands from there, each operand serving both of its units.  The next
+// page is on its way into registers while the current one is being used.  Tiles late in a sequence see more
+// keys, so they are started first.
+constexpr int PF_WAVES = 4;
+constexpr int PF_THREADS = PF_WAVES * WAVE;
+constexpr int PF_UNITS = 2;                                // units of 16 columns held by a wave
+constexpr int K_STRIDE = HD + 8;                           // padded rows: fragment reads of 16 rows spread over banks
+constexpr int V_STRIDE = PAGE_TOKENS + 8;
+constexpr int PAGE_CHUNKS = PAGE_TOKENS * HD / 8;          // 16-byte chunks in a page of K (and of V^T)
+constexpr int PF_LOADS = (PAGE_CHUNKS + PF_THREADS - 1) / PF_THREADS;
+constexpr bool PF_SHARE = (PAGE_TOKENS * K_STRIDE + HD * V_STRIDE) * 2 > 60 * 1024;   // too big for 64 KB: V reuses K's space
+
+struct PagePrefetch { bf16x8 k[PF_LOADS], v[PF_LOADS]; };
+
+__device__ inline void prefetch_keys(const bf16_t* __restrict__ kp, PagePrefetch& pf) {
+#pragma unroll
+    for (int i = 0; i < PF_LOADS; ++i) {
+        const int c = i * PF_THREADS + threadIdx.x;
+        pf.k[i] = load_bf16x8(kp + (size_t)(c < PAGE_CHUNKS ? c : 0) * 8);
+    }
+}
+__device__ inline void prefetch_values(const bf16_t* __restrict__ vp, PagePrefetch& pf) {
+#pragma unroll
+    for (int i = 0; i < PF_LOADS; ++i) {
+        const int c = i * PF_THREADS + threadIdx.x;
+        pf.v[i] = load_bf16x8(vp + (size_t)(c < PAGE_CHUNKS ? c : 0) * 8);
+    }
+}
+__device__ inline void stage_keys(const PagePrefetch& pf, bf16_t* k_lds) {
+#pragma unroll
+    for (int i = 0; i < PF_LOADS; ++i) {
+        const int c = i * PF_THREADS + threadIdx.x;
+        if (c < PAGE_CHUNKS) *reinterpret_cast<bf16x8*>(k_lds + (c / CHUNKS) * K_STRIDE + (c % CHUNKS) * 8) = pf.k[i];
+    }
+}
+__device__ inline void stage_values(const PagePrefetch& pf, bf16_t* v_lds) {
+#pragma unroll
+    for (int i = 0; i < PF_LOADS; ++i) {
+        const int c = i * PF_THREADS + threadIdx.x;
+        if (c < PAGE_CHUNKS) *reinterpret_cast<bf16x8*>(v_lds + (c / 8) * V_STRIDE + (c % 8) * 8) = pf.v[i];
+    }
+}
+
+struct Unit {                 // one (head, 16 query positions): the wave's share of it
+    bool live;                // false: the wave has no such unit (fewer units than slots)
+    bool valid;               // this lane's column is a real query
+    int pos, first;           // the column's position and the first key it sees
+    size_t row;               // the column's row in q and out
+    int head;
+    bf16x8 qv[KSTEPS];
+    Columns c;
+};
+
+__device__ inline void unit_scores(const bf16_t* k_lds, Unit (&u)[PF_UNITS], int page_first_key, float scale_log2,
+                                   int r, int g, bf16x8 (&pv)[PF_UNITS][2], float (&alpha)[PF_UNITS]) {
+    f32x4 s[PF_UNITS][4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        const bf16_t* krow = k_lds + tile_key(t, r) * K_STRIDE;
+#pragma unroll
+        for (int x = 0; x < PF_UNITS; ++x) s[x][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < KSTEPS; ++j) {
+            const int chunk = j * 4 + g;
+            const bool ok = (CHUNKS % 4 == 0) || chunk < CHUNKS;
+            bf16x8 kf = *reinterpret_cast<const bf16x8*>(krow + (ok ? chunk : 0) * 8);
+            if (!ok) kf = zero_bf16x8();
+#pragma unroll
+            for (int x = 0; x < PF_UNITS; ++x) s[x][t] = mfma_16x16x32(kf, u[x].qv[j], s[x][t]);
+        }
+    }
+#pragma unroll
+    for (int x = 0; x < PF_UNITS; ++x) {
+        Columns& c = u[x].c;
+        const int lo = u[x].first - page_first_key, hi = u[x].pos - page_first_key;
+        float mx = -INFINITY;
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int key = tile_key(t, 4 * g + i);
+                const float v = (key >= lo && key <= hi) ? s[x][t][i] * scale_log2 : -INFINITY;
+                s[x][t][i] = v;
+                mx = fmaxf(mx, v);
+            }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+        const float m_new = fmaxf(c.m, mx);
+        const float m_sub = m_new == -INFINITY ? 0.f : m_new;       // see score_page
+        alpha[x] = exp2f(c.m - m_sub);
+        float sum = 0.f;
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float p = exp2f(s[x][2 * h + e / 4][e % 4] - m_sub);
+                sum += p;
+                pv[x][h][e] = (__bf16)p;
+            }
+        c.l = c.l * alpha[x] + sum;
+        c.m = m_new;
+    }
+}
+
+__device__ inline void unit_values(const bf16_t* v_lds, Unit (&u)[PF_UNITS], int r, int g,
+                                   const bf16x8 (&pv)[PF_UNITS][2], const float (&alpha)[PF_UNITS]) {
+#pragma unroll
+    for (int dt = 0; dt < DTILES; ++dt) {
+        const bf16_t* vrow = v_lds + (dt * 16 + r) * V_STRIDE;
+        f32x4 acc[PF_UNITS];
+#pragma unroll
+        for (int x = 0; x < PF_UNITS; ++x) acc[x] = u[x].c.o[dt] * alpha[x];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const bf16x8 vf = *reinterpret_cast<const bf16x8*>(vrow + h * 32 + g * 8);
+#pragma unroll
+            for (int x = 0; x < PF_UNITS; ++x) acc[x] = mfma_16x16x32(vf, pv[x][h], acc[x]);
+        }
+#pragma unroll
+        for (int x = 0; x < PF_UNITS; ++x) u[x].c.o[dt] = acc[x];
+    }
+}
+
+// grid (query tiles, nkv * head groups, sequences)
+__global__ __launch_bounds__(PF_THREADS) void attention_prefill_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ block_table, int max_pages, const int* __restrict__ seq_slot,
     const int* __restrict__ seq_start, const int* __restrict__ seq_new, const int* __restrict__ cu_new, int nh,
-    int nkv, float scale_log2, int window, bf16_t* __restrict__ out) {
-    const int b = blockIdx.z, kvh = blockIdx.y;
-    const int q0 = blockIdx.x * 16;
+    int nkv, float scale_log2, int window, int qb, int hg, bf16_t* __restrict__ out) {
+    constexpr int K_TILE = PAGE_TOKENS * K_STRIDE, V_TILE = HD * V_STRIDE;
+    __shared__ __attribute__((aligned(16))) bf16_t k_lds[PF_SHARE && V_TILE > K_TILE ? V_TILE : K_TILE];
+    __shared__ __attribute__((aligned(16))) bf16_t v_own[PF_SHARE ? 8 : V_TILE];
+    bf16_t* v_lds = PF_SHARE ? k_lds : v_own;
+
+    const int b = blockIdx.z;
+    const int G = nh / nkv, n_hg = (G + hg - 1) / hg;
+    const int kvh = blockIdx.y / n_hg, hgi = blockIdx.y % n_hg;
     const int n_new = seq_new[b];
+    const int q0 = (gridDim.x - 1 - blockIdx.x) * qb;            // late tiles first: they have the most keys
     if (q0 >= n_new) return;
-    const int G = nh / nkv;
     const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE, r = lane % 16, g = lane / 16;
     const int start = seq_start[b];
-    const bool valid = q0 + r < n_new;                  // column r is query position q0 + r of the step
-    const int pos = start + min(q0 + r, n_new - 1);     // its position in the sequence
-    const int row = cu_new[b] + min(q0 + r, n_new - 1);
-    // the tile's key range: from the first key of its first query to the last query's own position
-    const int tile_last = start + min(q0 + 15, n_new - 1);
-    const int tile_first = window > 0 ? max(0, start + q0 - window + 1) : 0;
-    const int my_first = window > 0 ? max(0, pos - window + 1) : 0;
+    const int heads_here = min(hg, G - hgi * hg);
+    const int n_units = heads_here * (qb / 16);
     const int* pages = block_table + (size_t)seq_slot[b] * max_pages;
 
-    for (int hq = wave; hq < G; hq += 4) {
-        const int head = kvh * G + hq;
-        bf16x8 qv[KSTEPS];
-        load_query(q + ((size_t)row * nh + head) * HD, true, g, qv);
-        Columns c;
-        c.m = -INFINITY;
-        c.l = 0.f;
+    Unit u[PF_UNITS];
 #pragma unroll
-        for (int dt = 0; dt < DTILES; ++dt) c.o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
-        // a column whose own range misses a page of the tile entirely adds nothing there (see score_page)
-        attend_pages(k_cache, v_cache, pages, nkv, kvh, tile_first / PAGE_TOKENS, tile_last / PAGE_TOKENS + 1, qv, my_first,
-                     pos, scale_log2, c, r, g);
-        float l = c.l;
+    for (int x = 0; x < PF_UNITS; ++x) {
+        const int unit = wave + x * PF_WAVES;
+        u[x].live = unit < n_units;
+        const int un = u[x].live ? unit : 0;
+        const int qi = q0 + (un / heads_here) * 16 + r;            // query index within the step
+        u[x].head = kvh * G + hgi * hg + un % heads_here;
+        u[x].valid = u[x].live && qi < n_new;
+        const int qc = min(qi, n_new - 1);
+        u[x].pos = start + qc;
+        u[x].first = window > 0 ? max(0, u[x].pos - window + 1) : 0;
+        u[x].row = (size_t)cu_new[b] + qc;
+        load_query(q + (u[x].row * nh + u[x].head) * HD, true, g, u[x].qv);
+        u[x].c.m = -INFINITY;
+        u[x].c.l = 0.f;
+#pragma unroll
+        for (int dt = 0; dt < DTILES; ++dt) u[x].c.o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+
+    const int tile_last = start + min(q0 + qb - 1, n_new - 1);
+    const int tile_first = window > 0 ? max(0, start + q0 - window + 1) : 0;
+    const int p_lo = tile_first / PAGE_TOKENS, p_hi = tile_last / PAGE_TOKENS;
+    PagePrefetch pf;
+    {
+        const size_t base = ((size_t)pages[p_lo] * nkv + kvh) * PAGE_TOKENS * HD;
+        prefetch_keys(k_cache + base, pf);
+        prefetch_values(v_cache + base, pf);
+    }
+    for (int p = p_lo; p <= p_hi; ++p) {
+        const bool more = p < p_hi;
+        const size_t next = more ? ((size_t)pages[p + 1] * nkv + kvh) * PAGE_TOKENS * HD : 0;
+        bf16x8 pv[PF_UNITS][2];
+        float alpha[PF_UNITS];
+        __syncthreads();                                        // everyone is done with the previous page
+        stage_keys(pf, k_lds);
+        if (!PF_SHARE) stage_values(pf, v_lds);
+        __syncthreads();
+        if (more) prefetch_keys(k_cache + next, pf);            // in flight while this page is used
+        unit_scores(k_lds, u, p * PAGE_TOKENS, scale_log2, r, g, pv, alpha);
+        if (PF_SHARE) {
+            __syncthreads();
+            stage_values(pf, v_lds);
+            __syncthreads();
+        }
+        if (more && !PF_SHARE) prefetch_values(v_cache + next, pf);
+        unit_values(v_lds, u, r, g, pv, alpha);
+        if (more && PF_SHARE) prefetch_values(v_cache + next, pf);
+    }
+
+#pragma unroll
+    for (int x = 0; x < PF_UNITS; ++x) {
+        float l = u[x].c.l;
         l += __shfl_xor(l, 16, WAVE);
         l += __shfl_xor(l, 32, WAVE);
-        if (valid) {
+        if (u[x].valid) {
             const float inv = 1.0f / l;
-            bf16_t* o = out + ((size_t)row * nh + head) * HD;
+            bf16_t* o = out + (u[x].row * nh + u[x].head) * HD;
 #pragma unroll
             for (int dt = 0; dt < DTILES; ++dt)
 #pragma unroll
-                for (int i = 0; i < 4; ++i) o[dt * 16 + 4 * g + i] = f32_to_bf16(c.o[dt][i] * inv);
+                for (int i = 0; i < 4; ++i) o[dt * 16 + 4 * g + i] = f32_to_bf16(u[x].c.o[dt][i] * inv);
         }
     }
 }
@@ -346,11 +512,15 @@ PALM_API int palm_attention_prefill(hipStream_t stream, const void* q, const voi
                "attention_prefill: seqs=%d max_new=%d heads=%d kv=%d", n_seqs, max_new, nh, nkv);
     PALM_CHECK(window >= 0 && max_pages > 0, "attention_prefill: window=%d max_pages=%d", window, max_pages);
     if (n_seqs == 0 || max_new == 0) return 0;
-    PALM_CHECK(nkv <= 65535 && n_seqs <= 65535, "attention_prefill: grid too large");
-    dim3 grid((max_new + 15) / 16, nkv, n_seqs);
-    attention_prefill_kernel<<<grid, 4 * WAVE, 0, stream>>>((const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache,
-                                                           block_table, max_pages, seq_slot, seq_start, seq_new, cu_new, nh,
-                                                           nkv, scale * LOG2E, window, (bf16_t*)out);
+    const int G = nh / nkv;
+    const int hg = G < 8 ? G : 8;                              // query heads of the group served by one block
+    const int qb = 16 * (8 / hg > 0 ? 8 / hg : 1);             // query positions in a tile: at most 8 units a block
+    const int n_hg = (G + hg - 1) / hg;
+    PALM_CHECK(nkv * n_hg <= 65535 && n_seqs <= 65535, "attention_prefill: grid too large");
+    dim3 grid((max_new + qb - 1) / qb, nkv * n_hg, n_seqs);
+    attention_prefill_kernel<<<grid, PF_THREADS, 0, stream>>>((const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache,
+                                                             block_table, max_pages, seq_slot, seq_start, seq_new, cu_new, nh,
+                                                             nkv, scale * LOG2E, window, qb, hg, (bf16_t*)out);
     PALM_LAUNCHED();
     return 0;
 }

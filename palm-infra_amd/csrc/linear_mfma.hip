@@ -110,7 +110,7 @@ template <typename TC, int EPI>
 static void dispatch_thin(hipStream_t stream, const void* a, const void* w, void* c, int M, int N, int K) {
     const bool deep = (K + SUPER_K - 1) / SUPER_K >= 16;       // enough super-steps to feed eight waves
     if (M <= 16) {
-        if (deep) launch_thin<1, 8, 4, TC, EPI>(stream, a, w, c, M, N, K);
+        if (deep) launch_thin<1, 8, 2, TC, EPI>(stream, a, w, c, M, N, K);      // two super-steps in flight a wave, two blocks a CU: measured best
         else launch_thin<1, 4, 2, TC, EPI>(stream, a, w, c, M, N, K);
     } else if (M <= 32) {
         if (deep) launch_thin<2, 8, 2, TC, EPI>(stream, a, w, c, M, N, K);
