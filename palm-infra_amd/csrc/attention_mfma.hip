@@ -297,7 +297,12 @@ PALM_API int palm_attention_decode(hipStream_t stream, const void* q, const void
 constexpr int PF_WAVES = 4;
 constexpr int PF_THREADS = PF_WAVES * WAVE;
 constexpr int PF_UNITS = 2;                                // units of 16 columns held by a wave
-constexpr int K_STRIDE = HD + 8;                           // padded rows: fragment reads of 16 rows spread over banks
+// K rows in LDS are a multiple of eight 16-byte chunks long and a row's chunks are permuted by its number
+// (chunk ^ swizzle(row)): the eight lanes that LDS serves together read one chunk column of keys
+// {0..3, 8..11} (or {4..7, 12..15}, ..), which the permutation sends to eight different bank groups.
+constexpr int K_CHUNKS = (CHUNKS + 7) / 8 * 8;
+constexpr int K_STRIDE = K_CHUNKS * 8;
+__device__ inline int k_swizzle(int row) { return (row & 3) | (((row >> 3) & 1) << 2); }
 constexpr int V_STRIDE = PAGE_TOKENS + 8;
 constexpr int PAGE_CHUNKS = PAGE_TOKENS * HD / 8;          // 16-byte chunks in a page of K (and of V^T)
 constexpr int PF_LOADS = (PAGE_CHUNKS + PF_THREADS - 1) / PF_THREADS;
@@ -323,7 +328,7 @@ __device__ inline void stage_keys(const PagePrefetch& pf, bf16_t* k_lds) {
 #pragma unroll
     for (int i = 0; i < PF_LOADS; ++i) {
         const int c = i * PF_THREADS + threadIdx.x;
-        if (c < PAGE_CHUNKS) *reinterpret_cast<bf16x8*>(k_lds + (c / CHUNKS) * K_STRIDE + (c % CHUNKS) * 8) = pf.k[i];
+        if (c < PAGE_CHUNKS) *reinterpret_cast<bf16x8*>(k_lds + (c / CHUNKS) * K_STRIDE + ((c % CHUNKS) ^ k_swizzle(c / CHUNKS)) * 8) = pf.k[i];
     }
 }
 __device__ inline void stage_values(const PagePrefetch& pf, bf16_t* v_lds) {
@@ -349,14 +354,15 @@ __device__ inline void unit_scores(const bf16_t* k_lds, Unit (&u)[PF_UNITS], int
     f32x4 s[PF_UNITS][4];
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
-        const bf16_t* krow = k_lds + tile_key(t, r) * K_STRIDE;
+        const int key_row = tile_key(t, r);
+        const bf16_t* krow = k_lds + key_row * K_STRIDE;
 #pragma unroll
         for (int x = 0; x < PF_UNITS; ++x) s[x][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int j = 0; j < KSTEPS; ++j) {
             const int chunk = j * 4 + g;
             const bool ok = (CHUNKS % 4 == 0) || chunk < CHUNKS;
-            bf16x8 kf = *reinterpret_cast<const bf16x8*>(krow + (ok ? chunk : 0) * 8);
+            bf16x8 kf = *reinterpret_cast<const bf16x8*>(krow + ((ok ? chunk : 0) ^ k_swizzle(key_row)) * 8);
             if (!ok) kf = zero_bf16x8();
 #pragma unroll
             for (int x = 0; x < PF_UNITS; ++x) s[x][t] = mfma_16x16x32(kf, u[x].qv[j], s[x][t]);

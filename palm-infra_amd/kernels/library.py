@@ -32,7 +32,7 @@ FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-fno-gpu-rdc",
          "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option"]
 
 CORE_SOURCES = ["elementwise.hip", "linear.hip", "rope_store.hip", "attention_simple.hip", "sampling.hip",
-                "linear_mfma.hip"]
+                "linear_mfma.hip", "linear_wide.hip"]
 ATTENTION_SOURCES = ["attention_mfma.hip"]
 HEADERS = ["common.h", "mfma.h"]
 

@@ -32,6 +32,8 @@ _SIGNATURES = {
     "palm_attention_simple": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                               c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
     "palm_linear_thin": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int],
+    "palm_linear_wide": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "palm_linear_wide_splits": [c_int, c_int, c_int, c_int],
     "palm_argmax": [c_void_p, c_void_p, c_int, c_int, c_void_p],
     "palm_apply_penalties": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_float, c_float, c_float],
     "palm_sample": [c_void_p, c_void_p, c_int, c_int, c_void_p, c_float, c_int, c_float, c_float, c_void_p, c_void_p],
@@ -47,7 +49,7 @@ def core():
         lib = library.load("core")
         for name, argtypes in _SIGNATURES.items():
             fn = getattr(lib, name)
-            fn.argtypes, fn.restype = argtypes, c_int
+            fn.argtypes, fn.restype = argtypes, c_int      # (palm_linear_wide_splits returns a count, not a status)
         if lib.palm_page_tokens() != PAGE_TOKENS:
             raise KernelError(f"the kernels were built for pages of {lib.palm_page_tokens()} tokens, "
                               f"the cache uses {PAGE_TOKENS}")
@@ -293,6 +295,9 @@ def linear_library(a: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     return torch.matmul(a, w.t())
 
 
+THIN_TOKENS = 16      # up to here every wave fetches its own activations; above, a block shares them through LDS
+
+
 def thin_serves(a: torch.Tensor, w: torch.Tensor) -> bool:
     """The matrix-core kernel for thin products takes bfloat16 operands whose rows start on 16 bytes."""
     return a.dtype == BF16 and w.dtype == BF16 and a.shape[1] % 8 == 0
@@ -312,8 +317,15 @@ def linear_thin(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, gated:
     N = w.shape[0]
     _need(not gated or N % 2 == 0, f"linear_thin: a gated product needs an even number of weight rows, got {N}")
     out = torch.empty((M, N // 2 if gated else N), dtype=out_dtype, device=a.device)
-    library.call(core(), "palm_linear_thin", _stream(), _p(a), _p(w), _p(out), _code(out, "linear_thin out"), M, N, K,
-                 1 if gated else 0)
+    if M <= THIN_TOKENS:
+        library.call(core(), "palm_linear_thin", _stream(), _p(a), _p(w), _p(out), _code(out, "linear_thin out"), M, N, K,
+                     1 if gated else 0)
+        return out
+    # more rows than one block of 16: the kernel that shares the activations through LDS, K split if need be
+    splits = core().palm_linear_wide_splits(M, N, K, 1 if gated else 0)
+    work = torch.empty((splits * M * N,), dtype=F32, device=a.device) if splits > 1 else None
+    library.call(core(), "palm_linear_wide", _stream(), _p(a), _p(w), _p(out), _code(out, "linear_wide out"), M, N, K,
+                 1 if gated else 0, splits, _p(work))
     return out
 
 
