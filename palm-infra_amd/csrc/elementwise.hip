@@ -178,9 +178,37 @@ __global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int
     }
 }
 
+// bfloat16 rows whose half is a multiple of 8: eight outputs a thread, 16-byte reads and writes
+__global__ void swiglu_bf16x8_kernel(const bf16_t* __restrict__ gu, bf16_t* __restrict__ out, int n_rows, int inter) {
+    const int per_row = inter / 8;
+    const size_t total = (size_t)n_rows * per_row;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        const size_t r = i / per_row, c = (i % per_row) * 8;
+        const uint4 g4 = *reinterpret_cast<const uint4*>(gu + r * 2 * inter + c);
+        const uint4 u4 = *reinterpret_cast<const uint4*>(gu + r * 2 * inter + inter + c);
+        const uint32_t gw[4] = {g4.x, g4.y, g4.z, g4.w}, uw[4] = {u4.x, u4.y, u4.z, u4.w};
+        uint32_t ow[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float g0 = __uint_as_float(gw[j] << 16), g1 = __uint_as_float(gw[j] & 0xffff0000u);
+            const float u0 = __uint_as_float(uw[j] << 16), u1 = __uint_as_float(uw[j] & 0xffff0000u);
+            const float o0 = g0 / (1.0f + expf(-g0)) * u0, o1 = g1 / (1.0f + expf(-g1)) * u1;
+            ow[j] = (uint32_t)f32_to_bf16(o0).bits | ((uint32_t)f32_to_bf16(o1).bits << 16);
+        }
+        *reinterpret_cast<uint4*>(out + r * inter + c) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+    }
+}
+
 PALM_API int palm_swiglu(hipStream_t stream, const void* gate_up, int dtype, void* out, int n_rows, int inter) {
     PALM_CHECK(n_rows >= 0 && inter > 0, "swiglu: rows=%d intermediate=%d", n_rows, inter);
     if (n_rows == 0) return 0;
+    if (dtype == PALM_BF16 && inter % 8 == 0 && ((uintptr_t)gate_up | (uintptr_t)out) % 16 == 0) {
+        const size_t work = (size_t)n_rows * (inter / 8);
+        const int blocks = (int)((work + 255) / 256 < 16384 ? (work + 255) / 256 : 16384);
+        swiglu_bf16x8_kernel<<<blocks, 256, 0, stream>>>((const bf16_t*)gate_up, (bf16_t*)out, n_rows, inter);
+        PALM_LAUNCHED();
+        return 0;
+    }
     const size_t total = (size_t)n_rows * inter;
     const int blocks = (int)((total + 255) / 256 < 65536 ? (total + 255) / 256 : 65536);
     PALM_DTYPE_SWITCH(dtype, T,
