@@ -168,7 +168,12 @@ __device__ inline void load_query(const bf16_t* qrow, bool valid, int g, bf16x8 
 // ---- decode ---------------------------------------------------------------------------------------
 // grid (slices, nkv * query groups, sequences), one wave each.  Workspace per (sequence, head, slice):
 // m, l, then HD floats of the unnormalised output.
-__global__ __launch_bounds__(WAVE) void attention_decode_kernel(
+#if PALM_HEAD_DIM <= 128
+#define DECODE_WAVES_PER_SIMD __attribute__((amdgpu_waves_per_eu(2)))     // fits without spilling up to this head size
+#else
+#define DECODE_WAVES_PER_SIMD
+#endif
+__global__ __launch_bounds__(WAVE) DECODE_WAVES_PER_SIMD void attention_decode_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ block_table, int max_pages, const int* __restrict__ seq_slot,
     const int* __restrict__ seq_start, int nh, int nkv, float scale_log2, int window, int n_slices,
@@ -349,41 +354,60 @@ struct Unit {                 // one (head, 16 query positions): the wave's shar
     Columns c;
 };
 
+__device__ inline void read_key_fragments(const bf16_t* k_lds, int t, int r, int g, bf16x8 (&kf)[KSTEPS]) {
+    const int key_row = tile_key(t, r);
+    const bf16_t* krow = k_lds + key_row * K_STRIDE;
+#pragma unroll
+    for (int j = 0; j < KSTEPS; ++j) {
+        const int chunk = j * 4 + g;
+        const bool ok = (CHUNKS % 4 == 0) || chunk < CHUNKS;
+        kf[j] = *reinterpret_cast<const bf16x8*>(krow + ((ok ? chunk : 0) ^ k_swizzle(key_row)) * 8);
+        if (!ok) kf[j] = zero_bf16x8();
+    }
+}
+
+// Scores and softmax of one page for the wave's units.  The fragments of key tile t+1 are read from LDS
+// before the products of tile t run, so a read's latency hides behind arithmetic.  `interior`: every key of
+// the page is visible to every column of the wave (the usual case away from the diagonal), no masking then.
 __device__ inline void unit_scores(const bf16_t* k_lds, Unit (&u)[PF_UNITS], int page_first_key, float scale_log2,
-                                   int r, int g, bf16x8 (&pv)[PF_UNITS][2], float (&alpha)[PF_UNITS]) {
+                                   int r, int g, bool interior, bf16x8 (&pv)[PF_UNITS][2], float (&alpha)[PF_UNITS]) {
     f32x4 s[PF_UNITS][4];
+    bf16x8 kf[2][KSTEPS];
+    read_key_fragments(k_lds, 0, r, g, kf[0]);
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
-        const int key_row = tile_key(t, r);
-        const bf16_t* krow = k_lds + key_row * K_STRIDE;
+        if (t < 3) read_key_fragments(k_lds, t + 1, r, g, kf[(t + 1) & 1]);
 #pragma unroll
         for (int x = 0; x < PF_UNITS; ++x) s[x][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int j = 0; j < KSTEPS; ++j) {
-            const int chunk = j * 4 + g;
-            const bool ok = (CHUNKS % 4 == 0) || chunk < CHUNKS;
-            bf16x8 kf = *reinterpret_cast<const bf16x8*>(krow + ((ok ? chunk : 0) ^ k_swizzle(key_row)) * 8);
-            if (!ok) kf = zero_bf16x8();
+        for (int j = 0; j < KSTEPS; ++j)
 #pragma unroll
-            for (int x = 0; x < PF_UNITS; ++x) s[x][t] = mfma_16x16x32(kf, u[x].qv[j], s[x][t]);
-        }
+            for (int x = 0; x < PF_UNITS; ++x) s[x][t] = mfma_16x16x32(kf[t & 1][j], u[x].qv[j], s[x][t]);
     }
 #pragma unroll
     for (int x = 0; x < PF_UNITS; ++x) {
         Columns& c = u[x].c;
-        const int lo = u[x].first - page_first_key, hi = u[x].pos - page_first_key;
         float mx = -INFINITY;
+        if (interior) {
 #pragma unroll
-        for (int t = 0; t < 4; ++t)
+            for (int t = 0; t < 4; ++t)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int key = tile_key(t, 4 * g + i);
-                const float v = (key >= lo && key <= hi) ? s[x][t][i] * scale_log2 : -INFINITY;
-                s[x][t][i] = v;
-                mx = fmaxf(mx, v);
-            }
+                for (int i = 0; i < 4; ++i) mx = fmaxf(mx, s[x][t][i]);
+        } else {
+            const int lo = u[x].first - page_first_key, hi = u[x].pos - page_first_key;
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int key = tile_key(t, 4 * g + i);
+                    const float v = (key >= lo && key <= hi) ? s[x][t][i] : -INFINITY;
+                    s[x][t][i] = v;
+                    mx = fmaxf(mx, v);
+                }
+        }
         mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
         mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+        mx *= scale_log2;                                           // the scale is positive: the maximum commutes with it
         const float m_new = fmaxf(c.m, mx);
         const float m_sub = m_new == -INFINITY ? 0.f : m_new;       // see score_page
         alpha[x] = exp2f(c.m - m_sub);
@@ -392,7 +416,7 @@ __device__ inline void unit_scores(const bf16_t* k_lds, Unit (&u)[PF_UNITS], int
         for (int h = 0; h < 2; ++h)
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                const float p = exp2f(s[x][2 * h + e / 4][e % 4] - m_sub);
+                const float p = exp2f(fmaf(s[x][2 * h + e / 4][e % 4], scale_log2, -m_sub));
                 sum += p;
                 pv[x][h][e] = (__bf16)p;
             }
@@ -401,27 +425,42 @@ __device__ inline void unit_scores(const bf16_t* k_lds, Unit (&u)[PF_UNITS], int
     }
 }
 
+// The weighted values of one page.  `rescale` false: no column's maximum moved (every alpha is 1), the
+// outputs stay where the matrix cores keep them.
 __device__ inline void unit_values(const bf16_t* v_lds, Unit (&u)[PF_UNITS], int r, int g,
-                                   const bf16x8 (&pv)[PF_UNITS][2], const float (&alpha)[PF_UNITS]) {
+                                   const bf16x8 (&pv)[PF_UNITS][2], const float (&alpha)[PF_UNITS], bool rescale) {
+    if (rescale) {
+#pragma unroll
+        for (int x = 0; x < PF_UNITS; ++x)
+#pragma unroll
+            for (int dt = 0; dt < DTILES; ++dt) u[x].c.o[dt] = u[x].c.o[dt] * alpha[x];
+    }
+    bf16x8 vf[2][2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) vf[0][h] = *reinterpret_cast<const bf16x8*>(v_lds + r * V_STRIDE + h * 32 + g * 8);
 #pragma unroll
     for (int dt = 0; dt < DTILES; ++dt) {
-        const bf16_t* vrow = v_lds + (dt * 16 + r) * V_STRIDE;
-        f32x4 acc[PF_UNITS];
+        if (dt + 1 < DTILES) {
+            const bf16_t* vrow = v_lds + ((dt + 1) * 16 + r) * V_STRIDE;
 #pragma unroll
-        for (int x = 0; x < PF_UNITS; ++x) acc[x] = u[x].c.o[dt] * alpha[x];
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            const bf16x8 vf = *reinterpret_cast<const bf16x8*>(vrow + h * 32 + g * 8);
-#pragma unroll
-            for (int x = 0; x < PF_UNITS; ++x) acc[x] = mfma_16x16x32(vf, pv[x][h], acc[x]);
+            for (int h = 0; h < 2; ++h) vf[(dt + 1) & 1][h] = *reinterpret_cast<const bf16x8*>(vrow + h * 32 + g * 8);
         }
 #pragma unroll
-        for (int x = 0; x < PF_UNITS; ++x) u[x].c.o[dt] = acc[x];
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int x = 0; x < PF_UNITS; ++x) u[x].c.o[dt] = mfma_16x16x32(vf[dt & 1][h], pv[x][h], u[x].c.o[dt]);
     }
 }
 
 // grid (query tiles, nkv * head groups, sequences)
-__global__ __launch_bounds__(PF_THREADS) void attention_prefill_kernel(
+// Two waves on a SIMD, where the head size lets the registers fit without spilling: a second block on the
+// compute unit runs while one waits at a barrier or for LDS.
+#if PALM_HEAD_DIM <= 128
+#define PF_WAVES_PER_SIMD __attribute__((amdgpu_waves_per_eu(2)))
+#else
+#define PF_WAVES_PER_SIMD
+#endif
+__global__ __launch_bounds__(PF_THREADS) PF_WAVES_PER_SIMD void attention_prefill_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ block_table, int max_pages, const int* __restrict__ seq_slot,
     const int* __restrict__ seq_start, const int* __restrict__ seq_new, const int* __restrict__ cu_new, int nh,
@@ -482,14 +521,24 @@ __global__ __launch_bounds__(PF_THREADS) void attention_prefill_kernel(
         if (!PF_SHARE) stage_values(pf, v_lds);
         __syncthreads();
         if (more) prefetch_keys(k_cache + next, pf);            // in flight while this page is used
-        unit_scores(k_lds, u, p * PAGE_TOKENS, scale_log2, r, g, pv, alpha);
+        // is every key of this page visible to every column of this wave?
+        bool inside = true;
+#pragma unroll
+        for (int x = 0; x < PF_UNITS; ++x)
+            inside = inside && u[x].first <= p * PAGE_TOKENS && u[x].pos >= p * PAGE_TOKENS + PAGE_TOKENS - 1;
+        const bool interior = __all(inside);
+        unit_scores(k_lds, u, p * PAGE_TOKENS, scale_log2, r, g, interior, pv, alpha);
+        bool moved = false;
+#pragma unroll
+        for (int x = 0; x < PF_UNITS; ++x) moved = moved || alpha[x] != 1.0f;
+        const bool rescale = __any(moved);
         if (PF_SHARE) {
             __syncthreads();
             stage_values(pf, v_lds);
             __syncthreads();
         }
         if (more && !PF_SHARE) prefetch_values(v_cache + next, pf);
-        unit_values(v_lds, u, r, g, pv, alpha);
+        unit_values(v_lds, u, r, g, pv, alpha, rescale);
         if (more && PF_SHARE) prefetch_values(v_cache + next, pf);
     }
 
