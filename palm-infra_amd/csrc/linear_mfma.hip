@@ -15,6 +15,8 @@
 // RT = 2 halves the activation reads per weight byte but was measured slower; RT = 1 is what runs.
 #include "mfma.h"
 
+#include <type_traits>
+
 enum ThinEpilogue : int { EPI_STORE = 0, EPI_SWIGLU = 1 };
 
 constexpr int SUPER_K = 128;
@@ -120,15 +122,175 @@ static void launch_thin(hipStream_t stream, const void* a, const void* w, void* 
         (const bf16_t*)a, (const bf16_t*)w, (TC*)c, M, N, K);
 }
 
+// The same product for up to 16 rows and a long K, as a stream: fewer blocks than strips, each walking over
+// its strips (strip = block, block + grid, ...) with the weight reads of the next steps always in flight, also
+// across the end of a strip.  A wave keeps a ring of U super-steps: it uses the oldest and at once asks for
+// the one U ahead into the same registers, so the memory pipe never drains between a block's first and last
+// byte; only the last U steps of a block ask for nothing.  With TREG > 0 a wave's share of the activations
+// (super-steps wave, wave + NW, ..., TREG of them, the same for every strip) is read once and stays in
+// registers; with TREG == 0 it is read again beside every weight read.  At eight rows the register form is
+// what brings the gated product from 45 to 36 us and the head from 260 to 212 us: an activation read costs
+// the cache path as much as a weight read although it brings nothing new.
+// T: steps a wave makes for one strip, a multiple of U; steps beyond K read nothing and count as zeros
+// (EXACT says there are none, and then nothing is masked).
+constexpr int STREAM_WAVES = 8;
+constexpr int STREAM_SLOTS = 512;      // blocks that run at once: two on each of 256 compute units
+
+template <int U, int TREG, bool EXACT, typename TC, int EPI>
+__global__ __launch_bounds__(STREAM_WAVES * WAVE) void linear_stream_kernel(const bf16_t* __restrict__ A,
+                                                                            const bf16_t* __restrict__ W,
+                                                                            TC* __restrict__ C, int M, int N, int K,
+                                                                            int n_strips, int T_given) {
+    constexpr int NW = STREAM_WAVES;
+    constexpr bool AREG = TREG > 0;
+    __shared__ float part[2][NW][16][17];
+    const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
+    const int r = lane % 16, g = lane / 16;
+    const int inter = N / 2;
+    const int T = AREG ? TREG : T_given;
+
+    auto row_of = [&](int strip) -> const bf16_t* {
+        int wrow;
+        if (EPI == EPI_SWIGLU) wrow = (r < 8 ? 0 : inter) + min(strip * 8 + (r % 8), inter - 1);
+        else wrow = min(strip * 16 + r, N - 1);
+        return W + (size_t)wrow * K + g * 8;
+    };
+    const bf16_t* xp = A + (size_t)min(r, M - 1) * K + g * 8;
+
+    // the read cursor runs U steps ahead of the arithmetic
+    int ask_strip = blockIdx.x, ask_t = 0;
+    const bf16_t* ask_row = row_of(ask_strip);
+    bf16x8 wv[U][4], xv[U][4];
+    int present[U];                                          // bit j: chunk j of the slot lies inside K
+    auto ask = [&](int u) {
+        const int k0 = (ask_t * NW + wave) * SUPER_K;
+        int mask = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const bool ok = EXACT || (k0 + j * 32 + g * 8 < K);
+            const int at = ok ? k0 + j * 32 : 0;             // an absent chunk reads the row's start and is masked
+            wv[u][j] = load_bf16x8(ask_row + at);
+            if (!AREG) xv[u][j] = load_bf16x8(xp + at);
+            mask |= (ok ? 1 : 0) << j;
+        }
+        present[u] = mask;
+        if (++ask_t == T) {
+            ask_t = 0;
+            ask_strip += gridDim.x;
+            ask_row = row_of(min(ask_strip, n_strips - 1));
+        }
+    };
+#pragma unroll
+    for (int u = 0; u < U; ++u) ask(u);                      // weights first: they come from furthest away
+
+    bf16x8 xa[AREG ? TREG : 1][4];
+    if (AREG) {
+#pragma unroll
+        for (int t = 0; t < TREG; ++t) {
+            const int k0 = (t * NW + wave) * SUPER_K;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const bool ok = EXACT || (k0 + j * 32 + g * 8 < K);
+                const bf16x8 v = load_bf16x8(xp + (ok ? k0 + j * 32 : 0));
+                xa[t][j] = ok ? v : zero_bf16x8();
+            }
+        }
+    }
+
+    int buf = 0;
+    for (int strip = blockIdx.x; strip < n_strips; strip += gridDim.x) {
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        const bool last = strip + (int)gridDim.x >= n_strips;
+        // U steps: use each slot and, if `refill`, ask for the step U ahead into it
+        auto steps = [&](int t, auto refill) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    bf16x8 wj = wv[u][j];
+                    bf16x8 xj = AREG ? xa[AREG && t + u < TREG ? t + u : 0][j] : xv[u][j];
+                    if (!EXACT) {
+                        const bool ok = (present[u] >> j) & 1;
+                        wj = ok ? wj : zero_bf16x8();
+                        if (!AREG) xj = ok ? xj : zero_bf16x8();
+                    }
+                    acc = mfma_16x16x32(wj, xj, acc);
+                }
+                if (decltype(refill)::value) ask(u);
+            }
+        };
+        if (AREG) {
+#pragma unroll
+            for (int t = 0; t + U < TREG; t += U) steps(t, std::true_type{});
+            if (last) steps(TREG - U, std::false_type{});
+            else steps(TREG - U, std::true_type{});
+        } else {
+            for (int t = 0; t + U < T; t += U) steps(0, std::true_type{});
+            if (last) steps(0, std::false_type{});
+            else steps(0, std::true_type{});
+        }
+
+        // partial tiles of the waves are added in a fixed order; two buffers, so one barrier a strip is enough
+#pragma unroll
+        for (int i = 0; i < 4; ++i) part[buf][wave][4 * g + i][r] = acc[i];
+        __syncthreads();
+        if (EPI == EPI_SWIGLU) {
+            if (threadIdx.x < 128) {
+                const int c = threadIdx.x % 8, col = threadIdx.x / 8;
+                float gate = 0.f, up = 0.f;
+#pragma unroll
+                for (int w = 0; w < NW; ++w) { gate += part[buf][w][c][col]; up += part[buf][w][c + 8][col]; }
+                const int feat = strip * 8 + c;
+                if (col < M && feat < inter) C[(size_t)col * inter + feat] = from_float<TC>(gate / (1.0f + expf(-gate)) * up);
+            }
+        } else {
+            if (threadIdx.x < 256) {
+                const int row = threadIdx.x % 16, col = threadIdx.x / 16;
+                float v = 0.f;
+#pragma unroll
+                for (int w = 0; w < NW; ++w) v += part[buf][w][row][col];
+                const int feat = strip * 16 + row;
+                if (col < M && feat < N) C[(size_t)col * N + feat] = from_float<TC>(v);
+            }
+        }
+        buf ^= 1;
+    }
+}
+
+template <int U, int TREG, typename TC, int EPI>
+static void launch_stream(hipStream_t stream, const void* a, const void* w, void* c, int M, int N, int K) {
+    const int strips = EPI == EPI_SWIGLU ? (N / 2 + 7) / 8 : (N + 15) / 16;
+    const int n_super = (K + SUPER_K - 1) / SUPER_K;
+    int T = (n_super + STREAM_WAVES - 1) / STREAM_WAVES;
+    T = (T + U - 1) / U * U;
+    if (TREG > 0) T = TREG;
+    // every block the same number of strips, as far as that goes
+    const int rounds = (strips + STREAM_SLOTS - 1) / STREAM_SLOTS;
+    const int grid = (strips + rounds - 1) / rounds;
+    const bool exact = K % SUPER_K == 0 && T * STREAM_WAVES == n_super;
+    if (exact)
+        linear_stream_kernel<U, TREG, true, TC, EPI><<<grid, STREAM_WAVES * WAVE, 0, stream>>>(
+            (const bf16_t*)a, (const bf16_t*)w, (TC*)c, M, N, K, strips, T);
+    else
+        linear_stream_kernel<U, TREG, false, TC, EPI><<<grid, STREAM_WAVES * WAVE, 0, stream>>>(
+            (const bf16_t*)a, (const bf16_t*)w, (TC*)c, M, N, K, strips, T);
+}
+
 template <typename TC, int EPI>
 static void dispatch_thin(hipStream_t stream, const void* a, const void* w, void* c, int M, int N, int K) {
-    const bool deep = (K + SUPER_K - 1) / SUPER_K >= 16;       // enough super-steps to feed eight waves
+    const int n_super = (K + SUPER_K - 1) / SUPER_K;
+    const bool deep = n_super >= 16;                           // enough super-steps to feed eight waves
+    if (M <= 16 && deep) {
+        const int per_wave = (n_super + STREAM_WAVES - 1) / STREAM_WAVES;
+        if (per_wave <= 2) launch_stream<2, 2, TC, EPI>(stream, a, w, c, M, N, K);
+        else if (per_wave <= 4) launch_stream<2, 4, TC, EPI>(stream, a, w, c, M, N, K);
+        else launch_stream<4, 0, TC, EPI>(stream, a, w, c, M, N, K);
+        return;
+    }
     if (M <= 16) {
-        // eight waves, two super-steps in flight each, two blocks on a compute unit: measured best
-        // (two strips a block, RT = 2, were measured slower at every size: 50.6 against 43.1 us for the gated
-        // product at 8 rows, 327 against 243 us for the head)
-        if (deep) launch_thin<1, 8, 2, 1, TC, EPI>(stream, a, w, c, M, N, K);
-        else launch_thin<1, 4, 2, 1, TC, EPI>(stream, a, w, c, M, N, K);
+        // a short K: one strip a block, four waves (two strips a block, RT = 2, were measured slower at every
+        // size)
+        launch_thin<1, 4, 2, 1, TC, EPI>(stream, a, w, c, M, N, K);
     } else if (M <= 32) {
         if (deep) launch_thin<2, 8, 2, 1, TC, EPI>(stream, a, w, c, M, N, K);
         else launch_thin<2, 4, 2, 1, TC, EPI>(stream, a, w, c, M, N, K);

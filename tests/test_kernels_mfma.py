@@ -21,7 +21,8 @@ def rand(*shape, seed=0, scale=1.0, dtype=BF16):
 
 
 @pytest.mark.parametrize("M", [1, 8, 16, 17, 33, 64, 70, 150])
-@pytest.mark.parametrize("N,K", [(7, 8), (130, 64), (515, 80), (1000, 224), (96, 4096), (4096, 1536), (300, 12288)])
+@pytest.mark.parametrize("N,K", [(7, 8), (130, 64), (515, 80), (1000, 224), (96, 4096), (4096, 1536), (300, 12288),
+                                 (1000, 2048), (515, 2056), (130, 5000), (9000, 2048), (8200, 3080)])
 def test_linear_thin_against_the_plain_product(ops, M, N, K):
     a, w = rand(M, K, seed=M + K), rand(N, K, seed=N, scale=0.5)
     ref = P.linear(a, w)
@@ -48,7 +49,7 @@ def test_linear_thin_orientation(ops):
 
 
 @pytest.mark.parametrize("M", [1, 8, 20, 64])
-@pytest.mark.parametrize("I,K", [(5, 16), (176, 80), (224, 96), (1536, 512)])
+@pytest.mark.parametrize("I,K", [(5, 16), (176, 80), (224, 96), (1536, 512), (4500, 2048), (300, 3000), (100, 6000)])
 def test_linear_thin_gated(ops, M, I, K):
     a, w = rand(M, K, seed=M), rand(2 * I, K, seed=I, scale=0.3)
     g, u = P.linear(a, w[:I]), P.linear(a, w[I:])
