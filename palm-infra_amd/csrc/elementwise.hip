@@ -40,8 +40,13 @@ PALM_API int palm_embed(hipStream_t stream, const void* table, int table_dtype, 
 // One block per output row.  src row = rows ? rows[r] : r.  v = x[src] (+ delta[src]).  If update_x the
 // sum is written back to x (only without `rows`), so the residual stream is updated and normed in one
 // pass over it.  Statistics and products in 32-bit; the product order is (v * r) * w.
+// delta may be `planes` planes of partial sums, plane_stride elements apart (a projection that cut its K into
+// ranges); they are added one after the other, plane 0 first.
+constexpr int NORM_MAX_PLANES = 4;
+
 template <typename TX, typename TD, typename TO>
-__global__ void rmsnorm_kernel(TX* __restrict__ x, const TD* __restrict__ delta, const float* __restrict__ w,
+__global__ void rmsnorm_kernel(TX* __restrict__ x, const TD* __restrict__ delta, int planes, size_t plane_stride,
+                               const float* __restrict__ w,
                                const int* __restrict__ rows, TO* __restrict__ out, int width, float eps,
                                int update_x) {
     __shared__ float scratch[16];
@@ -52,7 +57,7 @@ __global__ void rmsnorm_kernel(TX* __restrict__ x, const TD* __restrict__ delta,
     float ss = 0.f;
     for (int d = threadIdx.x; d < width; d += blockDim.x) {
         float v = to_float(xr[d]);
-        if (dr) v += to_float(dr[d]);
+        if (dr) for (int p = 0; p < planes; ++p) v += to_float(dr[p * plane_stride + d]);
         ss += v * v;
     }
     ss = block_sum(ss, scratch);
@@ -60,7 +65,7 @@ __global__ void rmsnorm_kernel(TX* __restrict__ x, const TD* __restrict__ delta,
     TO* o = out + (size_t)r * width;
     for (int d = threadIdx.x; d < width; d += blockDim.x) {
         float v = to_float(xr[d]);
-        if (dr) v += to_float(dr[d]);
+        if (dr) for (int p = 0; p < planes; ++p) v += to_float(dr[p * plane_stride + d]);
         if (update_x) xr[d] = from_float<TX>(v);
         o[d] = from_float<TO>(v * inv * w[d]);
     }
@@ -86,8 +91,9 @@ __device__ inline void store4(bf16_t* p, const float (&v)[4]) {
     *reinterpret_cast<uint2*>(p) = t;
 }
 
-template <typename TX, typename TD, typename TO, int ITERS>
-__global__ void rmsnorm_fast_kernel(TX* __restrict__ x, const TD* __restrict__ delta, const float* __restrict__ w,
+template <typename TX, typename TD, typename TO, int ITERS, int PLANES>
+__global__ void rmsnorm_fast_kernel(TX* __restrict__ x, const TD* __restrict__ delta, int planes, size_t plane_stride,
+                                    const float* __restrict__ w,
                                     const int* __restrict__ rows, TO* __restrict__ out, int width, float eps,
                                     int update_x) {
     __shared__ float scratch[16];
@@ -95,14 +101,17 @@ __global__ void rmsnorm_fast_kernel(TX* __restrict__ x, const TD* __restrict__ d
     const size_t src = rows ? (size_t)rows[r] : (size_t)r;
     TX* xr = x + src * width;
     const TD* dr = delta ? delta + src * width : nullptr;
-    float v[ITERS][4], d[ITERS][4], wt[ITERS][4];
+    float v[ITERS][4], d[PLANES][ITERS][4], wt[ITERS][4];
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
         const int i = (it * blockDim.x + threadIdx.x) * 4;
         const int at = i < width ? i : 0;                   // a thread beyond the row reads its start and adds nothing
         load4(xr + at, v[it]);
         load4(w + at, wt[it]);
-        if (dr) load4(dr + at, d[it]);
+        if (dr) {
+#pragma unroll
+            for (int p = 0; p < PLANES; ++p) load4(dr + (size_t)min(p, planes - 1) * plane_stride + at, d[p][it]);   // an absent plane reads the last one and adds nothing
+        }
     }
     float ss = 0.f;
 #pragma unroll
@@ -110,7 +119,10 @@ __global__ void rmsnorm_fast_kernel(TX* __restrict__ x, const TD* __restrict__ d
         const bool in = (it * blockDim.x + threadIdx.x) * 4 < width;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            if (dr) v[it][e] += d[it][e];
+            if (dr) {
+#pragma unroll
+                for (int p = 0; p < PLANES; ++p) v[it][e] += p < planes ? d[p][it][e] : 0.f;
+            }
             if (in) ss += v[it][e] * v[it][e];
         }
     }
@@ -130,7 +142,8 @@ __global__ void rmsnorm_fast_kernel(TX* __restrict__ x, const TD* __restrict__ d
 }
 
 template <typename TX, typename TD, typename TO>
-static bool launch_rmsnorm_fast(hipStream_t stream, void* x, const void* delta, const float* weight, float eps,
+static bool launch_rmsnorm_fast(hipStream_t stream, void* x, const void* delta, int planes, size_t plane_stride,
+                                const float* weight, float eps,
                                 const int* rows, int n_out_rows, int width, void* out, int update_x) {
     if (width % 4 != 0 || width > 32768) return false;
     const int quads = width / 4;
@@ -138,30 +151,40 @@ static bool launch_rmsnorm_fast(hipStream_t stream, void* x, const void* delta, 
     int threads = (quads + iters - 1) / iters;
     threads = (threads + WAVE - 1) / WAVE * WAVE;
     if (threads > 1024) return false;
-#define PALM_NORM_CASE(IT) case IT: rmsnorm_fast_kernel<TX, TD, TO, IT><<<n_out_rows, threads, 0, stream>>>( \
-        (TX*)x, (const TD*)delta, weight, rows, (TO*)out, width, eps, update_x); break;
+#define PALM_NORM_CASE(IT) case IT: \
+        if (planes > 1) rmsnorm_fast_kernel<TX, TD, TO, IT, NORM_MAX_PLANES><<<n_out_rows, threads, 0, stream>>>( \
+            (TX*)x, (const TD*)delta, planes, plane_stride, weight, rows, (TO*)out, width, eps, update_x); \
+        else rmsnorm_fast_kernel<TX, TD, TO, IT, 1><<<n_out_rows, threads, 0, stream>>>( \
+            (TX*)x, (const TD*)delta, 1, plane_stride, weight, rows, (TO*)out, width, eps, update_x); \
+        break;
     switch (iters) { PALM_NORM_CASE(1) PALM_NORM_CASE(2) PALM_NORM_CASE(4) PALM_NORM_CASE(8) }
 #undef PALM_NORM_CASE
     return true;
 }
 
-PALM_API int palm_rmsnorm(hipStream_t stream, void* x, int x_dtype, const void* delta, int delta_dtype,
+// delta_planes > 1: delta is [delta_planes, rows of x, width] float32.
+PALM_API int palm_rmsnorm(hipStream_t stream, void* x, int x_dtype, const void* delta, int delta_dtype, int delta_planes,
                           const float* weight, float eps, const int* rows, int n_out_rows, int width,
-                          void* out, int out_dtype, int update_x) {
+                          void* out, int out_dtype, int update_x, long long x_rows) {
     PALM_CHECK(n_out_rows >= 0 && width > 0, "rmsnorm: rows=%d width=%d", n_out_rows, width);
     PALM_CHECK(!(update_x && rows), "rmsnorm: the residual cannot be updated through a row selection");
     PALM_CHECK(!(update_x && !delta), "rmsnorm: update_x without a delta has nothing to add");
+    PALM_CHECK(delta_planes >= 1 && delta_planes <= NORM_MAX_PLANES, "rmsnorm: %d planes of delta (at most %d)",
+               delta_planes, NORM_MAX_PLANES);
+    PALM_CHECK(delta_planes == 1 || (delta && delta_dtype == PALM_F32), "rmsnorm: planes of delta are float32");
     if (n_out_rows == 0) return 0;
+    const size_t plane_stride = (size_t)x_rows * width;
     {
         bool done = false;
         PALM_DTYPE_SWITCH(x_dtype, TX, PALM_DTYPE_SWITCH(delta_dtype, TD, PALM_DTYPE_SWITCH(out_dtype, TO,
-            done = launch_rmsnorm_fast<TX, TD, TO>(stream, x, delta, weight, eps, rows, n_out_rows, width, out, update_x))));
+            done = launch_rmsnorm_fast<TX, TD, TO>(stream, x, delta, delta_planes, plane_stride, weight, eps, rows, n_out_rows,
+                                                   width, out, update_x))));
         if (done) { PALM_LAUNCHED(); return 0; }
     }
     const int threads = width >= 1024 ? 256 : (width >= 256 ? 128 : 64);
     PALM_DTYPE_SWITCH(x_dtype, TX, PALM_DTYPE_SWITCH(delta_dtype, TD, PALM_DTYPE_SWITCH(out_dtype, TO,
         rmsnorm_kernel<TX, TD, TO><<<n_out_rows, threads, 0, stream>>>(
-            (TX*)x, (const TD*)delta, weight, rows, (TO*)out, width, eps, update_x))));
+            (TX*)x, (const TD*)delta, delta_planes, plane_stride, weight, rows, (TO*)out, width, eps, update_x))));
     PALM_LAUNCHED();
     return 0;
 }

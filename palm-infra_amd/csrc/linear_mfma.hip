@@ -133,14 +133,20 @@ static void launch_thin(hipStream_t stream, const void* a, const void* w, void* 
 // the cache path as much as a weight read although it brings nothing new.
 // T: steps a wave makes for one strip, a multiple of U; steps beyond K read nothing and count as zeros
 // (EXACT says there are none, and then nothing is masked).
+// Few strips and a long K (an output projection: 256 strips) leave most of the chip without work.  Then K is
+// cut into `parts` ranges, blockIdx.y names the range, and the block writes its partial sums to plane
+// blockIdx.y of a [parts, M, N] float32 result; whoever reads the result adds the planes in their order (the
+// norm that follows adds them to the residual stream), so the sum is the same bits every time.
 constexpr int STREAM_WAVES = 8;
 constexpr int STREAM_SLOTS = 512;      // blocks that run at once: two on each of 256 compute units
+constexpr int STREAM_SLOTS_CUT = 768;  // with K cut into ranges a block's work is short: three
 
 template <int U, int TREG, bool EXACT, typename TC, int EPI>
 __global__ __launch_bounds__(STREAM_WAVES * WAVE) void linear_stream_kernel(const bf16_t* __restrict__ A,
                                                                             const bf16_t* __restrict__ W,
                                                                             TC* __restrict__ C, int M, int N, int K,
                                                                             int n_strips, int T_given) {
+    // this block's range of K starts at super-step blockIdx.y * T * NW, its results go to plane blockIdx.y
     constexpr int NW = STREAM_WAVES;
     constexpr bool AREG = TREG > 0;
     __shared__ float part[2][NW][16][17];
@@ -148,6 +154,8 @@ __global__ __launch_bounds__(STREAM_WAVES * WAVE) void linear_stream_kernel(cons
     const int r = lane % 16, g = lane / 16;
     const int inter = N / 2;
     const int T = AREG ? TREG : T_given;
+    const int first_super = blockIdx.y * T * NW;
+    if (EPI == EPI_STORE) C += (size_t)blockIdx.y * M * N;
 
     auto row_of = [&](int strip) -> const bf16_t* {
         int wrow;
@@ -163,7 +171,7 @@ __global__ __launch_bounds__(STREAM_WAVES * WAVE) void linear_stream_kernel(cons
     bf16x8 wv[U][4], xv[U][4];
     int present[U];                                          // bit j: chunk j of the slot lies inside K
     auto ask = [&](int u) {
-        const int k0 = (ask_t * NW + wave) * SUPER_K;
+        const int k0 = (first_super + ask_t * NW + wave) * SUPER_K;
         int mask = 0;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -187,7 +195,7 @@ __global__ __launch_bounds__(STREAM_WAVES * WAVE) void linear_stream_kernel(cons
     if (AREG) {
 #pragma unroll
         for (int t = 0; t < TREG; ++t) {
-            const int k0 = (t * NW + wave) * SUPER_K;
+            const int k0 = (first_super + t * NW + wave) * SUPER_K;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const bool ok = EXACT || (k0 + j * 32 + g * 8 < K);
@@ -257,17 +265,43 @@ __global__ __launch_bounds__(STREAM_WAVES * WAVE) void linear_stream_kernel(cons
     }
 }
 
+// steps a wave makes for one strip when K is cut into `parts` ranges
+static int stream_steps(int n_super, int parts) {
+    const int per_part = (n_super + parts - 1) / parts;
+    return (per_part + STREAM_WAVES - 1) / STREAM_WAVES;
+}
+
+// The steps the kernel variants make for a wish of `steps`: 2 or 4 with the activations in registers, else a
+// multiple of 4.
+static int stream_steps_served(int steps) { return steps <= 2 ? 2 : (steps + 3) / 4 * 4; }
+
+// Into how many ranges K is best cut for an [M, K] x [N, K]^T product whose reader can add planes: enough
+// to give every compute unit two or three blocks, no fewer than two steps for a wave, and no range empty.
+static int stream_parts(int M, int N, int K) {
+    const int n_super = (K + SUPER_K - 1) / SUPER_K;
+    if (M > 16 || n_super < 16) return 1;
+    const int strips = (N + 15) / 16;
+    int parts = max(1, min(min(768 / strips, n_super / (2 * STREAM_WAVES)), 4));
+    for (;;) {      // rounding the steps up can leave the last ranges without work: fewer ranges then
+        const int covered = stream_steps_served(stream_steps(n_super, parts)) * STREAM_WAVES;
+        const int needed = (n_super + covered - 1) / covered;
+        if (needed == parts) return parts;
+        parts = needed;
+    }
+}
+
 template <int U, int TREG, typename TC, int EPI>
-static void launch_stream(hipStream_t stream, const void* a, const void* w, void* c, int M, int N, int K) {
+static void launch_stream(hipStream_t stream, const void* a, const void* w, void* c, int M, int N, int K, int parts) {
     const int strips = EPI == EPI_SWIGLU ? (N / 2 + 7) / 8 : (N + 15) / 16;
     const int n_super = (K + SUPER_K - 1) / SUPER_K;
-    int T = (n_super + STREAM_WAVES - 1) / STREAM_WAVES;
+    int T = stream_steps(n_super, parts);
     T = (T + U - 1) / U * U;
     if (TREG > 0) T = TREG;
     // every block the same number of strips, as far as that goes
-    const int rounds = (strips + STREAM_SLOTS - 1) / STREAM_SLOTS;
-    const int grid = (strips + rounds - 1) / rounds;
-    const bool exact = K % SUPER_K == 0 && T * STREAM_WAVES == n_super;
+    const int slots = parts > 1 ? max(1, STREAM_SLOTS_CUT / parts) : STREAM_SLOTS;
+    const int rounds = (strips + slots - 1) / slots;
+    const dim3 grid((strips + rounds - 1) / rounds, parts);
+    const bool exact = K % SUPER_K == 0 && parts * T * STREAM_WAVES == n_super;
     if (exact)
         linear_stream_kernel<U, TREG, true, TC, EPI><<<grid, STREAM_WAVES * WAVE, 0, stream>>>(
             (const bf16_t*)a, (const bf16_t*)w, (TC*)c, M, N, K, strips, T);
@@ -277,14 +311,14 @@ static void launch_stream(hipStream_t stream, const void* a, const void* w, void
 }
 
 template <typename TC, int EPI>
-static void dispatch_thin(hipStream_t stream, const void* a, const void* w, void* c, int M, int N, int K) {
+static void dispatch_thin(hipStream_t stream, const void* a, const void* w, void* c, int M, int N, int K, int parts) {
     const int n_super = (K + SUPER_K - 1) / SUPER_K;
     const bool deep = n_super >= 16;                           // enough super-steps to feed eight waves
     if (M <= 16 && deep) {
-        const int per_wave = (n_super + STREAM_WAVES - 1) / STREAM_WAVES;
-        if (per_wave <= 2) launch_stream<2, 2, TC, EPI>(stream, a, w, c, M, N, K);
-        else if (per_wave <= 4) launch_stream<2, 4, TC, EPI>(stream, a, w, c, M, N, K);
-        else launch_stream<4, 0, TC, EPI>(stream, a, w, c, M, N, K);
+        const int per_wave = stream_steps(n_super, parts);
+        if (per_wave <= 2) launch_stream<2, 2, TC, EPI>(stream, a, w, c, M, N, K, parts);
+        else if (per_wave <= 4) launch_stream<2, 4, TC, EPI>(stream, a, w, c, M, N, K, parts);
+        else launch_stream<4, 0, TC, EPI>(stream, a, w, c, M, N, K, parts);
         return;
     }
     if (M <= 16) {
@@ -300,9 +334,16 @@ static void dispatch_thin(hipStream_t stream, const void* a, const void* w, void
     }
 }
 
+PALM_API int palm_linear_thin_parts(int M, int N, int K) { return stream_parts(M, N, K); }
+
 // a [M, K] bfloat16, w [N, K] bfloat16; c [M, N] (EPI_STORE) or [M, N/2] (EPI_SWIGLU) in bfloat16 or float32.
+// parts > 1 (at most palm_linear_thin_parts(M, N, K), float32, EPI_STORE): c is [parts, M, N] and the product is
+// the sum of its planes.
 PALM_API int palm_linear_thin(hipStream_t stream, const void* a, const void* w, void* c, int c_dtype, int M, int N,
-                              int K, int epilogue) {
+                              int K, int epilogue, int parts) {
+    PALM_CHECK(parts >= 1, "linear_thin: parts = %d", parts);
+    PALM_CHECK(parts == 1 || (epilogue == EPI_STORE && c_dtype == PALM_F32 && parts <= stream_parts(M, N, K)),
+               "linear_thin: %d partial planes are not served for M=%d N=%d K=%d, this epilogue and result type", parts, M, N, K);
     PALM_CHECK(M >= 0 && N > 0 && K > 0, "linear_thin: M=%d N=%d K=%d", M, N, K);
     PALM_CHECK(K % 8 == 0, "linear_thin: K = %d is not a multiple of 8 (rows must start on 16 bytes)", K);
     PALM_CHECK(epilogue == EPI_STORE || epilogue == EPI_SWIGLU, "linear_thin: epilogue %d", epilogue);
@@ -311,9 +352,9 @@ PALM_API int palm_linear_thin(hipStream_t stream, const void* a, const void* w, 
     if (M == 0) return 0;
     PALM_CHECK((M + 63) / 64 <= 65535, "linear_thin: M=%d is more than one launch takes", M);
     if (epilogue == EPI_SWIGLU) {
-        PALM_DTYPE_SWITCH(c_dtype, TC, dispatch_thin<TC, EPI_SWIGLU>(stream, a, w, c, M, N, K));
+        PALM_DTYPE_SWITCH(c_dtype, TC, dispatch_thin<TC, EPI_SWIGLU>(stream, a, w, c, M, N, K, 1));
     } else {
-        PALM_DTYPE_SWITCH(c_dtype, TC, dispatch_thin<TC, EPI_STORE>(stream, a, w, c, M, N, K));
+        PALM_DTYPE_SWITCH(c_dtype, TC, dispatch_thin<TC, EPI_STORE>(stream, a, w, c, M, N, K, parts));
     }
     PALM_LAUNCHED();
     return 0;

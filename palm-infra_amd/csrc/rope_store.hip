@@ -17,9 +17,12 @@
 constexpr int MAX_HEAD_DIM = 512;
 
 // One wave per (token, head).  pairing 0: pairs (i, i + rot/2); pairing 1: pairs (2i, 2i + 1).
-template <typename T>
+// qkv may come as `planes` planes of partial sums (a projection that cut its K into ranges), plane_stride
+// elements apart; they are added in their order.
+template <typename TIN, typename T>
 __global__ __launch_bounds__(WAVE) void qk_norm_rope_store_kernel(
-    const T* __restrict__ qkv, T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache,
+    const TIN* __restrict__ qkv, int planes, size_t plane_stride,
+    T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache,
     const int* __restrict__ block_table, int max_pages, const int* __restrict__ tok_slot,
     const int* __restrict__ positions, const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w,
     float eps, const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rotary_dim, int pairing,
@@ -31,11 +34,12 @@ __global__ __launch_bounds__(WAVE) void qk_norm_rope_store_kernel(
     const int lane = threadIdx.x;
     const int kind = head < nh ? 0 : (head < nh + nkv ? 1 : 2);
     if (kind != 0 && !write_cache) return;
-    const T* src = qkv + ((size_t)t * (nh + 2 * nkv) + head) * hd;
+    const TIN* src = qkv + ((size_t)t * (nh + 2 * nkv) + head) * hd;
 
     float ss = 0.f;
     for (int d = lane; d < hd; d += WAVE) {
-        const float v = to_float(src[d]);
+        float v = to_float(src[d]);
+        for (int p = 1; p < planes; ++p) v += to_float(src[p * plane_stride + d]);
         vals[d] = v;
         ss += v * v;
     }
@@ -79,7 +83,9 @@ __global__ __launch_bounds__(WAVE) void qk_norm_rope_store_kernel(
     for (int d = lane; d < hd; d += WAVE) dst[d] = from_float<T>(vals[d]);
 }
 
-PALM_API int palm_qk_norm_rope_store(hipStream_t stream, const void* qkv, int dtype, void* q_out, void* k_cache,
+// dtype: the element type of q_out and of the cache, and of qkv if planes == 1; with planes > 1 qkv is
+// [planes, n_tokens, (nh + 2 nkv) * hd] float32.
+PALM_API int palm_qk_norm_rope_store(hipStream_t stream, const void* qkv, int dtype, int planes, void* q_out, void* k_cache,
                                      void* v_cache, const int* block_table, int max_pages, const int* tok_slot,
                                      const int* positions, const float* q_norm_w, const float* k_norm_w, float eps,
                                      const float* cos_t, const float* sin_t, int rotary_dim, int pairing,
@@ -93,13 +99,22 @@ PALM_API int palm_qk_norm_rope_store(hipStream_t stream, const void* qkv, int dt
     PALM_CHECK((cos_t == nullptr) == (sin_t == nullptr), "qk_norm_rope_store: cos and sin tables come together");
     PALM_CHECK(!write_cache || (k_cache && v_cache && block_table && tok_slot && max_pages > 0),
                "qk_norm_rope_store: a cache write needs the cache, the page table and the slots");
+    PALM_CHECK(planes >= 1, "qk_norm_rope_store: %d planes", planes);
     if (n_tokens == 0) return 0;
     dim3 grid(n_tokens, nh + 2 * nkv);
     PALM_CHECK(grid.y <= 65535, "qk_norm_rope_store: %d heads are more than one launch takes", (int)grid.y);
-    PALM_DTYPE_SWITCH(dtype, T,
-        qk_norm_rope_store_kernel<T><<<grid, WAVE, 0, stream>>>(
-            (const T*)qkv, (T*)q_out, (T*)k_cache, (T*)v_cache, block_table, max_pages, tok_slot, positions,
-            q_norm_w, k_norm_w, eps, cos_t, sin_t, rotary_dim, pairing, nh, nkv, hd, write_cache));
+    const size_t plane_stride = (size_t)n_tokens * (nh + 2 * nkv) * hd;
+    if (planes > 1) {
+        PALM_DTYPE_SWITCH(dtype, T,
+            (qk_norm_rope_store_kernel<float, T><<<grid, WAVE, 0, stream>>>(
+                (const float*)qkv, planes, plane_stride, (T*)q_out, (T*)k_cache, (T*)v_cache, block_table, max_pages,
+                tok_slot, positions, q_norm_w, k_norm_w, eps, cos_t, sin_t, rotary_dim, pairing, nh, nkv, hd, write_cache)));
+    } else {
+        PALM_DTYPE_SWITCH(dtype, T,
+            (qk_norm_rope_store_kernel<T, T><<<grid, WAVE, 0, stream>>>(
+                (const T*)qkv, 1, plane_stride, (T*)q_out, (T*)k_cache, (T*)v_cache, block_table, max_pages,
+                tok_slot, positions, q_norm_w, k_norm_w, eps, cos_t, sin_t, rotary_dim, pairing, nh, nkv, hd, write_cache)));
+    }
     PALM_LAUNCHED();
     return 0;
 }

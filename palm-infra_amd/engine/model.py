@@ -49,6 +49,8 @@ class DecoderModel:
         pending = None
         for i, call in enumerate(self.order):
             ctx.layer_cache = cache.layer_caches[i]
+            reader = self.layers[self.order[i + 1].layer] if i + 1 < len(self.order) else self.final_norm
+            ctx.next_takes_planes = bool(getattr(reader, "takes_planes", False))
             x, pending = self.layers[call.layer].forward(x, pending, ctx)
         ctx.layer_cache = None
         h = self.final_norm(x, delta=pending, rows=want_rows)

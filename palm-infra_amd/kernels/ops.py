@@ -20,18 +20,19 @@ PAGE_TOKENS = 64
 
 _SIGNATURES = {
     "palm_embed": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_void_p],
-    "palm_rmsnorm": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_float, c_void_p, c_int, c_int,
-                     c_void_p, c_int, c_int],
+    "palm_rmsnorm": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p, c_float, c_void_p, c_int, c_int,
+                     c_void_p, c_int, c_int, c_longlong],
     "palm_swiglu": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int],
     "palm_cast": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_longlong],
     "palm_linear": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int],
-    "palm_qk_norm_rope_store": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
+    "palm_qk_norm_rope_store": [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                                 c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                                 c_int, c_int, c_int],
     "palm_rope_table": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int],
     "palm_attention_simple": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                               c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
-    "palm_linear_thin": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int],
+    "palm_linear_thin": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int],
+    "palm_linear_thin_parts": [c_int, c_int, c_int],
     "palm_linear_wide": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "palm_linear_wide_splits": [c_int, c_int, c_int, c_int],
     "palm_argmax": [c_void_p, c_void_p, c_int, c_int, c_void_p],
@@ -117,20 +118,27 @@ def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor | None = Non
 def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.dtype, delta: torch.Tensor | None = None,
             update_x: bool = False, rows: torch.Tensor | None = None) -> torch.Tensor:
     """out[r] = norm(x[src] + delta[src]) * weight, src = rows[r] or r; with update_x the sum is written
-    back to x (the residual stream).  x is [n, width]; statistics in float32."""
+    back to x (the residual stream).  x is [n, width]; statistics in float32.  delta may also be float32
+    planes [P, n, width], which are added one after the other."""
     _dev("rmsnorm", x, weight, delta, rows)
     _i32("rmsnorm", rows)
     _need(x.dim() == 2, f"rmsnorm: x {tuple(x.shape)} is not [rows, width]")
     n, width = x.shape
     _need(weight.shape == (width,) and weight.dtype == F32, f"rmsnorm: weight {tuple(weight.shape)} {weight.dtype}, "
           f"width {width} (norm weights are float32)")
-    _need(delta is None or delta.shape == x.shape, "rmsnorm: delta and x differ in shape")
+    planes = 1
+    if delta is not None and delta.dim() == 3:
+        planes = delta.shape[0]
+        _need(delta.dtype == F32 and delta.shape[1:] == x.shape and delta.is_contiguous(),
+              f"rmsnorm: delta planes {tuple(delta.shape)} {delta.dtype} for x {tuple(x.shape)} (planes are contiguous float32)")
+    else:
+        _need(delta is None or delta.shape == x.shape, "rmsnorm: delta and x differ in shape")
     _need(not update_x or (delta is not None and rows is None), "rmsnorm: update_x needs a delta and no row selection")
     n_out = n if rows is None else rows.shape[0]
     out = torch.empty((n_out, width), dtype=out_dtype, device=x.device)
     library.call(core(), "palm_rmsnorm", _stream(), _p(x), _code(x, "rmsnorm x"), _p(delta),
-                 _code(delta, "rmsnorm delta") if delta is not None else 0, _p(weight), float(eps), _p(rows), n_out, width,
-                 _p(out), _code(out, "rmsnorm out"), int(update_x))
+                 _code(delta, "rmsnorm delta") if delta is not None else 0, planes, _p(weight), float(eps), _p(rows), n_out, width,
+                 _p(out), _code(out, "rmsnorm out"), int(update_x), n)
     return out
 
 
@@ -184,13 +192,25 @@ def _check_cache(what, k_cache, v_cache, block_table, nkv, hd):
 
 def qk_norm_rope_store(qkv: torch.Tensor, nh: int, nkv: int, hd: int, positions: torch.Tensor, *, q_norm_w=None,
                        k_norm_w=None, eps: float = 0.0, cos=None, sin=None, rotary_dim: int = 0, pairing: int = 0,
-                       k_cache=None, v_cache=None, block_table=None, tok_slot=None, write_cache: bool = True) -> torch.Tensor:
+                       k_cache=None, v_cache=None, block_table=None, tok_slot=None, write_cache: bool = True,
+                       out_dtype: torch.dtype | None = None) -> torch.Tensor:
     """qkv [n, (nh + 2 nkv) hd] -> q [n, nh hd], normed and rotated by the cos/sin rows [n, rotary_dim/2];
-    k (normed, rotated) and v go to the cache page of (tok_slot[t], positions[t])."""
+    k (normed, rotated) and v go to the cache page of (tok_slot[t], positions[t]).  qkv may also be float32
+    planes [P, n, (nh + 2 nkv) hd] to be added up; ``out_dtype`` then names the type of q and of the cache."""
     _dev("qk_norm_rope_store", qkv, positions, q_norm_w, k_norm_w, cos, sin, k_cache, v_cache, block_table, tok_slot)
     _i32("qk_norm_rope_store", positions, block_table, tok_slot)
-    n = qkv.shape[0]
-    _need(qkv.dim() == 2 and qkv.shape[1] == (nh + 2 * nkv) * hd, f"qk_norm_rope_store: qkv {tuple(qkv.shape)} is not "
+    planes = 1
+    if qkv.dim() == 3:
+        planes = qkv.shape[0]
+        _need(qkv.dtype == F32 and qkv.is_contiguous() and out_dtype is not None,
+              "qk_norm_rope_store: planes are contiguous float32 and come with the type of the result")
+        n = qkv.shape[1]
+    else:
+        _need(qkv.dim() == 2, f"qk_norm_rope_store: qkv {tuple(qkv.shape)}")
+        n = qkv.shape[0]
+        out_dtype = out_dtype or qkv.dtype
+        _need(out_dtype == qkv.dtype, "qk_norm_rope_store: q and the cache have the type of qkv unless qkv comes in planes")
+    _need(qkv.shape[-1] == (nh + 2 * nkv) * hd, f"qk_norm_rope_store: qkv {tuple(qkv.shape)} is not "
           f"[n, ({nh} + 2*{nkv}) * {hd}]")
     _need(positions.shape == (n,), "qk_norm_rope_store: one position for each token")
     for w, nm in ((q_norm_w, "q"), (k_norm_w, "k")):
@@ -206,11 +226,11 @@ def qk_norm_rope_store(qkv: torch.Tensor, nh: int, nkv: int, hd: int, positions:
         _need(k_cache is not None and v_cache is not None and block_table is not None and tok_slot is not None,
               "qk_norm_rope_store: writing the cache needs cache, page table and slots")
         _check_cache("qk_norm_rope_store", k_cache, v_cache, block_table, nkv, hd)
-        _need(k_cache.dtype == qkv.dtype, f"qk_norm_rope_store: cache is {k_cache.dtype}, activations are {qkv.dtype}")
+        _need(k_cache.dtype == out_dtype, f"qk_norm_rope_store: cache is {k_cache.dtype}, activations are {out_dtype}")
         _need(tok_slot.shape == (n,), "qk_norm_rope_store: one slot for each token")
         max_pages = block_table.shape[1]
-    q_out = torch.empty((n, nh * hd), dtype=qkv.dtype, device=qkv.device)
-    library.call(core(), "palm_qk_norm_rope_store", _stream(), _p(qkv), _code(qkv, "qkv"), _p(q_out), _p(k_cache), _p(v_cache),
+    q_out = torch.empty((n, nh * hd), dtype=out_dtype, device=qkv.device)
+    library.call(core(), "palm_qk_norm_rope_store", _stream(), _p(qkv), _code(q_out, "qkv"), planes, _p(q_out), _p(k_cache), _p(v_cache),
                  _p(block_table), max_pages, _p(tok_slot), _p(positions), _p(q_norm_w), _p(k_norm_w), float(eps),
                  _p(cos), _p(sin), int(rotary_dim if cos is not None else 0), int(pairing), n, nh, nkv, hd, int(write_cache))
     return q_out
@@ -303,10 +323,15 @@ def thin_serves(a: torch.Tensor, w: torch.Tensor) -> bool:
     return a.dtype == BF16 and w.dtype == BF16 and a.shape[1] % 8 == 0
 
 
-def linear_thin(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, gated: bool = False) -> torch.Tensor:
+def linear_thin(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, gated: bool = False,
+                planes_ok: bool = False) -> torch.Tensor:
     """bfloat16 a [M, K] . w [N, K]^T on the matrix cores, the weight streamed once per 64 rows of a;
     result [M, N] in bfloat16 or float32.  With ``gated`` w is [gate rows | up rows] and the result is
-    silu(a gate^T) * (a up^T), [M, N/2]."""
+    silu(a gate^T) * (a up^T), [M, N/2].
+
+    ``planes_ok``: the caller can take the product as float32 planes [P, M, N] whose sum (in the order of the
+    planes) it is: for a few rows and few weight rows the kernel then cuts K into P ranges to fill the chip.
+    rmsnorm's ``delta`` and qk_norm_rope_store's ``qkv`` take such planes."""
     if not thin_serves(a, w):
         out = linear_exact(a, w, out_dtype)
         return swiglu(out) if gated else out
@@ -318,8 +343,11 @@ def linear_thin(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, gated:
     _need(not gated or N % 2 == 0, f"linear_thin: a gated product needs an even number of weight rows, got {N}")
     out = torch.empty((M, N // 2 if gated else N), dtype=out_dtype, device=a.device)
     if M <= THIN_TOKENS:
+        planes = core().palm_linear_thin_parts(M, N, K) if planes_ok and not gated else 1
+        if planes > 1:
+            out = torch.empty((planes, M, N), dtype=F32, device=a.device)
         library.call(core(), "palm_linear_thin", _stream(), _p(a), _p(w), _p(out), _code(out, "linear_thin out"), M, N, K,
-                     1 if gated else 0)
+                     1 if gated else 0, planes)
         return out
     # more rows than one block of 16: the kernel that shares the activations through LDS, K split if need be
     splits = core().palm_linear_wide_splits(M, N, K, 1 if gated else 0)

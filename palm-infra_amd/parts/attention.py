@@ -56,7 +56,7 @@ class Attention:
         lc = ctx.layer_cache
         if lc is None or lc.kv is None:
             raise RuntimeError("attention needs the keys and values of its layer; the step gave it no cache")
-        qkv = self.qkv(h)
+        qkv = self.qkv(h, planes_ok=True)
         tables = self.position.tables(ctx) if self.position is not None else None
         cos, sin = tables if tables is not None else (None, None)
         q = ops.qk_norm_rope_store(
@@ -65,6 +65,7 @@ class Attention:
             eps=self.q_norm.eps if self.q_norm else 0.0, cos=cos, sin=sin,
             rotary_dim=self.position.rotary_dim if tables is not None else 0,
             pairing=PAIRINGS[self.position.pairing] if tables is not None else 0,
-            k_cache=lc.k, v_cache=lc.v, block_table=lc.kv.table_dev, tok_slot=ctx.tok_slot, write_cache=lc.writes)
+            k_cache=lc.k, v_cache=lc.v, block_table=lc.kv.table_dev, tok_slot=ctx.tok_slot, write_cache=lc.writes,
+            out_dtype=h.dtype)
         o = ops.attention(q, lc.k, lc.v, lc.kv.table_dev, ctx, self.nh, self.nkv, self.hd, self.scale, self.window)
-        return self.out(o)
+        return self.out(o, planes_ok=bool(getattr(ctx, "planes_ok", False)))

@@ -89,6 +89,8 @@ class StepContext:
     is_decode: bool = False      # every sequence brings exactly one token
     decode_slices: int = 0       # if set: into how many slices decode attention cuts a key range (else chosen per call)
     layer_cache: object = None   # the LayerCache of the run-order entry that is running
+    planes_ok: bool = False      # the reader of the running branch's output adds float32 planes [P, n, width]
+    next_takes_planes: bool = False   # the same for what the running layer hands on as pending (set by the model)
     memo: dict = field(default_factory=dict)   # what parts make once per step (rotation tables)
     host: dict = field(default_factory=dict)   # the same facts as Python lists, for parts that plan on the host
 

@@ -22,4 +22,4 @@ class GatedSiluFeedForward:
                              f"do not fit hidden {self.hidden}, intermediate {self.inter}")
 
     def forward(self, h: torch.Tensor, ctx) -> torch.Tensor:
-        return self.down(self.gate_up.gated(h))
+        return self.down(self.gate_up.gated(h), planes_ok=bool(getattr(ctx, "planes_ok", False)))

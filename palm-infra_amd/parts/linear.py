@@ -22,12 +22,15 @@ class Linear:
         self.weight = weight
         self.out_features, self.in_features = weight.shape
 
-    def __call__(self, x: torch.Tensor, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+    def __call__(self, x: torch.Tensor, out_dtype: torch.dtype | None = None, planes_ok: bool = False) -> torch.Tensor:
+        """``planes_ok``: the caller hands the result to a reader that adds float32 planes [P, n, out] (a norm's
+        ``delta``, the q/k/v of qk_norm_rope_store); a thin product with few weight rows may then come as such
+        planes, each the sum over one range of the inner size."""
         out_dtype = out_dtype or x.dtype
         w = self.weight
         if x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16:
             if x.shape[0] <= THIN_ROWS or out_dtype != torch.bfloat16:
-                return ops.linear_thin(x, w, out_dtype)
+                return ops.linear_thin(x, w, out_dtype, planes_ok=planes_ok)
             return ops.linear_library(x, w)
         return ops.linear_exact(x, w, out_dtype)
 

@@ -12,6 +12,7 @@ from .base import register_part
 @register_part("norm", "rms")
 class RMSNorm:
     capturable = True      # launches the same kernels whatever the step holds: may be recorded into a HIP graph
+    takes_planes = True    # ``delta`` may be float32 planes [P, n, width], added one after the other
 
     def __init__(self, spec, builder):
         self.width = int(spec.params["width"])

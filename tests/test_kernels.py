@@ -68,6 +68,51 @@ def test_rmsnorm_adds_the_pending_branch_in_32_bit(ops, out_dtype, delta_dtype):
     assert torch.allclose(sel.double(), P.rms_norm(x.double() + d.double(), w, 1e-5)[[6, 0, 3]], atol=2e-5)
 
 
+@pytest.mark.parametrize("planes", [2, 3, 4])
+@pytest.mark.parametrize("width", [96, 4096, 5000])
+def test_rmsnorm_adds_planes_of_partial_sums_in_their_order(ops, planes, width):
+    x, w = rand(5, width, seed=2), rand(width, seed=4) + 1.0
+    d = rand(planes, 5, width, seed=3) * torch.tensor([1.0, 1e3, 1e-3, 7.0])[:planes, None, None]   # the order of the sum shows
+    want_x = x.clone()
+    for p in range(planes):
+        want_x = want_x + d[p]
+    xd = x.to(DEV)
+    got = ops.rmsnorm(xd, w.to(DEV), 1e-5, BF16, delta=d.to(DEV), update_x=True).cpu()
+    assert torch.equal(xd.cpu(), want_x)
+    assert torch.allclose(got.double(), P.rms_norm(want_x.double(), w, 1e-5), atol=2e-2, rtol=1e-2)
+    rows = torch.tensor([4, 0], dtype=torch.int32).to(DEV)
+    sel = ops.rmsnorm(x.to(DEV), w.to(DEV), 1e-5, F32, delta=d.to(DEV), rows=rows).cpu()
+    assert torch.allclose(sel.double(), P.rms_norm(want_x.double(), w, 1e-5)[[4, 0]], atol=1e-4)
+    with pytest.raises(Exception, match="planes"):
+        ops.rmsnorm(x.to(DEV), w.to(DEV), 1e-5, F32, delta=torch.zeros(5, 5, width, device=DEV))
+    with pytest.raises(Exception, match="planes"):
+        ops.rmsnorm(x.to(DEV), w.to(DEV), 1e-5, F32, delta=torch.zeros(2, 5, width, device=DEV, dtype=BF16))
+
+
+def test_qk_norm_rope_store_adds_planes(ops):
+    nh, nkv, hd, n = 6, 2, 80, 5
+    planes = rand(3, n, (nh + 2 * nkv) * hd, seed=11)
+    whole = (planes[0] + planes[1]) + planes[2]
+    qw, kw = rand(hd, seed=1) + 1.0, rand(hd, seed=2) + 1.0
+    pos = torch.arange(60, 60 + n, dtype=torch.int32).to(DEV)
+    table = torch.tensor([[2, 1]], dtype=torch.int32).to(DEV)
+    slot = torch.zeros(n, dtype=torch.int32).to(DEV)
+    inv = torch.from_numpy((1.0 / np.power(np.float32(1e4), 2.0 * np.arange(hd // 2, dtype=np.float32) / hd)).astype(np.float32))
+    cos, sin = ops.rope_table(pos, inv.to(DEV))
+    results = []
+    for qkv, kw_extra in ((whole.to(BF16).to(DEV), {}), (planes.to(DEV), {"out_dtype": BF16})):
+        kc, vc = _paged(4, nkv, hd, BF16)
+        q = ops.qk_norm_rope_store(qkv, nh, nkv, hd, pos, q_norm_w=qw.to(DEV), k_norm_w=kw.to(DEV), eps=1e-6, cos=cos, sin=sin,
+                                   rotary_dim=hd, pairing=0, k_cache=kc, v_cache=vc, block_table=table, tok_slot=slot, **kw_extra)
+        results.append((q.cpu().float(), kc.cpu().float(), vc.cpu().float()))
+    # the planes are added in 32-bit, the single input was rounded to bfloat16 first: equal within that rounding
+    for a, b in zip(*results):
+        assert torch.allclose(a, b, atol=6e-2, rtol=2e-2)
+    assert float(results[1][1].abs().max()) > 0.5
+    with pytest.raises(Exception, match="planes"):
+        ops.qk_norm_rope_store(planes.to(DEV), nh, nkv, hd, pos, write_cache=False)
+
+
 @pytest.mark.parametrize("dtype", [F32, BF16])
 def test_swiglu(ops, dtype):
     gu = rand(9, 2 * 176, seed=5, scale=3.0, dtype=dtype)

@@ -1,5 +1,7 @@
 """The matrix-core kernels alone against their plain references: the thin linear product (with and
 without the gated epilogue) and the bfloat16 attention kernels, at sizes other than the tiny models'."""
+import math
+
 import pytest
 import torch
 
@@ -31,6 +33,24 @@ def test_linear_thin_against_the_plain_product(ops, M, N, K):
     assert torch.allclose(got32.double(), ref, atol=2e-4 * (K ** 0.5), rtol=1e-5), float((got32.double() - ref).abs().max())
     got16 = ops.linear_thin(a.to(DEV), w.to(DEV), BF16).cpu()
     assert torch.equal(got16, got32.to(BF16))                          # one rounding at the end
+
+
+@pytest.mark.parametrize("M", [1, 8, 16])
+@pytest.mark.parametrize("N,K,planes", [(4096, 4096, 2), (2048, 12288, 3), (1000, 12288, 3), (6144, 4096, 2), (4096, 6000, 2),
+                                        (4096, 2048, 1), (16384, 4096, 1), (515, 520, 1)])
+def test_linear_thin_as_planes_of_partial_sums(ops, M, N, K, planes):
+    a, w = rand(M, K, seed=M, dtype=BF16), rand(N, K, seed=N + K, dtype=BF16)
+    got = ops.linear_thin(a.to(DEV), w.to(DEV), F32, planes_ok=True).cpu()
+    want = P.linear(a, w)
+    if planes == 1:
+        assert got.shape == (M, N)
+    else:
+        assert got.shape == (planes, M, N) and got.dtype == F32
+        assert all(float(got[p].abs().max()) > 0 for p in range(planes))
+        got = got.double().sum(0)
+    assert torch.allclose(got.double(), want, atol=2e-4 * (K ** 0.5), rtol=1e-5)
+    # bfloat16 results and gated products never come in planes
+    assert ops.linear_thin(a.to(DEV), w.to(DEV), BF16, planes_ok=False).shape == (M, N)
 
 
 def test_linear_thin_orientation(ops):
