@@ -34,9 +34,32 @@ __device__ inline BestPair better(BestPair a, BestPair b) {
 // argmax of one row by the whole block; every thread returns the result
 __device__ BestPair block_argmax(const float* __restrict__ row, int V, BestPair* scratch) {
     BestPair best{-INFINITY, 0x7fffffff};
-    for (int i = threadIdx.x; i < V; i += blockDim.x) {
+    // a thread's indices rise, so a tie keeps the lower one: the elements before the first 16-byte border, then
+    // the body four at a time (four reads in flight), then the rest
+    const int head = min(V, (int)(((16 - ((uintptr_t)row & 15)) & 15) / 4));
+    const int n4 = (V - head) / 4;
+    for (int i = threadIdx.x; i < head; i += blockDim.x) {
         const float v = row[i];
-        if (v > best.v) { best.v = v; best.i = i; }      // indices rise, so a tie keeps the lower one
+        if (v > best.v) { best.v = v; best.i = i; }
+    }
+    const float4* body = reinterpret_cast<const float4*>(row + head);
+    for (int i0 = threadIdx.x; i0 < n4; i0 += 4 * blockDim.x) {
+        float4 q[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) q[u] = body[min(i0 + u * (int)blockDim.x, n4 - 1)];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int i4 = i0 + u * (int)blockDim.x;
+            if (i4 >= n4) break;
+            const float e[4] = {q[u].x, q[u].y, q[u].z, q[u].w};
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                if (e[k] > best.v) { best.v = e[k]; best.i = head + 4 * i4 + k; }
+        }
+    }
+    for (int i = head + 4 * n4 + threadIdx.x; i < V; i += blockDim.x) {
+        const float v = row[i];
+        if (v > best.v) { best.v = v; best.i = i; }
     }
     if (best.i == 0x7fffffff && threadIdx.x == 0) best.i = 0;
     for (int off = WAVE / 2; off > 0; off >>= 1) {

@@ -349,6 +349,15 @@ def test_argmax_takes_the_first_maximum(ops):
     got = ops.argmax(lg.to(DEV)).cpu().tolist()
     assert got == [int(lg[0].argmax()), 17, 0, 999, 0, int(lg[5].argmax())]
     assert ops.argmax(torch.tensor([[0.5, 3.0, 2.0]]).to(DEV)).item() == 1       # tests/test_sampler.cpp:26-27
+    # rows that do not start on 16 bytes, a width that is no multiple of four, ties at both ends of a wide row
+    for V in (1003, 151937, 5):
+        lg = rand(5, V, seed=V)
+        lg[1, 2] = lg[1, V - 1] = 70.0
+        lg[2, V - 1] = 70.0
+        lg[3, V - 2] = lg[3, V // 2] = 70.0
+        lg[4, :] = float("-inf")
+        want = [int(lg[0].argmax()), 2, V - 1, min(V - 2, V // 2), 0]
+        assert ops.argmax(lg.to(DEV)).cpu().tolist() == want, V
 
 
 def _sample(ops, lg, u, **kw):
