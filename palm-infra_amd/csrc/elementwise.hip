@@ -189,6 +189,31 @@ PALM_API int palm_rmsnorm(hipStream_t stream, void* x, int x_dtype, const void* 
     return 0;
 }
 
+// Rows that a product left without their norm's factor (linear_mfma.hip, RowNorm): out = a * f(row),
+// f = 1 / sqrt(sum of the row's pieces / width + eps).  Only for a reader that cannot apply the factor itself.
+template <typename T>
+__global__ void scale_rows_kernel(const T* __restrict__ a, const float* __restrict__ ss, int pieces, int n_rows,
+                                  float eps, int width, T* __restrict__ out) {
+    __shared__ float scratch[16];
+    const int r = blockIdx.x;
+    float sum = 0.f;
+    for (int p = threadIdx.x; p < pieces; p += blockDim.x) sum += ss[(size_t)r * pieces + p];
+    sum = block_sum(sum, scratch);
+    const float f = 1.0f / sqrtf(sum / (float)width + eps);
+    for (int d = threadIdx.x; d < width; d += blockDim.x)
+        out[(size_t)r * width + d] = from_float<T>(to_float(a[(size_t)r * width + d]) * f);
+}
+
+PALM_API int palm_scale_rows(hipStream_t stream, const void* a, int dtype, const float* ss, int pieces, int n_rows,
+                             float eps, int width, void* out) {
+    PALM_CHECK(n_rows >= 0 && width > 0 && pieces > 0, "scale_rows: rows=%d width=%d pieces=%d", n_rows, width, pieces);
+    if (n_rows == 0) return 0;
+    PALM_DTYPE_SWITCH(dtype, T,
+        scale_rows_kernel<T><<<n_rows, 256, 0, stream>>>((const T*)a, ss, pieces, n_rows, eps, width, (T*)out));
+    PALM_LAUNCHED();
+    return 0;
+}
+
 // ---- SwiGLU ---------------------------------------------------------------------------------------
 template <typename T>
 __global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int n_rows, int inter) {

@@ -137,6 +137,27 @@ static void launch_thin(hipStream_t stream, const void* a, const void* w, void* 
 // cut into `parts` ranges, blockIdx.y names the range, and the block writes its partial sums to plane
 // blockIdx.y of a [parts, M, N] float32 result; whoever reads the result adds the planes in their order (the
 // norm that follows adds them to the residual stream), so the sum is the same bits every time.
+//
+// The norm around a product can be folded into it (RowNorm), which saves the norm's own kernel in a decode
+// step.  RMSNorm is y = x * f * w with one factor f = 1 / sqrt(mean(x^2) + eps) for the row, so
+// (x * f * w) . W^T = f * ((x * w) . W^T): a product whose activations are x * w, not yet multiplied by f, only
+// has to multiply its result rows by f, and f needs nothing but the row's sum of squares.
+//   out side: the product is a branch's output d.  The block that owns a strip of 16 features adds d to the
+//             residual stream (x += d, each element by exactly one thread), stores x * w_out rounded to
+//             bfloat16 as the next product's activations, and the strip's share of each row's sum of squares
+//             in ss_out[row * strips + strip].
+//   in side:  every block adds up the pieces ss_in[row * pieces + piece] in a fixed order, and multiplies its
+//             results by f(row) before the epilogue.
+struct RowNorm {
+    const float* ss_in;      // [M, pieces_in] or null (a row's pieces side by side: 32 lanes read them in one go)
+    int pieces_in;
+    float eps_in;
+    int width_in;            // the row length the mean is over
+    float* resid;            // [M, N] float32, updated; or null
+    const float* w_out;      // [N]
+    float* ss_out;           // [M, strips]
+};
+
 constexpr int STREAM_WAVES = 8;
 constexpr int STREAM_SLOTS = 512;      // blocks that run at once: two on each of 256 compute units
 constexpr int STREAM_SLOTS_CUT = 768;  // with K cut into ranges a block's work is short: three
@@ -145,11 +166,12 @@ template <int U, int TREG, bool EXACT, typename TC, int EPI>
 __global__ __launch_bounds__(STREAM_WAVES * WAVE) void linear_stream_kernel(const bf16_t* __restrict__ A,
                                                                             const bf16_t* __restrict__ W,
                                                                             TC* __restrict__ C, int M, int N, int K,
-                                                                            int n_strips, int T_given) {
+                                                                            int n_strips, int T_given, RowNorm norm) {
     // this block's range of K starts at super-step blockIdx.y * T * NW, its results go to plane blockIdx.y
     constexpr int NW = STREAM_WAVES;
     constexpr bool AREG = TREG > 0;
     __shared__ float part[2][NW][16][17];
+    __shared__ float row_factor[16];
     const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
     const int r = lane % 16, g = lane / 16;
     const int inter = N / 2;
@@ -205,10 +227,39 @@ __global__ __launch_bounds__(STREAM_WAVES * WAVE) void linear_stream_kernel(cons
         }
     }
 
+    __builtin_amdgcn_sched_barrier(0);       // the weight reads above go out first, whatever follows
+    // The rows' factors: 32 threads a row add up the pieces, every block in the same order.  The reads go out
+    // here and are used only when the first strip's products are done, so nothing waits for them.
+    const int f_col = min((int)threadIdx.x / 32, M - 1), f_piece = threadIdx.x % 32;
+    float piece[8];
+    if (norm.ss_in) {
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            piece[u] = norm.ss_in[(size_t)f_col * norm.pieces_in + min(f_piece + 32 * u, norm.pieces_in - 1)];
+    }
+    auto publish_row_factors = [&]() {
+        float sum = 0.f;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) sum += f_piece + 32 * u < norm.pieces_in ? piece[u] : 0.f;
+        for (int p = 256 + f_piece; p < norm.pieces_in; p += 32) sum += norm.ss_in[(size_t)f_col * norm.pieces_in + p];
+#pragma unroll
+        for (int off = 16; off > 0; off >>= 1) sum += __shfl_xor(sum, off, WAVE);
+        if (f_piece == 0) row_factor[threadIdx.x / 32] = 1.0f / sqrtf(sum / (float)norm.width_in + norm.eps_in);
+    };
+
     int buf = 0;
     for (int strip = blockIdx.x; strip < n_strips; strip += gridDim.x) {
         f32x4 acc = {0.f, 0.f, 0.f, 0.f};
         const bool last = strip + (int)gridDim.x >= n_strips;
+        // the residual element this thread will add to, asked for before the strip's products
+        float x_old = 0.f, w_next = 0.f;
+        if (EPI == EPI_STORE && norm.resid && threadIdx.x < 256) {
+            const int feat = strip * 16 + threadIdx.x % 16, col = threadIdx.x / 16;
+            if (col < M && feat < N) {
+                x_old = norm.resid[(size_t)col * N + feat];
+                w_next = norm.w_out[feat];
+            }
+        }
         // U steps: use each slot and, if `refill`, ask for the step U ahead into it
         auto steps = [&](int t, auto refill) {
 #pragma unroll
@@ -241,6 +292,7 @@ __global__ __launch_bounds__(STREAM_WAVES * WAVE) void linear_stream_kernel(cons
         // partial tiles of the waves are added in a fixed order; two buffers, so one barrier a strip is enough
 #pragma unroll
         for (int i = 0; i < 4; ++i) part[buf][wave][4 * g + i][r] = acc[i];
+        if (norm.ss_in && strip == (int)blockIdx.x) publish_row_factors();
         __syncthreads();
         if (EPI == EPI_SWIGLU) {
             if (threadIdx.x < 128) {
@@ -248,6 +300,7 @@ __global__ __launch_bounds__(STREAM_WAVES * WAVE) void linear_stream_kernel(cons
                 float gate = 0.f, up = 0.f;
 #pragma unroll
                 for (int w = 0; w < NW; ++w) { gate += part[buf][w][c][col]; up += part[buf][w][c + 8][col]; }
+                if (norm.ss_in) { gate *= row_factor[col]; up *= row_factor[col]; }
                 const int feat = strip * 8 + c;
                 if (col < M && feat < inter) C[(size_t)col * inter + feat] = from_float<TC>(gate / (1.0f + expf(-gate)) * up);
             }
@@ -257,8 +310,22 @@ __global__ __launch_bounds__(STREAM_WAVES * WAVE) void linear_stream_kernel(cons
                 float v = 0.f;
 #pragma unroll
                 for (int w = 0; w < NW; ++w) v += part[buf][w][row][col];
+                if (norm.ss_in) v *= row_factor[col];
                 const int feat = strip * 16 + row;
-                if (col < M && feat < N) C[(size_t)col * N + feat] = from_float<TC>(v);
+                const bool mine = col < M && feat < N;
+                if (norm.resid) {
+                    const float x_new = x_old + v;
+                    if (mine) {
+                        norm.resid[(size_t)col * N + feat] = x_new;
+                        C[(size_t)col * N + feat] = from_float<TC>(x_new * w_next);
+                    }
+                    float sq = mine ? x_new * x_new : 0.f;          // the 16 features of a row sit in 16 lanes side by side
+#pragma unroll
+                    for (int off = 8; off > 0; off >>= 1) sq += __shfl_xor(sq, off, WAVE);
+                    if (row == 0 && col < M) norm.ss_out[(size_t)col * n_strips + strip] = sq;
+                } else if (mine) {
+                    C[(size_t)col * N + feat] = from_float<TC>(v);
+                }
             }
         }
         buf ^= 1;
@@ -291,7 +358,8 @@ static int stream_parts(int M, int N, int K) {
 }
 
 template <int U, int TREG, typename TC, int EPI>
-static void launch_stream(hipStream_t stream, const void* a, const void* w, void* c, int M, int N, int K, int parts) {
+static void launch_stream(hipStream_t stream, const void* a, const void* w, void* c, int M, int N, int K, int parts,
+                          const RowNorm& norm) {
     const int strips = EPI == EPI_SWIGLU ? (N / 2 + 7) / 8 : (N + 15) / 16;
     const int n_super = (K + SUPER_K - 1) / SUPER_K;
     int T = stream_steps(n_super, parts);
@@ -304,21 +372,23 @@ static void launch_stream(hipStream_t stream, const void* a, const void* w, void
     const bool exact = K % SUPER_K == 0 && parts * T * STREAM_WAVES == n_super;
     if (exact)
         linear_stream_kernel<U, TREG, true, TC, EPI><<<grid, STREAM_WAVES * WAVE, 0, stream>>>(
-            (const bf16_t*)a, (const bf16_t*)w, (TC*)c, M, N, K, strips, T);
+            (const bf16_t*)a, (const bf16_t*)w, (TC*)c, M, N, K, strips, T, norm);
     else
         linear_stream_kernel<U, TREG, false, TC, EPI><<<grid, STREAM_WAVES * WAVE, 0, stream>>>(
-            (const bf16_t*)a, (const bf16_t*)w, (TC*)c, M, N, K, strips, T);
+            (const bf16_t*)a, (const bf16_t*)w, (TC*)c, M, N, K, strips, T, norm);
 }
 
 template <typename TC, int EPI>
-static void dispatch_thin(hipStream_t stream, const void* a, const void* w, void* c, int M, int N, int K, int parts) {
+static void dispatch_thin(hipStream_t stream, const void* a, const void* w, void* c, int M, int N, int K, int parts,
+                          const RowNorm& norm) {
     const int n_super = (K + SUPER_K - 1) / SUPER_K;
     const bool deep = n_super >= 16;                           // enough super-steps to feed eight waves
-    if (M <= 16 && deep) {
+    const bool folded = norm.ss_in || norm.resid;              // only the stream kernel folds a norm in
+    if (M <= 16 && (deep || folded)) {
         const int per_wave = stream_steps(n_super, parts);
-        if (per_wave <= 2) launch_stream<2, 2, TC, EPI>(stream, a, w, c, M, N, K, parts);
-        else if (per_wave <= 4) launch_stream<2, 4, TC, EPI>(stream, a, w, c, M, N, K, parts);
-        else launch_stream<4, 0, TC, EPI>(stream, a, w, c, M, N, K, parts);
+        if (per_wave <= 2) launch_stream<2, 2, TC, EPI>(stream, a, w, c, M, N, K, parts, norm);
+        else if (per_wave <= 4) launch_stream<2, 4, TC, EPI>(stream, a, w, c, M, N, K, parts, norm);
+        else launch_stream<4, 0, TC, EPI>(stream, a, w, c, M, N, K, parts, norm);
         return;
     }
     if (M <= 16) {
@@ -339,9 +409,18 @@ PALM_API int palm_linear_thin_parts(int M, int N, int K) { return stream_parts(M
 // a [M, K] bfloat16, w [N, K] bfloat16; c [M, N] (EPI_STORE) or [M, N/2] (EPI_SWIGLU) in bfloat16 or float32.
 // parts > 1 (at most palm_linear_thin_parts(M, N, K), float32, EPI_STORE): c is [parts, M, N] and the product is
 // the sum of its planes.
+// ss_in (with pieces_in, eps_in, width_in = K) and resid (with w_out, ss_out) fold a norm in, see RowNorm; both
+// need M <= 16, resid needs EPI_STORE, parts == 1 and a bfloat16 c, which then holds the next activations.
 PALM_API int palm_linear_thin(hipStream_t stream, const void* a, const void* w, void* c, int c_dtype, int M, int N,
-                              int K, int epilogue, int parts) {
+                              int K, int epilogue, int parts, const float* ss_in, int pieces_in, float eps_in,
+                              float* resid, const float* w_out, float* ss_out) {
     PALM_CHECK(parts >= 1, "linear_thin: parts = %d", parts);
+    RowNorm norm{ss_in, pieces_in, eps_in, K, resid, w_out, ss_out};
+    PALM_CHECK(!(ss_in || resid) || M <= 16, "linear_thin: a norm is folded in for at most 16 rows, not %d", M);
+    PALM_CHECK(!ss_in || pieces_in > 0, "linear_thin: %d pieces of the rows' sums of squares", pieces_in);
+    PALM_CHECK(!resid || (epilogue == EPI_STORE && parts == 1 && c_dtype == PALM_BF16 && w_out && ss_out),
+               "linear_thin: adding to the residual stream needs a plain bfloat16 product in one plane, the next norm's "
+               "weight and room for the sums of squares");
     PALM_CHECK(parts == 1 || (epilogue == EPI_STORE && c_dtype == PALM_F32 && parts <= stream_parts(M, N, K)),
                "linear_thin: %d partial planes are not served for M=%d N=%d K=%d, this epilogue and result type", parts, M, N, K);
     PALM_CHECK(M >= 0 && N > 0 && K > 0, "linear_thin: M=%d N=%d K=%d", M, N, K);
@@ -352,9 +431,9 @@ PALM_API int palm_linear_thin(hipStream_t stream, const void* a, const void* w, 
     if (M == 0) return 0;
     PALM_CHECK((M + 63) / 64 <= 65535, "linear_thin: M=%d is more than one launch takes", M);
     if (epilogue == EPI_SWIGLU) {
-        PALM_DTYPE_SWITCH(c_dtype, TC, dispatch_thin<TC, EPI_SWIGLU>(stream, a, w, c, M, N, K, 1));
+        PALM_DTYPE_SWITCH(c_dtype, TC, dispatch_thin<TC, EPI_SWIGLU>(stream, a, w, c, M, N, K, 1, norm));
     } else {
-        PALM_DTYPE_SWITCH(c_dtype, TC, dispatch_thin<TC, EPI_STORE>(stream, a, w, c, M, N, K, parts));
+        PALM_DTYPE_SWITCH(c_dtype, TC, dispatch_thin<TC, EPI_STORE>(stream, a, w, c, M, N, K, parts, norm));
     }
     PALM_LAUNCHED();
     return 0;

@@ -192,8 +192,7 @@ class Engine:
             ctx = StepContext(n_tokens=Bb, n_seqs=Bb, max_new=1, max_total=key[1], dtype=self.dtype, token_ids=v[0],
                               positions=v[1], tok_slot=v[2], seq_slot=v[2], seq_start=v[3], seq_new=v[4],
                               cu_new=buf[5 * Bb:], is_decode=True)
-            rows = torch.arange(Bb, dtype=torch.int32).to(self.device)
-            state = self._decode_graphs[key] = {"buf": buf, "ctx": ctx, "rows": rows, "graph": None, "logits": None,
+            state = self._decode_graphs[key] = {"buf": buf, "ctx": ctx, "rows": None, "graph": None, "logits": None,
                                                 "calls": 0}
         state["buf"].copy_(torch.tensor(meta, dtype=torch.int32))
         ctx = state["ctx"]

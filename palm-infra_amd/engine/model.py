@@ -9,7 +9,7 @@ from __future__ import annotations
 import torch
 
 from ..config.spec import ModelSpec
-from ..parts import Builder, cache_needs
+from ..parts import Builder, ResidualSink, cache_needs
 
 
 class DecoderModel:
@@ -46,12 +46,17 @@ class DecoderModel:
         """Run the step's tokens through all layers; logits (float32) at the rows ``want_rows`` of the
         packed tokens (all rows if None)."""
         x = self.embedding.forward(ctx.token_ids)
-        pending = None
+        if not self.order:
+            return self.head.forward(self.final_norm(x, rows=want_rows))
+        # a layer gets its first norm's output and returns the output of the norm after it: the next layer's
+        # first norm, at the end the final norm over the wanted rows
+        h = self.layers[self.order[0].layer].entry_norm(x)
         for i, call in enumerate(self.order):
             ctx.layer_cache = cache.layer_caches[i]
-            reader = self.layers[self.order[i + 1].layer] if i + 1 < len(self.order) else self.final_norm
-            ctx.next_takes_planes = bool(getattr(reader, "takes_planes", False))
-            x, pending = self.layers[call.layer].forward(x, pending, ctx)
+            if i + 1 < len(self.order):
+                sink = ResidualSink(x, self.layers[self.order[i + 1].layer].entry_norm)
+            else:
+                sink = ResidualSink(x, self.final_norm, rows=want_rows)
+            h = self.layers[call.layer].forward(x, h, ctx, sink)
         ctx.layer_cache = None
-        h = self.final_norm(x, delta=pending, rows=want_rows)
         return self.head.forward(h)

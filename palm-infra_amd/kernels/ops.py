@@ -31,7 +31,9 @@ _SIGNATURES = {
     "palm_rope_table": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int],
     "palm_attention_simple": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                               c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
-    "palm_linear_thin": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int],
+    "palm_linear_thin": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                         c_void_p, c_int, c_float, c_void_p, c_void_p, c_void_p],
+    "palm_scale_rows": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_float, c_int, c_void_p],
     "palm_linear_thin_parts": [c_int, c_int, c_int],
     "palm_linear_wide": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "palm_linear_wide_splits": [c_int, c_int, c_int, c_int],
@@ -323,15 +325,61 @@ def thin_serves(a: torch.Tensor, w: torch.Tensor) -> bool:
     return a.dtype == BF16 and w.dtype == BF16 and a.shape[1] % 8 == 0
 
 
+def _row_ss(what: str, a: torch.Tensor, row_ss) -> int:
+    """Checks the pieces of the rows' sums of squares that come with rows lacking their norm's factor."""
+    if row_ss is None:
+        return 0
+    _dev(what, a, row_ss)
+    _need(row_ss.dim() == 2 and row_ss.shape[0] == a.shape[0] and row_ss.dtype == F32 and row_ss.is_contiguous()
+          and row_ss.shape[1] > 0, f"{what}: sums of squares {tuple(row_ss.shape)} {row_ss.dtype} for {a.shape[0]} rows")
+    _need(a.shape[0] <= THIN_TOKENS and thin_serves(a, a), f"{what}: a norm is folded into products of at most {THIN_TOKENS} bfloat16 rows")
+    return row_ss.shape[1]
+
+
+def scale_rows(a: torch.Tensor, row_ss: torch.Tensor, eps: float) -> torch.Tensor:
+    """a[r] / sqrt(sum of row_ss[r, :] / width + eps): rows that lack their norm's factor, made whole."""
+    _dev("scale_rows", a, row_ss)
+    _need(a.dim() == 2 and row_ss.dim() == 2 and row_ss.shape[0] == a.shape[0] and row_ss.dtype == F32 and row_ss.is_contiguous()
+          and row_ss.shape[1] > 0, f"scale_rows: rows {tuple(a.shape)}, sums of squares {tuple(row_ss.shape)} {row_ss.dtype}")
+    out = torch.empty_like(a)
+    library.call(core(), "palm_scale_rows", _stream(), _p(a), _code(a, "scale_rows"), _p(row_ss), row_ss.shape[1], a.shape[0],
+                 float(eps), a.shape[1], _p(out))
+    return out
+
+
+def linear_thin_into_residual(a: torch.Tensor, w: torch.Tensor, x: torch.Tensor, norm_w: torch.Tensor, row_ss=None,
+                              row_eps: float = 0.0):
+    """A branch's last product and what follows it, for up to 16 rows: x += a . w^T (x float32 [M, N], in
+    place); returns (x * norm_w rounded to bfloat16, the pieces [M, N/16] of each row's sum of squares of x):
+    the next norm's output but for the row factor.  row_ss / row_eps: a itself lacks a row factor."""
+    _dev("linear_thin_into_residual", a, w, x, norm_w)
+    M, K = a.shape
+    N = w.shape[0]
+    _need(thin_serves(a, w) and M <= THIN_TOKENS and w.shape[1] == K, f"linear_thin_into_residual: a {tuple(a.shape)} {a.dtype}, "
+          f"w {tuple(w.shape)} {w.dtype} (bfloat16, at most {THIN_TOKENS} rows, K a multiple of 8)")
+    _need(x.shape == (M, N) and x.dtype == F32 and x.is_contiguous(), f"linear_thin_into_residual: residual {tuple(x.shape)} {x.dtype}")
+    _need(norm_w.shape == (N,) and norm_w.dtype == F32, "linear_thin_into_residual: the norm's weight is float32 [N]")
+    pieces = _row_ss("linear_thin_into_residual", a, row_ss)
+    values = torch.empty((M, N), dtype=BF16, device=a.device)
+    ss = torch.empty((M, (N + 15) // 16), dtype=F32, device=a.device)
+    library.call(core(), "palm_linear_thin", _stream(), _p(a), _p(w), _p(values), _code(values, "values"), M, N, K, 0, 1,
+                 _p(row_ss), pieces, float(row_eps), _p(x), _p(norm_w), _p(ss))
+    return values, ss
+
+
 def linear_thin(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, gated: bool = False,
-                planes_ok: bool = False) -> torch.Tensor:
+                planes_ok: bool = False, row_ss=None, row_eps: float = 0.0) -> torch.Tensor:
     """bfloat16 a [M, K] . w [N, K]^T on the matrix cores, the weight streamed once per 64 rows of a;
     result [M, N] in bfloat16 or float32.  With ``gated`` w is [gate rows | up rows] and the result is
     silu(a gate^T) * (a up^T), [M, N/2].
 
     ``planes_ok``: the caller can take the product as float32 planes [P, M, N] whose sum (in the order of the
     planes) it is: for a few rows and few weight rows the kernel then cuts K into P ranges to fill the chip.
-    rmsnorm's ``delta`` and qk_norm_rope_store's ``qkv`` take such planes."""
+    rmsnorm's ``delta`` and qk_norm_rope_store's ``qkv`` take such planes.
+
+    ``row_ss`` [M, pieces] float32 with ``row_eps``: the rows of a lack the factor 1 / sqrt(mean square + eps) of
+    their norm, whose sums of squares come in pieces; the result rows are multiplied by it (at most 16 rows)."""
+    pieces = _row_ss("linear_thin", a, row_ss)
     if not thin_serves(a, w):
         out = linear_exact(a, w, out_dtype)
         return swiglu(out) if gated else out
@@ -347,7 +395,7 @@ def linear_thin(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, gated:
         if planes > 1:
             out = torch.empty((planes, M, N), dtype=F32, device=a.device)
         library.call(core(), "palm_linear_thin", _stream(), _p(a), _p(w), _p(out), _code(out, "linear_thin out"), M, N, K,
-                     1 if gated else 0, planes)
+                     1 if gated else 0, planes, _p(row_ss), pieces, float(row_eps), None, None, None)
         return out
     # more rows than one block of 16: the kernel that shares the activations through LDS, K split if need be
     splits = core().palm_linear_wide_splits(M, N, K, 1 if gated else 0)

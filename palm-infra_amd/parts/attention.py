@@ -52,7 +52,9 @@ class Attention:
         p = spec.params
         return [KVNeed(int(p["num_kv_heads"]), int(p["head_dim"]), int(p["window"]) if p.get("window") else None)]
 
-    def forward(self, h: torch.Tensor, ctx) -> torch.Tensor:
+    takes_sink = True
+
+    def forward(self, h, ctx, sink=None):
         lc = ctx.layer_cache
         if lc is None or lc.kv is None:
             raise RuntimeError("attention needs the keys and values of its layer; the step gave it no cache")
@@ -66,6 +68,6 @@ class Attention:
             rotary_dim=self.position.rotary_dim if tables is not None else 0,
             pairing=PAIRINGS[self.position.pairing] if tables is not None else 0,
             k_cache=lc.k, v_cache=lc.v, block_table=lc.kv.table_dev, tok_slot=ctx.tok_slot, write_cache=lc.writes,
-            out_dtype=h.dtype)
+            out_dtype=self.dtype)
         o = ops.attention(q, lc.k, lc.v, lc.kv.table_dev, ctx, self.nh, self.nkv, self.hd, self.scale, self.window)
-        return self.out(o, planes_ok=bool(getattr(ctx, "planes_ok", False)))
+        return self.out(o, sink=sink)

@@ -12,8 +12,14 @@ which model it is in.  Interfaces, by category:
   mixer         ``forward(h, ctx)`` -> branch output [n, hidden]; ``cache_needs(spec)`` (static) -> what it
                 keeps per sequence (``KVNeed`` / ``StateNeed``); reads ``ctx.layer_cache``.
   feed_forward  ``forward(h, ctx)`` -> branch output [n, hidden].
-  block         ``forward(x, pending, ctx)`` -> (x, pending): the arrangement of norms, mixer and feed-forward
-                around the residual stream; ``pending`` is a branch output that the next norm adds.
+                A mixer or feed-forward may set ``takes_sink = True`` and have ``forward(h, ctx, sink=None)``: h
+                may then be ``Prenormed`` rows, and with a sink the part returns what the sink's norm makes of
+                the residual stream after its output is added (parts/residual.py), usually by handing the sink
+                to its last ``Linear``.
+  block         ``entry_norm``: the norm applied to the residual stream before the block's first branch;
+                ``forward(x, h, ctx, sink)`` -> normed rows: x is the residual stream (updated in place), h is
+                ``entry_norm`` of x (a tensor or ``Prenormed`` rows), sink names the norm that reads x after the
+                block and the rows it wants; what that norm gives is returned.
   embedding     ``forward(token_ids)`` -> float32 [n, hidden].
   head          ``forward(h)`` -> float32 logits [rows, vocab].
 """
@@ -89,8 +95,6 @@ class StepContext:
     is_decode: bool = False      # every sequence brings exactly one token
     decode_slices: int = 0       # if set: into how many slices decode attention cuts a key range (else chosen per call)
     layer_cache: object = None   # the LayerCache of the run-order entry that is running
-    planes_ok: bool = False      # the reader of the running branch's output adds float32 planes [P, n, width]
-    next_takes_planes: bool = False   # the same for what the running layer hands on as pending (set by the model)
     memo: dict = field(default_factory=dict)   # what parts make once per step (rotation tables)
     host: dict = field(default_factory=dict)   # the same facts as Python lists, for parts that plan on the host
 

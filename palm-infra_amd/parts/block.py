@@ -1,14 +1,16 @@
 """The arrangement of a layer's parts around the residual stream.
 
 ``pre_norm``: x += mixer(norm(x)); x += feed_forward(norm(x)) (models/qwen3.py:254-287).  The residual
-stream x is float32; a branch's output is not added at once but handed on as ``pending``, and the next
-norm adds it in the same pass in which it norms (the sum is made in 32-bit and written back to x).
-A branch may hand its output on as float32 planes [P, n, width] of partial sums if ``ctx.planes_ok`` says
-that the norm which reads it adds them up; a part that ignores the flag returns [n, width] as ever.
+stream x is float32.  A branch's output is never added by a kernel of its own: it goes into a
+``ResidualSink`` (parts/residual.py), and either the norm that reads x next adds it in the pass in which it
+norms (the sum is made in 32-bit and written back to x), or the branch's last product does both.  So the
+block gets its first norm's output from whoever ran before it, and returns the output of the norm that comes
+after it.
 """
 from __future__ import annotations
 
 from .base import cache_needs, register_part
+from .residual import ResidualSink, run_branch
 
 
 @register_part("block", "pre_norm")
@@ -29,16 +31,9 @@ class PreNormBlock:
         return cache_needs(spec.parts["mixer"])
 
     @property
-    def takes_planes(self) -> bool:
-        """Whether ``pending`` may come as float32 planes [P, n, width] (the first norm adds them up)."""
-        return bool(getattr(self.mixer_norm, "takes_planes", False))
+    def entry_norm(self):
+        return self.mixer_norm
 
-    def forward(self, x, pending, ctx):
-        h = self.mixer_norm(x, delta=pending, update=pending is not None)
-        ctx.planes_ok = bool(getattr(self.feed_forward_norm, "takes_planes", False))
-        a = self.mixer.forward(h, ctx)
-        h = self.feed_forward_norm(x, delta=a, update=True)
-        ctx.planes_ok = ctx.next_takes_planes
-        out = self.feed_forward.forward(h, ctx)
-        ctx.planes_ok = False
-        return x, out
+    def forward(self, x, h, ctx, sink):
+        h = run_branch(self.mixer, h, ctx, ResidualSink(x, self.feed_forward_norm))
+        return run_branch(self.feed_forward, h, ctx, sink)

@@ -21,5 +21,7 @@ class GatedSiluFeedForward:
             raise ValueError(f"feed-forward: weights {tuple(self.gate_up.weight.shape)}, {tuple(self.down.weight.shape)} "
                              f"do not fit hidden {self.hidden}, intermediate {self.inter}")
 
-    def forward(self, h: torch.Tensor, ctx) -> torch.Tensor:
-        return self.down(self.gate_up.gated(h), planes_ok=bool(getattr(ctx, "planes_ok", False)))
+    takes_sink = True
+
+    def forward(self, h, ctx, sink=None):
+        return self.down(self.gate_up.gated(h), sink=sink)

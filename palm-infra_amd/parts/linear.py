@@ -10,6 +10,7 @@ from __future__ import annotations
 import torch
 
 from ..kernels import ops
+from .residual import Prenormed
 
 # above this many rows the library's large tiles win over streaming the weight once per 64 rows
 THIN_ROWS = 64
@@ -22,21 +23,49 @@ class Linear:
         self.weight = weight
         self.out_features, self.in_features = weight.shape
 
-    def __call__(self, x: torch.Tensor, out_dtype: torch.dtype | None = None, planes_ok: bool = False) -> torch.Tensor:
-        """``planes_ok``: the caller hands the result to a reader that adds float32 planes [P, n, out] (a norm's
+    def __call__(self, x, out_dtype: torch.dtype | None = None, planes_ok: bool = False, sink=None):
+        """x: rows [n, in], or ``Prenormed`` rows (their row factor is applied to the result).
+
+        ``planes_ok``: the caller hands the result to a reader that adds float32 planes [P, n, out] (a norm's
         ``delta``, the q/k/v of qk_norm_rope_store); a thin product with few weight rows may then come as such
-        planes, each the sum over one range of the inner size."""
-        out_dtype = out_dtype or x.dtype
+        planes, each the sum over one range of the inner size.
+
+        ``sink`` (a ``ResidualSink``): the product is a branch's output; what comes back is what the sink's
+        norm makes of the residual stream after the add, as a tensor or as ``Prenormed`` rows."""
+        if sink is not None:
+            return self._into(x, sink)
         w = self.weight
+        if isinstance(x, Prenormed):
+            if self._folds(x.values):
+                return ops.linear_thin(x.values, w, out_dtype or x.dtype, planes_ok=planes_ok, row_ss=x.ss, row_eps=x.eps)
+            x = x.materialize()
+        out_dtype = out_dtype or x.dtype
         if x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16:
             if x.shape[0] <= THIN_ROWS or out_dtype != torch.bfloat16:
                 return ops.linear_thin(x, w, out_dtype, planes_ok=planes_ok)
             return ops.linear_library(x, w)
         return ops.linear_exact(x, w, out_dtype)
 
-    def gated(self, x: torch.Tensor) -> torch.Tensor:
+    def _folds(self, rows: torch.Tensor) -> bool:
+        """Whether the kernel that folds a norm into the product serves these rows."""
+        return rows.shape[0] <= ops.THIN_TOKENS and ops.thin_serves(rows, self.weight)
+
+    def _into(self, x, sink):
+        rows = x.values if isinstance(x, Prenormed) else x
+        if (sink.foldable and self._folds(rows) and sink.x.shape == (rows.shape[0], self.out_features)
+                and rows.dtype == torch.bfloat16):
+            ss_in, eps_in = (x.ss, x.eps) if isinstance(x, Prenormed) else (None, 0.0)
+            values, ss = ops.linear_thin_into_residual(rows, self.weight, sink.x, sink.norm.weight, row_ss=ss_in, row_eps=eps_in)
+            return Prenormed(values, ss, sink.norm.eps)
+        return sink.finish(self(x, planes_ok=sink.takes_planes))
+
+    def gated(self, x) -> torch.Tensor:
         """silu(x G^T) * (x U^T) for a weight that is [G rows | U rows]: in one kernel when the product is thin,
         else the product and then the activation."""
+        if isinstance(x, Prenormed):
+            if self._folds(x.values):
+                return ops.linear_thin(x.values, self.weight, x.dtype, gated=True, row_ss=x.ss, row_eps=x.eps)
+            x = x.materialize()
         if x.shape[0] <= THIN_ROWS and ops.thin_serves(x, self.weight):
             return ops.linear_thin(x, self.weight, x.dtype, gated=True)
         return ops.swiglu(self(x))

@@ -13,6 +13,7 @@ from .base import register_part
 class RMSNorm:
     capturable = True      # launches the same kernels whatever the step holds: may be recorded into a HIP graph
     takes_planes = True    # ``delta`` may be float32 planes [P, n, width], added one after the other
+    folds_into_products = True   # y = x * f(row) * weight, f = 1 / sqrt(mean(x^2) + eps): see parts/residual.py
 
     def __init__(self, spec, builder):
         self.width = int(spec.params["width"])

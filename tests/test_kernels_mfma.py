@@ -53,6 +53,60 @@ def test_linear_thin_as_planes_of_partial_sums(ops, M, N, K, planes):
     assert ops.linear_thin(a.to(DEV), w.to(DEV), BF16, planes_ok=False).shape == (M, N)
 
 
+@pytest.mark.parametrize("M", [1, 5, 16])
+@pytest.mark.parametrize("N,K", [(80, 64), (4096, 4096), (1000, 1096), (515, 12288), (8200, 2048)])
+def test_linear_thin_into_the_residual_stream_and_on_with_the_row_factor(ops, M, N, K):
+    """A product that adds its result to the residual stream and leaves the next norm's output but for the row
+    factor; then a product (plain, in planes, gated) that takes such rows: together they are
+    x += a W1^T;  y = rms_norm(x, w) W2^T."""
+    eps = 1e-5
+    a, w1 = rand(M, K, seed=M), rand(N, K, seed=N, scale=0.1)
+    x0, nw = rand(M, N, seed=3, dtype=F32) * 3, rand(N, seed=4, dtype=F32) + 1.0
+    xd = x0.to(DEV)
+    values, ss = ops.linear_thin_into_residual(a.to(DEV), w1.to(DEV), xd, nw.to(DEV))
+    x_ref = x0.double() + P.linear(a, w1)
+    assert torch.allclose(xd.cpu().double(), x_ref, atol=2e-4 * (K ** 0.5), rtol=1e-5)          # 32-bit, in place
+    assert values.dtype == BF16 and ss.shape == (M, (N + 15) // 16)
+    assert torch.allclose(ss.cpu().double().sum(1), (x_ref ** 2).sum(1), rtol=1e-4)
+    assert torch.allclose(values.cpu().double(), x_ref * nw.double(), atol=3e-2, rtol=1e-2)
+    whole = ops.scale_rows(values, ss, eps).cpu().double()
+    normed = P.rms_norm(x_ref, nw.double(), eps)
+    assert torch.allclose(whole, normed, atol=3e-2, rtol=1e-2)
+    # the reader: the same rows go in with and without their factor
+    # (rows whose length is no multiple of 8 go the way of the exact kernel, made whole first)
+    for N2, gated in ((96, False), (6144, False), (2 * 176, True), (2 * 4500, True)) if N % 8 == 0 else ():
+        w2 = rand(N2, N, seed=N2, scale=0.2)
+        for planes_ok in (False, True):
+            if gated and planes_ok:
+                continue
+            got = ops.linear_thin(values, w2.to(DEV), F32, gated=gated, planes_ok=planes_ok, row_ss=ss, row_eps=eps).cpu().double()
+            want = ops.linear_thin(ops.scale_rows(values, ss, eps), w2.to(DEV), F32, gated=gated).cpu().double()
+            if got.dim() == 3:
+                got = got.sum(0)
+            scale = float(want.abs().max())
+            # scale_rows rounds the rows to bfloat16 once more than the fold does: a few parts in a thousand
+            assert torch.allclose(got, want, atol=1.5e-2 * scale), (N2, gated, planes_ok, float((got - want).abs().max()), scale)
+    # and both at once: rows without their factor in, residual stream and the next such rows out
+    if N % 8 == 0:
+        w3 = rand(N, N, seed=9, scale=0.05)
+        x1 = xd.clone()
+        v2, ss2 = ops.linear_thin_into_residual(values, w3.to(DEV), x1, nw.to(DEV), row_ss=ss, row_eps=eps)
+        x1_ref = x_ref + P.linear(normed.to(BF16), w3)
+        assert torch.allclose(x1.cpu().double(), x1_ref, atol=2e-2 * float(x1_ref.abs().max()))
+        assert torch.allclose(ss2.cpu().double().sum(1), (x1.cpu().double() ** 2).sum(1), rtol=1e-4)
+
+
+def test_the_folded_norm_refuses_what_it_does_not_serve(ops):
+    from palm_infra_amd.kernels import KernelError
+    a, w, x, nw = rand(17, 64).to(DEV), rand(32, 64).to(DEV), torch.zeros(17, 32, device=DEV), torch.ones(32, device=DEV)
+    with pytest.raises(KernelError, match="16"):
+        ops.linear_thin_into_residual(a, w, x, nw)
+    with pytest.raises(KernelError, match="residual"):
+        ops.linear_thin_into_residual(a[:4].contiguous(), w, x[:4, :8].contiguous(), nw)
+    with pytest.raises(KernelError, match="sums of squares"):
+        ops.linear_thin(a[:4].contiguous(), w, F32, row_ss=torch.zeros(5, 2, device=DEV), row_eps=1e-6)
+
+
 def test_linear_thin_orientation(ops):
     """One weight row and one token stand out: the product must land at [token, feature], not transposed,
     and every k must be used exactly once."""

@@ -181,13 +181,15 @@ def test_embedding_and_head_parts(dtype):
     assert lg.dtype == F32 and torch.allclose(lg.double(), P.linear(h, table), atol=1e-4 if dtype == F32 else 2e-2)
 
 
+@pytest.mark.parametrize("n_rows", [70, 5])
 @pytest.mark.parametrize("dtype", [F32, BF16])
-def test_block_part_is_a_plain_decoder_layer(dtype, model_dirs):
-    """One layer of tiny model C, built as a block from the model's description and run alone."""
+def test_block_part_is_a_plain_decoder_layer(dtype, n_rows, model_dirs):
+    """One layer of tiny model C, built as a block from the model's description and run alone: with many rows
+    (the norms run as kernels of their own) and with few (in bfloat16 the products fold them in)."""
     import tiny
     from palm_infra_amd.cache import ModelCache
     from palm_infra_amd.config import config_from_dir
-    from palm_infra_amd.parts import Builder, cache_needs, make_context
+    from palm_infra_amd.parts import Builder, Prenormed, ResidualSink, as_tensor, cache_needs, make_context
     from palm_infra_amd.weights import ModelFiles, load_weights
     name = "float32" if dtype == F32 else "bfloat16"
     d = model_dirs["C"][name]
@@ -199,17 +201,24 @@ def test_block_part_is_a_plain_decoder_layer(dtype, model_dirs):
     slot = cache.open()
     cfg, w = P.read_model(d)
     S = P.sizes(cfg)
-    x0 = rand(70, S["H"], seed=5)
-    pend = rand(70, S["H"], seed=6).to(dtype)
-    cache.reserve([(slot, 70)])
-    ctx = make_context([slot], [0], [[0] * 70], dtype, DEV)
+    x0 = rand(n_rows, S["H"], seed=5)
+    cache.reserve([(slot, n_rows)])
+    ctx = make_context([slot], [0], [[0] * n_rows], dtype, DEV)
     ctx.layer_cache = cache.layer_caches[0]
     xd = x0.to(DEV)
-    x_out, pending = block.forward(xd, pend.to(DEV), ctx)
-    assert x_out is xd and x_out.dtype == F32                    # the residual stream stays 32-bit and in place
-    got = x_out.cpu().double() + pending.cpu().double()
-    ref = P.decoder_layer(x0.double() + pend.double(), w, 1, S, list(range(70)))
-    assert torch.allclose(got, ref, atol=tol(dtype) * float(ref.abs().max()))
+    h = block.entry_norm(xd)
+    out = block.forward(xd, h, ctx, ResidualSink(xd, block.entry_norm))      # the reader after it: the same norm again
+    assert isinstance(out, Prenormed) == (dtype == BF16 and n_rows <= 16)
+    ref = P.decoder_layer(x0.double(), w, 1, S, list(range(n_rows)))
+    assert xd.dtype == F32 and torch.allclose(xd.cpu().double(), ref, atol=tol(dtype) * float(ref.abs().max()))   # in place, 32-bit
+    ref_out = P.rms_norm(ref, w["model.layers.1.input_layernorm.weight"].double(), S["eps"])
+    got_out = as_tensor(out).cpu().double()
+    assert torch.allclose(got_out, ref_out, atol=tol(dtype) * float(ref_out.abs().max()))
+    # rows picked by the reader: nothing is written back, only those rows come out
+    x2 = x0.to(DEV)
+    rows = torch.tensor([n_rows - 1, 0], dtype=torch.int32).to(DEV)
+    picked = as_tensor(block.forward(x2, block.entry_norm(x2), ctx, ResidualSink(x2, block.entry_norm, rows=rows))).cpu().double()
+    assert torch.allclose(picked, ref_out[[n_rows - 1, 0]], atol=tol(dtype) * float(ref_out.abs().max()))
 
 
 def test_unknown_kind_names_the_registered_ones():
