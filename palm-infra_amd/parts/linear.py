@@ -12,8 +12,10 @@ import torch
 from ..kernels import ops
 from .residual import Prenormed
 
-# above this many rows the library's large tiles win over streaming the weight once per 64 rows
-THIN_ROWS = 64
+# Up to this many rows the kernel that streams the weight past one block of 16 rows is the fastest; above, the
+# library is (measured at Qwen3-8B's four shapes with 17, 32 and 64 rows: 15 to 49 us against 18 to 66 us of
+# the kernel that shares 64 rows through LDS, which still serves products with a float32 result).
+THIN_ROWS = 16
 
 
 class Linear:
