@@ -220,6 +220,90 @@ def test_qk_norm_rope_store(ops, dtype, nh, nkv, hd):
                 assert float(kc[page, :, r].abs().max()) == 0.0 and float(vc[page, :, :, r].abs().max()) == 0.0
 
 
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("nh,nkv,hd", [(5, 5, 48), (6, 2, 80), (3, 1, 128), (8, 2, 16), (4, 4, 32), (9, 3, 64), (2, 1, 256), (3, 1, 144)])
+def test_qk_norm_rope_store_of_many_tokens(ops, dtype, nh, nkv, hd):
+    """Prompts go through kernels of their own (heads held in registers, v written tile by tile): three
+    sequences that start inside pages, cross page borders, and fill no tile of 64 tokens."""
+    starts, counts, slots = [60, 0, 130], [70, 41, 3], [2, 0, 3]
+    n = sum(counts)
+    pos = [s + j for s, c in zip(starts, counts) for j in range(c)]
+    tslot = [sl for sl, c in zip(slots, counts) for _ in range(c)]
+    qkv = rand(n, (nh + 2 * nkv) * hd, seed=hd, dtype=dtype)
+    qw, kw = rand(hd, seed=1) + 1.0, rand(hd, seed=2) + 1.0
+    eps, theta = 1e-5, 10000.0
+    table = torch.full((4, 3), 9, dtype=torch.int32)
+    table[2] = torch.tensor([5, 1, 7])
+    table[0, :1] = torch.tensor([3])
+    table[3] = torch.tensor([9, 9, 0])
+    kc, vc = _paged(10, nkv, hd, dtype)
+    inv = torch.from_numpy((1.0 / np.power(np.float32(theta), 2.0 * np.arange(hd // 2, dtype=np.float32) / hd)).astype(np.float32))
+    pos_d = torch.tensor(pos, dtype=torch.int32).to(DEV)
+    cos, sin = ops.rope_table(pos_d, inv.to(DEV))
+    q = ops.qk_norm_rope_store(qkv.to(DEV), nh, nkv, hd, pos_d, q_norm_w=qw.to(DEV), k_norm_w=kw.to(DEV), eps=eps, cos=cos, sin=sin,
+                               rotary_dim=hd, pairing=0, k_cache=kc, v_cache=vc, block_table=table.to(DEV),
+                               tok_slot=torch.tensor(tslot, dtype=torch.int32).to(DEV)).cpu()
+    x = qkv.double()
+    rq = x[:, :nh * hd].reshape(n, nh, hd)
+    rk = x[:, nh * hd:(nh + nkv) * hd].reshape(n, nkv, hd)
+    rv = x[:, (nh + nkv) * hd:].reshape(n, nkv, hd)
+    c64, s64 = P.rope_table(pos, hd, theta)
+    rq = P.rope_half_split(P.rms_norm(rq, qw, eps), c64, s64)
+    rk = P.rope_half_split(P.rms_norm(rk, kw, eps), c64, s64)
+    t = 5e-5 if dtype == F32 else 4e-2
+    assert torch.allclose(q.double().reshape(n, nh, hd), rq, atol=t)
+    kc, vc = kc.cpu().double(), vc.cpu().double()
+    written = torch.zeros(10, 64, dtype=torch.bool)
+    for i in range(n):
+        page = int(table[tslot[i], pos[i] // 64])
+        assert torch.allclose(kc[page, :, pos[i] % 64], rk[i], atol=t), i
+        assert torch.allclose(vc[page, :, :, pos[i] % 64], rv[i], atol=1e-12 if dtype == F32 else 0), i   # v is stored as it is
+        written[page, pos[i] % 64] = True
+    rest = ~written
+    assert float(kc.permute(0, 2, 1, 3)[rest].abs().max()) == 0.0 and float(vc.permute(0, 3, 1, 2)[rest].abs().max()) == 0.0
+    # the same tokens a few at a time (the kernel for few tokens) leave the same cache, up to the last bit of a sum
+    kc2, vc2 = _paged(10, nkv, hd, dtype)
+    for a in range(0, n, 9):
+        sl = slice(a, a + 9)
+        ops.qk_norm_rope_store(qkv[sl].contiguous().to(DEV), nh, nkv, hd, pos_d[sl].contiguous(), q_norm_w=qw.to(DEV), k_norm_w=kw.to(DEV),
+                               eps=eps, cos=cos[sl].contiguous(), sin=sin[sl].contiguous(), rotary_dim=hd, pairing=0, k_cache=kc2,
+                               v_cache=vc2, block_table=table.to(DEV), tok_slot=torch.tensor(tslot[sl], dtype=torch.int32).to(DEV))
+    assert torch.allclose(kc2.cpu().double(), kc, atol=1e-5 if dtype == F32 else 4e-2) and torch.equal(vc2.cpu().double(), vc)
+
+
+def test_qk_norm_rope_store_of_many_tokens_in_planes_and_other_rotations(ops):
+    nh, nkv, hd, n = 6, 2, 64, 100
+    i32 = lambda xs: torch.tensor(xs, dtype=torch.int32).to(DEV)
+    pos, slot = i32(list(range(30, 30 + n))), i32([1] * n)
+    table = i32([[9, 9, 9], [4, 2, 6]])
+    qw, kw = (rand(hd, seed=1) + 1.0).to(DEV), (rand(hd, seed=2) + 1.0).to(DEV)
+    planes = rand(3, n, (nh + 2 * nkv) * hd, seed=11)
+    whole = ((planes[0] + planes[1]) + planes[2]).to(BF16)
+    for pairing, rot, norms, writes in ((0, hd, True, True), (1, hd, True, True), (1, 24, False, True), (0, 0, True, True),
+                                        (0, 32, True, True), (0, hd, True, False)):
+        cos = sin = None
+        if rot:
+            inv = torch.from_numpy((1.0 / np.power(np.float32(1e6), 2.0 * np.arange(rot // 2, dtype=np.float32) / rot)).astype(np.float32))
+            cos, sin = ops.rope_table(pos, inv.to(DEV))
+        kw_args = dict(q_norm_w=qw if norms else None, k_norm_w=kw if norms else None, eps=1e-6, cos=cos, sin=sin, rotary_dim=rot,
+                       pairing=pairing, block_table=table, tok_slot=slot, write_cache=writes)
+        results = []
+        # all at once from planes (the kernels for many tokens where they serve), and eleven at a time from one tensor
+        kc, vc = _paged(10, nkv, hd, BF16)
+        q = ops.qk_norm_rope_store(planes.to(DEV), nh, nkv, hd, pos, k_cache=kc, v_cache=vc, out_dtype=BF16, **kw_args)
+        kc2, vc2 = _paged(10, nkv, hd, BF16)
+        qs = []
+        for a in range(0, n, 11):
+            sl = slice(a, a + 11)
+            args = dict(kw_args, cos=None if cos is None else cos[sl].contiguous(), sin=None if sin is None else sin[sl].contiguous(),
+                        tok_slot=slot[sl].contiguous())
+            qs.append(ops.qk_norm_rope_store(whole[sl].contiguous().to(DEV), nh, nkv, hd, pos[sl].contiguous(), k_cache=kc2, v_cache=vc2, **args))
+        case = (pairing, rot, norms, writes)
+        assert torch.allclose(q.float(), torch.cat(qs).float(), atol=6e-2, rtol=2e-2), case
+        assert torch.allclose(kc.float(), kc2.float(), atol=6e-2, rtol=2e-2) and torch.allclose(vc.float(), vc2.float(), atol=2e-2, rtol=1e-2), case
+        assert (float(kc.abs().max()) > 0.5) == writes, case
+
+
 def test_rotation_variants_interleaved_partial_and_none(ops):
     n, nh, nkv, hd, rot = 4, 2, 1, 32, 16
     pos = [3, 4, 5, 6]
