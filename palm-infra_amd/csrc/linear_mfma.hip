@@ -1,9 +1,10 @@
-// C[M, N] = A[M, K] . W[N, K]^T for few rows (decode steps, logits rows): bfloat16 operands on the matrix
-// cores, 32-bit accumulation, the weight streamed from HBM once per 64 rows of A.  The product itself is the
+// C[M, N] = A[M, K] . W[N, K]^T for up to 16 rows (decode steps, logits rows): bfloat16 operands on the matrix
+// cores, 32-bit accumulation, the weight streamed from HBM once.  The product itself is the
 // reference's matmul (kernels/matmul_dense.cpp:939-953); its GEMV paths (kernels/matmul_dense.cpp:1282-1332)
 // are what this kernel stands for.  An epilogue can apply the gated activation of the feed-forward
 // (out = silu(gate) * up, engine/cuda_ops.cu:100-112) so that the [M, 2I] product never goes to memory.
 //
+// Two kernels: for a short K the one described next, for a long K the stream kernel further down.
 // Work split.  A block owns RT strips of 16 weight rows (16 output features each) and all of K; its waves
 // take every NW-th "super-step" of 128 k-values and their partial tiles are added in LDS in a fixed order (no
 // atomics: the same input gives the same bits).  In a super-step lane (r, g) of a wave makes four 16-byte
@@ -391,17 +392,8 @@ static void dispatch_thin(hipStream_t stream, const void* a, const void* w, void
         else launch_stream<4, 0, TC, EPI>(stream, a, w, c, M, N, K, parts, norm);
         return;
     }
-    if (M <= 16) {
-        // a short K: one strip a block, four waves (two strips a block, RT = 2, were measured slower at every
-        // size)
-        launch_thin<1, 4, 2, 1, TC, EPI>(stream, a, w, c, M, N, K);
-    } else if (M <= 32) {
-        if (deep) launch_thin<2, 8, 2, 1, TC, EPI>(stream, a, w, c, M, N, K);
-        else launch_thin<2, 4, 2, 1, TC, EPI>(stream, a, w, c, M, N, K);
-    } else {
-        if (deep) launch_thin<4, 8, 2, 1, TC, EPI>(stream, a, w, c, M, N, K);
-        else launch_thin<4, 4, 1, 1, TC, EPI>(stream, a, w, c, M, N, K);
-    }
+    // a short K: one strip a block, four waves (two strips a block, RT = 2, were measured slower at every size)
+    launch_thin<1, 4, 2, 1, TC, EPI>(stream, a, w, c, M, N, K);
 }
 
 PALM_API int palm_linear_thin_parts(int M, int N, int K) { return stream_parts(M, N, K); }
@@ -429,7 +421,7 @@ PALM_API int palm_linear_thin(hipStream_t stream, const void* a, const void* w, 
     PALM_CHECK(epilogue != EPI_SWIGLU || N % 2 == 0, "linear_thin: a gated product needs an even N, got %d", N);
     PALM_CHECK(((uintptr_t)a | (uintptr_t)w) % 16 == 0, "linear_thin: operands must be 16-byte aligned");
     if (M == 0) return 0;
-    PALM_CHECK((M + 63) / 64 <= 65535, "linear_thin: M=%d is more than one launch takes", M);
+    PALM_CHECK(M <= 16, "linear_thin: %d rows are more than the 16 of one block of tokens (linear_wide takes up to 64)", M);
     if (epilogue == EPI_SWIGLU) {
         PALM_DTYPE_SWITCH(c_dtype, TC, dispatch_thin<TC, EPI_SWIGLU>(stream, a, w, c, M, N, K, 1, norm));
     } else {

@@ -369,7 +369,7 @@ def linear_thin_into_residual(a: torch.Tensor, w: torch.Tensor, x: torch.Tensor,
 
 def linear_thin(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, gated: bool = False,
                 planes_ok: bool = False, row_ss=None, row_eps: float = 0.0) -> torch.Tensor:
-    """bfloat16 a [M, K] . w [N, K]^T on the matrix cores, the weight streamed once per 64 rows of a;
+    """bfloat16 a [M, K] . w [N, K]^T on the matrix cores, the weight streamed once per 16 rows of a (64 above 16);
     result [M, N] in bfloat16 or float32.  With ``gated`` w is [gate rows | up rows] and the result is
     silu(a gate^T) * (a up^T), [M, N/2].
 
