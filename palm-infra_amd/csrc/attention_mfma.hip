@@ -297,8 +297,13 @@ PALM_API int palm_attention_decode(hipStream_t stream, const void* q, const void
 // and a tile of QB query positions, QB = 16 * max(1, 8 / heads): at most eight "units" of 16 columns
 // (head, 16 positions), two for each wave.  A page of K and of V^T is read from memory once for the block,
 // into LDS; every wave takes its MFMA operands from there, each operand serving both of its units.  The next
-// page is on its way into registers while the current one is being used.  Tiles late in a sequence see more
-// keys, so they are started first.
+// page is on its way into registers while the current one is being used.
+// Causal attention gives a late tile of queries many more keys than an early one, and all blocks of a launch
+// run at once, so blocks of unequal work would leave half the chip waiting for the last ones.  A block's
+// 16-query sub-tiles are therefore taken alternately from the front and from the back of the sequence's new
+// tokens (sub-tile f with sub-tile N - 1 - f): every block then has about the same number of (unit, page)
+// products.  The early sub-tile's keys are among the late one's, so the block walks the late one's pages and
+// the early one's units just stop taking part (`active`) once the pages lie beyond them.
 constexpr int PF_WAVES = 4;
 constexpr int PF_THREADS = PF_WAVES * WAVE;
 constexpr int PF_UNITS = 2;                                // units of 16 columns held by a wave
@@ -346,6 +351,8 @@ __device__ inline void stage_values(const PagePrefetch& pf, bf16_t* v_lds) {
 
 struct Unit {                 // one (head, 16 query positions): the wave's share of it
     bool live;                // false: the wave has no such unit (fewer units than slots)
+    bool active;              // the page at hand holds keys that some column of the unit sees
+    int page_lo, page_hi;     // the pages that do
     bool valid;               // this lane's column is a real query
     int pos, first;           // the column's position and the first key it sees
     size_t row;               // the column's row in q and out
@@ -380,13 +387,17 @@ __device__ inline void unit_scores(const bf16_t* k_lds, Unit (&u)[PF_UNITS], int
 #pragma unroll
         for (int x = 0; x < PF_UNITS; ++x) s[x][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int j = 0; j < KSTEPS; ++j)
+        for (int x = 0; x < PF_UNITS; ++x) {
+            if (!u[x].active) continue;
 #pragma unroll
-            for (int x = 0; x < PF_UNITS; ++x) s[x][t] = mfma_16x16x32(kf[t & 1][j], u[x].qv[j], s[x][t]);
+            for (int j = 0; j < KSTEPS; ++j) s[x][t] = mfma_16x16x32(kf[t & 1][j], u[x].qv[j], s[x][t]);
+        }
     }
 #pragma unroll
     for (int x = 0; x < PF_UNITS; ++x) {
         Columns& c = u[x].c;
+        alpha[x] = 1.0f;
+        if (!u[x].active) continue;
         float mx = -INFINITY;
         if (interior) {
 #pragma unroll
@@ -431,9 +442,11 @@ __device__ inline void unit_values(const bf16_t* v_lds, Unit (&u)[PF_UNITS], int
                                    const bf16x8 (&pv)[PF_UNITS][2], const float (&alpha)[PF_UNITS], bool rescale) {
     if (rescale) {
 #pragma unroll
-        for (int x = 0; x < PF_UNITS; ++x)
+        for (int x = 0; x < PF_UNITS; ++x) {
+            if (!u[x].active) continue;
 #pragma unroll
             for (int dt = 0; dt < DTILES; ++dt) u[x].c.o[dt] = u[x].c.o[dt] * alpha[x];
+        }
     }
     bf16x8 vf[2][2];
 #pragma unroll
@@ -446,9 +459,11 @@ __device__ inline void unit_values(const bf16_t* v_lds, Unit (&u)[PF_UNITS], int
             for (int h = 0; h < 2; ++h) vf[(dt + 1) & 1][h] = *reinterpret_cast<const bf16x8*>(vrow + h * 32 + g * 8);
         }
 #pragma unroll
-        for (int h = 0; h < 2; ++h)
+        for (int x = 0; x < PF_UNITS; ++x) {
+            if (!u[x].active) continue;
 #pragma unroll
-            for (int x = 0; x < PF_UNITS; ++x) u[x].c.o[dt] = mfma_16x16x32(vf[dt & 1][h], pv[x][h], u[x].c.o[dt]);
+            for (int h = 0; h < 2; ++h) u[x].c.o[dt] = mfma_16x16x32(vf[dt & 1][h], pv[x][h], u[x].c.o[dt]);
+        }
     }
 }
 
@@ -474,21 +489,36 @@ __global__ __launch_bounds__(PF_THREADS) PF_WAVES_PER_SIMD void attention_prefil
     const int G = nh / nkv, n_hg = (G + hg - 1) / hg;
     const int kvh = blockIdx.y / n_hg, hgi = blockIdx.y % n_hg;
     const int n_new = seq_new[b];
-    const int q0 = (gridDim.x - 1 - blockIdx.x) * qb;            // late tiles first: they have the most keys
-    if (q0 >= n_new) return;
-    const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE, r = lane % 16, g = lane / 16;
+    // the block's sub-tiles of 16 queries: number s is, for even s, sub-tile f = first + s / 2 from the front, for
+    // odd s its partner n16 - 1 - f from the back (none if f is the middle one); a single sub-tile a block (eight
+    // heads a group) just counts from the back, the long ones first
+    const int subs = qb / 16, n16 = (n_new + 15) / 16;
+    const int first_front = blockIdx.x * (subs > 1 ? subs / 2 : 1);
+    if (subs > 1 ? 2 * first_front > n16 - 1 : first_front >= n16) return;
+    auto sub_tile = [&](int sub) -> int {                       // the sub-tile's index, or -1
+        if (subs == 1) return n16 - 1 - first_front;
+        const int f = first_front + sub / 2, partner = n16 - 1 - f;
+        if (f > partner) return -1;
+        return (sub & 1) ? (partner > f ? partner : -1) : f;
+    };
+    const int lane = threadIdx.x % WAVE, r = lane % 16, g = lane / 16;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);      // the same in every lane: what follows from it stays scalar
     const int start = seq_start[b];
     const int heads_here = min(hg, G - hgi * hg);
-    const int n_units = heads_here * (qb / 16);
+    const int n_units = heads_here * subs;
     const int* pages = block_table + (size_t)seq_slot[b] * max_pages;
 
     Unit u[PF_UNITS];
 #pragma unroll
     for (int x = 0; x < PF_UNITS; ++x) {
         const int unit = wave + x * PF_WAVES;
-        u[x].live = unit < n_units;
+        const int tile16 = unit < n_units ? sub_tile(unit / heads_here) : -1;
+        u[x].live = tile16 >= 0;
         const int un = u[x].live ? unit : 0;
-        const int qi = q0 + (un / heads_here) * 16 + r;            // query index within the step
+        const int q_first = max(tile16, 0) * 16;                   // the unit's first query, within the step
+        const int qi = q_first + r;
+        u[x].page_hi = (start + min(q_first + 15, n_new - 1)) / PAGE_TOKENS;
+        u[x].page_lo = window > 0 ? max(0, start + q_first - window + 1) / PAGE_TOKENS : 0;
         u[x].head = kvh * G + hgi * hg + un % heads_here;
         u[x].valid = u[x].live && qi < n_new;
         const int qc = min(qi, n_new - 1);
@@ -502,9 +532,14 @@ __global__ __launch_bounds__(PF_THREADS) PF_WAVES_PER_SIMD void attention_prefil
         for (int dt = 0; dt < DTILES; ++dt) u[x].c.o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
-    const int tile_last = start + min(q0 + qb - 1, n_new - 1);
-    const int tile_first = window > 0 ? max(0, start + q0 - window + 1) : 0;
-    const int p_lo = tile_first / PAGE_TOKENS, p_hi = tile_last / PAGE_TOKENS;
+    // the pages any of the block's sub-tiles sees (the same for all waves)
+    int p_lo = 0x7fffffff, p_hi = -1;
+    for (int sub = 0; sub < subs; ++sub) {
+        const int tile16 = sub_tile(sub);
+        if (tile16 < 0) continue;
+        p_hi = max(p_hi, (start + min(tile16 * 16 + 15, n_new - 1)) / PAGE_TOKENS);
+        p_lo = min(p_lo, window > 0 ? max(0, start + tile16 * 16 - window + 1) / PAGE_TOKENS : 0);
+    }
     PagePrefetch pf;
     {
         const size_t base = ((size_t)pages[p_lo] * nkv + kvh) * PAGE_TOKENS * HD;
@@ -521,11 +556,13 @@ __global__ __launch_bounds__(PF_THREADS) PF_WAVES_PER_SIMD void attention_prefil
         if (!PF_SHARE) stage_values(pf, v_lds);
         __syncthreads();
         if (more) prefetch_keys(k_cache + next, pf);            // in flight while this page is used
-        // is every key of this page visible to every column of this wave?
+        // is every key of this page visible to every column of this wave that takes part?
         bool inside = true;
 #pragma unroll
-        for (int x = 0; x < PF_UNITS; ++x)
-            inside = inside && u[x].first <= p * PAGE_TOKENS && u[x].pos >= p * PAGE_TOKENS + PAGE_TOKENS - 1;
+        for (int x = 0; x < PF_UNITS; ++x) {
+            u[x].active = u[x].live && p >= u[x].page_lo && p <= u[x].page_hi;
+            inside = inside && (!u[x].active || (u[x].first <= p * PAGE_TOKENS && u[x].pos >= p * PAGE_TOKENS + PAGE_TOKENS - 1));
+        }
         const bool interior = __all(inside);
         unit_scores(k_lds, u, p * PAGE_TOKENS, scale_log2, r, g, interior, pv, alpha);
         bool moved = false;
@@ -572,7 +609,8 @@ PALM_API int palm_attention_prefill(hipStream_t stream, const void* q, const voi
     const int qb = 16 * (8 / hg > 0 ? 8 / hg : 1);             // query positions in a tile: at most 8 units a block
     const int n_hg = (G + hg - 1) / hg;
     PALM_CHECK(nkv * n_hg <= 65535 && n_seqs <= 65535, "attention_prefill: grid too large");
-    dim3 grid((max_new + qb - 1) / qb, nkv * n_hg, n_seqs);
+    const int n16 = (max_new + 15) / 16, subs = qb / 16;
+    dim3 grid(subs > 1 ? ((n16 + 1) / 2 + subs / 2 - 1) / (subs / 2) : n16, nkv * n_hg, n_seqs);
     attention_prefill_kernel<<<grid, PF_THREADS, 0, stream>>>((const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache,
                                                              block_table, max_pages, seq_slot, seq_start, seq_new, cu_new, nh,
                                                              nkv, scale * LOG2E, window, qb, hg, (bf16_t*)out);
