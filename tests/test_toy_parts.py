@@ -227,3 +227,161 @@ def test_layers_with_and_without_a_window_in_one_model(model_dirs, dtype):
         tiny.assert_logits_close(torch.cat(got[i]), plain(reqs[i]), dtype, f"window model request {i}")
         eng.close(slots[i])
     eng.cache.check()
+
+
+# ---- another norm, a feed-forward with routing, another position encoding ----------------------------
+
+def register_more_toy_parts():
+    from palm_infra_amd.parts import register_part
+
+    @register_part("norm", "toy_centered")
+    class CenteredNorm:
+        """y = (x - mean) / sqrt(var + eps) * w: not of the form x * f(row) * w, so no product may fold it in
+        (it sets neither ``folds_into_products`` nor ``takes_planes``) and it always runs by itself."""
+
+        def __init__(self, spec, builder):
+            self.weight, self.eps, self.dtype = builder.tensor(spec, "weight"), float(spec.params["eps"]), builder.dtype
+
+        def __call__(self, x, delta=None, update=False, rows=None, out_dtype=None):
+            assert delta is None or delta.dim() == 2            # planes were not asked for
+            v = x if delta is None else x + delta.float()
+            if update:
+                x.copy_(v)
+            if rows is not None:
+                v = v[rows.long()]
+            c = v - v.mean(-1, keepdim=True)
+            return (c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + self.eps) * self.weight).to(out_dtype or self.dtype)
+
+    @register_part("feed_forward", "toy_routed")
+    class RoutedFeedForward:
+        """Each token goes to the one of E small experts (relu(h A_e^T) B_e^T) whose router logit is largest;
+        the router is computed in 32-bit.  Plain tensors in and out: it knows nothing of sinks."""
+
+        def __init__(self, spec, builder):
+            self.router = builder.tensor(spec, "router")            # [E, H]
+            self.a, self.b = builder.tensor(spec, "a"), builder.tensor(spec, "b")     # [E * I, H], [E * H, I]
+            self.n, self.dtype = int(spec.params["experts"]), builder.dtype
+
+        def forward(self, h, ctx):
+            assert isinstance(h, torch.Tensor)
+            H = h.shape[1]
+            choice = (h.float() @ self.router.float().T).argmax(-1)
+            a = self.a.float().reshape(self.n, -1, H)
+            b = self.b.float().reshape(self.n, H, -1)
+            hidden = torch.relu(torch.einsum("th,tih->ti", h.float(), a[choice]))
+            return torch.einsum("ti,thi->th", hidden, b[choice]).to(self.dtype)
+
+    @register_part("position", "toy_schedule")
+    class LinearSchedule:
+        """Rotation angles position * step * (i + 1) over the first ``rotary_dim`` elements, interleaved pairs."""
+        capturable = True
+        pairing = "interleaved"
+
+        def __init__(self, spec, builder):
+            self.rotary_dim, self.step = int(spec.params["rotary_dim"]), float(spec.params["step"])
+            self.device = builder.device
+
+        def tables(self, ctx):
+            if "toy_schedule" not in ctx.memo:
+                i = torch.arange(1, self.rotary_dim // 2 + 1, device=self.device, dtype=torch.float32)
+                ang = ctx.positions.float()[:, None] * (self.step * i)[None, :]
+                ctx.memo["toy_schedule"] = (torch.cos(ang).contiguous(), torch.sin(ang).contiguous())
+            return ctx.memo["toy_schedule"]
+
+
+def _rope_interleaved(x, cos, sin, rot):
+    """x [n, heads, hd] float64; pairs (2i, 2i + 1) for 2i < rot."""
+    out = x.clone()
+    a, b = x[..., 0:rot:2], x[..., 1:rot:2]
+    c, s = cos[:, None, :], sin[:, None, :]
+    out[..., 0:rot:2] = a * c - b * s
+    out[..., 1:rot:2] = a * s + b * c
+    return out
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_another_norm_a_routed_feed_forward_and_another_position_encoding(model_dirs, dtype):
+    """Tiny model A with layer 0's rotation replaced by a toy schedule (interleaved pairs over half the head)
+    and layer 1's feed-forward and its norm replaced by toy parts: built from the description alone, stepped
+    with prompts and single tokens, against the plain computation."""
+    from palm_infra_amd.config import PartSpec, config_from_dir, tensor
+    from palm_infra_amd.engine import Engine, StepEntry
+    from palm_infra_amd.weights import ModelFiles, load_weights
+    register_more_toy_parts()
+    d = model_dirs["A"][dtype]
+    tdt = torch.float32 if dtype == "float32" else torch.bfloat16
+    config = config_from_dir(d)
+    files = ModelFiles(d)
+    base = config.spec(files.names())
+    H, E, I, rot, step = base.hidden_size, 3, 40, 8, 0.07
+    l0, l1 = base.layers
+    mixer0 = l0.parts["mixer"]
+    mixer0 = dataclasses.replace(mixer0, parts=dict(mixer0.parts, position=PartSpec("position", "toy_schedule", {"rotary_dim": rot, "step": step})))
+    l0 = dataclasses.replace(l0, parts=dict(l0.parts, mixer=mixer0))
+    routed = PartSpec("feed_forward", "toy_routed", {"experts": E},
+                      {"router": tensor("toy.router", (E, H)), "a": tensor("toy.a", (E * I, H)), "b": tensor("toy.b", (E * H, I))})
+    centered = PartSpec("norm", "toy_centered", {"eps": 1e-5}, {"weight": tensor("toy.norm", (H,), "vector")})
+    l1 = dataclasses.replace(l1, parts=dict(l1.parts, feed_forward=routed, feed_forward_norm=centered))
+    spec = dataclasses.replace(base, layers=(l0, l1))
+    g = torch.Generator().manual_seed(5)
+    extra = {("toy.router",): torch.randn(E, H, generator=g).to(tdt), ("toy.a",): (torch.randn(E * I, H, generator=g) * 0.3).to(tdt),
+             ("toy.b",): (torch.randn(E * H, I, generator=g) * 0.3).to(tdt), ("toy.norm",): torch.rand(H, generator=g) + 0.5}
+    weights = ExtraWeights(load_weights(base, files, tdt, DEV), {k: v.to(DEV) for k, v in extra.items()})
+    eng = Engine(config, spec, weights, tdt, max_tokens=64 * 8)
+
+    cfg, w = P.read_model(d)
+    S = P.sizes(cfg)
+    nh, nkv, hd = S["nh"], S["nkv"], S["hd"]
+
+    def plain(ids):
+        n = len(ids)
+        pos = torch.arange(n, dtype=torch.float64)
+        x = P.embedding(w["model.embed_tokens.weight"], ids)
+        # layer 0 with the toy rotation
+        p = "model.layers.0."
+        h = P.rms_norm(x, w[p + "input_layernorm.weight"], S["eps"])
+        a = p + "self_attn."
+        q = P.rms_norm(P.linear(h, w[a + "q_proj.weight"]).reshape(n, nh, hd), w[a + "q_norm.weight"], S["eps"])
+        k = P.rms_norm(P.linear(h, w[a + "k_proj.weight"]).reshape(n, nkv, hd), w[a + "k_norm.weight"], S["eps"])
+        v = P.linear(h, w[a + "v_proj.weight"]).reshape(n, nkv, hd)
+        # the part makes its angles in 32-bit: position * (step * (i + 1))
+        i = torch.arange(1, rot // 2 + 1, dtype=torch.float32)
+        ang = (torch.arange(n, dtype=torch.float32)[:, None] * (step * i)[None, :]).double()
+        q, k = _rope_interleaved(q, ang.cos(), ang.sin(), rot), _rope_interleaved(k, ang.cos(), ang.sin(), rot)
+        x = x + P.linear(P.causal_attention(q, k, v, hd ** -0.5).reshape(n, -1), w[a + "o_proj.weight"])
+        h = P.rms_norm(x, w[p + "post_attention_layernorm.weight"], S["eps"])
+        x = x + P.swiglu_mlp(h, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+        # layer 1: plain attention, centered norm, routed experts
+        p = "model.layers.1."
+        h = P.rms_norm(x, w[p + "input_layernorm.weight"], S["eps"])
+        x = x + P.attention_block(h, w, p + "self_attn.", S, list(range(n)), None)
+        c = x - x.mean(-1, keepdim=True)
+        h = c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + 1e-5) * extra[("toy.norm",)].double()
+        if dtype == "bfloat16":
+            h = h.to(torch.bfloat16).double()                   # the choice of expert is made from the rounded rows
+        choice = (h.float() @ extra[("toy.router",)].float().T).argmax(-1)
+        A = extra[("toy.a",)].double().reshape(E, I, H)
+        B = extra[("toy.b",)].double().reshape(E, H, I)
+        hid = torch.relu(torch.einsum("th,tih->ti", h, A[choice]))
+        x = x + torch.einsum("ti,thi->th", hid, B[choice])
+        return P.linear(P.rms_norm(x, w["model.norm.weight"], S["eps"]), P.head_weight(w)), choice
+
+    reqs = tiny.prompts("A", [45, 12, 70], seed=23)
+    slots = [eng.open() for _ in reqs]
+    cuts = [40, 3, 33]                                           # a long piece, a short one (few rows: products fold norms in), a middle one
+    out = eng.step([StepEntry(s, r[:c], list(range(c))) for s, r, c in zip(slots, reqs, cuts)])
+    got, o = {i: [] for i in range(3)}, 0
+    for i, c in enumerate(cuts):
+        got[i].append(out[o:o + c]); o += c
+    fed = list(cuts)
+    while any(fed[i] < len(reqs[i]) for i in range(3)):
+        live = [i for i in range(3) if fed[i] < len(reqs[i])]
+        out = eng.step([StepEntry(slots[i], [reqs[i][fed[i]]], [0]) for i in live])
+        for r_, i in enumerate(live):
+            got[i].append(out[r_:r_ + 1]); fed[i] += 1
+    for i in range(3):
+        ref, choice = plain(reqs[i])
+        assert len(set(choice.tolist())) > 1                     # the router does choose
+        tiny.assert_logits_close(torch.cat(got[i]), ref, dtype, f"toy norm, routing and rotation, request {i}")
+        eng.close(slots[i])
+    eng.cache.check()
