@@ -33,6 +33,11 @@ constexpr int KSTEPS = (CHUNKS + 3) / 4;     // MFMA steps over d (32 values eac
 constexpr int DTILES = HD / 16;              // 16-row tiles of O^T
 constexpr float LOG2E = 1.4426950408889634f;
 
+// 2^x as the one hardware instruction.  The library's exp2f wraps it in a rescaling so that results below
+// 2^-126 come out as denormals; a softmax weight that small adds nothing to a sum whose largest term is 1, and
+// the wrapper costs a quarter of the kernel's vector instructions.  Arguments here are <= 0 (or -inf, giving 0).
+__device__ inline float exp2_weight(float x) { return __builtin_amdgcn_exp2f(x); }
+
 PALM_DEFINE_LAST_ERROR()
 PALM_API int palm_attention_head_dim() { return HD; }
 
@@ -106,13 +111,13 @@ __device__ inline float score_page(const PageOperands& ops, const bf16x8 (&qv)[K
     // border inside a tile of queries): its maximum is still -inf then; subtracting 0 instead keeps
     // every exponential at exp2(-inf) = 0 rather than NaN.
     const float m_sub = m_new == -INFINITY ? 0.f : m_new;
-    const float alpha = exp2f(c.m - m_sub);             // c.m = -inf before the first visible key: 0
+    const float alpha = exp2_weight(c.m - m_sub);       // c.m = -inf before the first visible key: 0
     float sum = 0.f;
 #pragma unroll
     for (int h = 0; h < 2; ++h)
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-            const float p = exp2f(s[2 * h + e / 4][e % 4] - m_sub);
+            const float p = exp2_weight(s[2 * h + e / 4][e % 4] - m_sub);
             sum += p;
             pv[h][e] = (__bf16)p;
         }
@@ -421,13 +426,13 @@ __device__ inline void unit_scores(const bf16_t* k_lds, Unit (&u)[PF_UNITS], int
         mx *= scale_log2;                                           // the scale is positive: the maximum commutes with it
         const float m_new = fmaxf(c.m, mx);
         const float m_sub = m_new == -INFINITY ? 0.f : m_new;       // see score_page
-        alpha[x] = exp2f(c.m - m_sub);
+        alpha[x] = exp2_weight(c.m - m_sub);
         float sum = 0.f;
 #pragma unroll
         for (int h = 0; h < 2; ++h)
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                const float p = exp2f(fmaf(s[x][2 * h + e / 4][e % 4], scale_log2, -m_sub));
+                const float p = exp2_weight(fmaf(s[x][2 * h + e / 4][e % 4], scale_log2, -m_sub));
                 sum += p;
                 pv[x][h][e] = (__bf16)p;
             }
@@ -487,13 +492,13 @@ __global__ __launch_bounds__(PF_THREADS) PF_WAVES_PER_SIMD void attention_prefil
 
     const int b = blockIdx.z;
     const int G = nh / nkv, n_hg = (G + hg - 1) / hg;
-    const int kvh = blockIdx.y / n_hg, hgi = blockIdx.y % n_hg;
+    const int kvh = blockIdx.x / n_hg, hgi = blockIdx.x % n_hg;       // the kv head runs fastest over the blocks, see the launch
     const int n_new = seq_new[b];
     // the block's sub-tiles of 16 queries: number s is, for even s, sub-tile f = first + s / 2 from the front, for
     // odd s its partner n16 - 1 - f from the back (none if f is the middle one); a single sub-tile a block (eight
     // heads a group) just counts from the back, the long ones first
     const int subs = qb / 16, n16 = (n_new + 15) / 16;
-    const int first_front = blockIdx.x * (subs > 1 ? subs / 2 : 1);
+    const int first_front = blockIdx.y * (subs > 1 ? subs / 2 : 1);
     if (subs > 1 ? 2 * first_front > n16 - 1 : first_front >= n16) return;
     auto sub_tile = [&](int sub) -> int {                       // the sub-tile's index, or -1
         if (subs == 1) return n16 - 1 - first_front;
@@ -610,7 +615,12 @@ PALM_API int palm_attention_prefill(hipStream_t stream, const void* q, const voi
     const int n_hg = (G + hg - 1) / hg;
     PALM_CHECK(nkv * n_hg <= 65535 && n_seqs <= 65535, "attention_prefill: grid too large");
     const int n16 = (max_new + 15) / 16, subs = qb / 16;
-    dim3 grid(subs > 1 ? ((n16 + 1) / 2 + subs / 2 - 1) / (subs / 2) : n16, nkv * n_hg, n_seqs);
+    // Blocks are handed to the chip's eight dies in turn by their number, and each die has an L2 of its own.  With
+    // the kv head as the fastest index, the blocks that a die gets belong to few kv heads (one, with eight of
+    // them), whose keys and values then stay in that die's L2 for all the query tiles that read them.
+    const int n_tiles = subs > 1 ? ((n16 + 1) / 2 + subs / 2 - 1) / (subs / 2) : n16;
+    PALM_CHECK(n_tiles <= 65535, "attention_prefill: %d new tokens are more than one launch takes", max_new);
+    dim3 grid(nkv * n_hg, n_tiles, n_seqs);
     attention_prefill_kernel<<<grid, PF_THREADS, 0, stream>>>((const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache,
                                                              block_table, max_pages, seq_slot, seq_start, seq_new, cu_new, nh,
                                                              nkv, scale * LOG2E, window, qb, hg, (bf16_t*)out);
