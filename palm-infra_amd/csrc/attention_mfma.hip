@@ -172,7 +172,8 @@ __device__ inline void load_query(const bf16_t* qrow, bool valid, int g, bf16x8 
 
 // ---- decode ---------------------------------------------------------------------------------------
 // grid (slices, nkv * query groups, sequences), one wave each.  Workspace per (sequence, head, slice):
-// m, l, then HD floats of the unnormalised output.
+// m, l, two floats unused, then HD floats of the unnormalised output (which so start on 16 bytes).
+constexpr int WORK_O = 4, WORK_STRIDE = HD + WORK_O;
 #if PALM_HEAD_DIM <= 128
 #define DECODE_WAVES_PER_SIMD __attribute__((amdgpu_waves_per_eu(2)))     // fits without spilling up to this head size
 #else
@@ -213,17 +214,19 @@ __global__ __launch_bounds__(WAVE) DECODE_WAVES_PER_SIMD void attention_decode_k
         const float inv = 1.0f / l;
         bf16_t* o = out + ((size_t)b * nh + head) * HD;
 #pragma unroll
-        for (int dt = 0; dt < DTILES; ++dt)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) o[dt * 16 + 4 * g + i] = f32_to_bf16(c.o[dt][i] * inv);
+        for (int dt = 0; dt < DTILES; ++dt) {
+            uint2 four;
+            four.x = (uint32_t)f32_to_bf16(c.o[dt][0] * inv).bits | ((uint32_t)f32_to_bf16(c.o[dt][1] * inv).bits << 16);
+            four.y = (uint32_t)f32_to_bf16(c.o[dt][2] * inv).bits | ((uint32_t)f32_to_bf16(c.o[dt][3] * inv).bits << 16);
+            *reinterpret_cast<uint2*>(o + dt * 16 + 4 * g) = four;
+        }
         return;
     }
-    float* w = work + (((size_t)b * nh + head) * n_slices + slice) * (HD + 2);
+    float* w = work + (((size_t)b * nh + head) * n_slices + slice) * WORK_STRIDE;
     if (g == 0) { w[0] = c.m; w[1] = l; }               // an empty slice leaves m = -inf, l = 0
 #pragma unroll
-    for (int dt = 0; dt < DTILES; ++dt)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) w[2 + dt * 16 + 4 * g + i] = c.o[dt][i];
+    for (int dt = 0; dt < DTILES; ++dt)                    // the lane's four elements of a tile lie side by side: one store
+        *reinterpret_cast<float4*>(w + WORK_O + dt * 16 + 4 * g) = make_float4(c.o[dt][0], c.o[dt][1], c.o[dt][2], c.o[dt][3]);
 }
 
 // One wave per (sequence, head): merge the slices in a fixed order.  Lane s first reads slice s's maximum
@@ -231,13 +234,13 @@ __global__ __launch_bounds__(WAVE) DECODE_WAVES_PER_SIMD void attention_decode_k
 // output element d over the slices, eight reads in flight at a time.
 __global__ __launch_bounds__(WAVE) void attention_merge_kernel(const float* __restrict__ work, int n_slices,
                                                                bf16_t* __restrict__ out) {
-    const float* w = work + (size_t)blockIdx.x * n_slices * (HD + 2);
+    const float* w = work + (size_t)blockIdx.x * n_slices * WORK_STRIDE;
     const int lane = threadIdx.x;
     float m = -INFINITY;
-    for (int s = lane; s < n_slices; s += WAVE) m = fmaxf(m, w[(size_t)s * (HD + 2)]);
+    for (int s = lane; s < n_slices; s += WAVE) m = fmaxf(m, w[(size_t)s * WORK_STRIDE]);
     m = wave_max(m);
     float l = 0.f;
-    for (int s = lane; s < n_slices; s += WAVE) l += w[(size_t)s * (HD + 2) + 1] * exp2f(w[(size_t)s * (HD + 2)] - m);
+    for (int s = lane; s < n_slices; s += WAVE) l += w[(size_t)s * WORK_STRIDE + 1] * exp2f(w[(size_t)s * WORK_STRIDE] - m);
     l = wave_sum(l);
     constexpr int PER = (HD + WAVE - 1) / WAVE;
     float o[PER];
@@ -248,11 +251,11 @@ __global__ __launch_bounds__(WAVE) void attention_merge_kernel(const float* __re
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
             const int s = min(s0 + u, n_slices - 1);
-            ms[u] = w[(size_t)s * (HD + 2)];
+            ms[u] = w[(size_t)s * WORK_STRIDE];
 #pragma unroll
             for (int i = 0; i < PER; ++i) {
                 const int d = min(lane + i * WAVE, HD - 1);
-                v[u][i] = w[(size_t)s * (HD + 2) + 2 + d];
+                v[u][i] = w[(size_t)s * WORK_STRIDE + WORK_O + d];
             }
         }
 #pragma unroll
@@ -270,7 +273,7 @@ __global__ __launch_bounds__(WAVE) void attention_merge_kernel(const float* __re
 }
 
 PALM_API int palm_attention_decode_workspace_floats(int n_seqs, int nh, int n_slices) {
-    return n_seqs * nh * n_slices * (HD + 2);
+    return n_seqs * nh * n_slices * WORK_STRIDE;
 }
 
 PALM_API int palm_attention_decode(hipStream_t stream, const void* q, const void* k_cache, const void* v_cache,
@@ -486,8 +489,10 @@ __global__ __launch_bounds__(PF_THREADS) PF_WAVES_PER_SIMD void attention_prefil
     const int* __restrict__ seq_start, const int* __restrict__ seq_new, const int* __restrict__ cu_new, int nh,
     int nkv, float scale_log2, int window, int qb, int hg, bf16_t* __restrict__ out) {
     constexpr int K_TILE = PAGE_TOKENS * K_STRIDE, V_TILE = HD * V_STRIDE;
-    __shared__ __attribute__((aligned(16))) bf16_t k_lds[PF_SHARE && V_TILE > K_TILE ? V_TILE : K_TILE];
-    __shared__ __attribute__((aligned(16))) bf16_t v_own[PF_SHARE ? 8 : V_TILE];
+    // Head sizes whose pages fit twice keep two pages of K and of V^T in LDS: while one is used the next is laid
+    // down beside it, and one barrier a page is enough.  Larger heads share one buffer between K and V^T.
+    __shared__ __attribute__((aligned(16))) bf16_t k_lds[PF_SHARE ? (V_TILE > K_TILE ? V_TILE : K_TILE) : 2 * K_TILE];
+    __shared__ __attribute__((aligned(16))) bf16_t v_own[PF_SHARE ? 8 : 2 * V_TILE];
     bf16_t* v_lds = PF_SHARE ? k_lds : v_own;
 
     const int b = blockIdx.z;
@@ -551,37 +556,64 @@ __global__ __launch_bounds__(PF_THREADS) PF_WAVES_PER_SIMD void attention_prefil
         prefetch_keys(k_cache + base, pf);
         prefetch_values(v_cache + base, pf);
     }
-    for (int p = p_lo; p <= p_hi; ++p) {
-        const bool more = p < p_hi;
-        const size_t next = more ? ((size_t)pages[p + 1] * nkv + kvh) * PAGE_TOKENS * HD : 0;
-        bf16x8 pv[PF_UNITS][2];
-        float alpha[PF_UNITS];
-        __syncthreads();                                        // everyone is done with the previous page
-        stage_keys(pf, k_lds);
-        if (!PF_SHARE) stage_values(pf, v_lds);
-        __syncthreads();
-        if (more) prefetch_keys(k_cache + next, pf);            // in flight while this page is used
-        // is every key of this page visible to every column of this wave that takes part?
+    // is every key of page p visible to every column of this wave that takes part?  (also marks who does)
+    auto page_is_interior = [&](int p) -> bool {
         bool inside = true;
 #pragma unroll
         for (int x = 0; x < PF_UNITS; ++x) {
             u[x].active = u[x].live && p >= u[x].page_lo && p <= u[x].page_hi;
             inside = inside && (!u[x].active || (u[x].first <= p * PAGE_TOKENS && u[x].pos >= p * PAGE_TOKENS + PAGE_TOKENS - 1));
         }
-        const bool interior = __all(inside);
-        unit_scores(k_lds, u, p * PAGE_TOKENS, scale_log2, r, g, interior, pv, alpha);
-        bool moved = false;
+        return __all(inside);
+    };
+    if (!PF_SHARE) {
+        stage_keys(pf, k_lds);
+        stage_values(pf, v_lds);
+        __syncthreads();
+        for (int p = p_lo; p <= p_hi; ++p) {
+            const int buf = (p - p_lo) & 1;
+            const bool more = p < p_hi;
+            if (more) {                                         // in flight while this page is used
+                const size_t next = ((size_t)pages[p + 1] * nkv + kvh) * PAGE_TOKENS * HD;
+                prefetch_keys(k_cache + next, pf);
+                prefetch_values(v_cache + next, pf);
+            }
+            bf16x8 pv[PF_UNITS][2];
+            float alpha[PF_UNITS];
+            const bool interior = page_is_interior(p);
+            unit_scores(k_lds + buf * K_TILE, u, p * PAGE_TOKENS, scale_log2, r, g, interior, pv, alpha);
+            bool moved = false;
 #pragma unroll
-        for (int x = 0; x < PF_UNITS; ++x) moved = moved || alpha[x] != 1.0f;
-        const bool rescale = __any(moved);
-        if (PF_SHARE) {
+            for (int x = 0; x < PF_UNITS; ++x) moved = moved || alpha[x] != 1.0f;
+            unit_values(v_lds + buf * V_TILE, u, r, g, pv, alpha, __any(moved));
+            if (more) {                                         // the other buffer's last readers passed the barrier a page ago
+                stage_keys(pf, k_lds + (buf ^ 1) * K_TILE);
+                stage_values(pf, v_lds + (buf ^ 1) * V_TILE);
+            }
+            __syncthreads();
+        }
+    } else {
+        for (int p = p_lo; p <= p_hi; ++p) {
+            const bool more = p < p_hi;
+            const size_t next = more ? ((size_t)pages[p + 1] * nkv + kvh) * PAGE_TOKENS * HD : 0;
+            bf16x8 pv[PF_UNITS][2];
+            float alpha[PF_UNITS];
+            __syncthreads();                                    // everyone is done with the previous page
+            stage_keys(pf, k_lds);
+            __syncthreads();
+            if (more) prefetch_keys(k_cache + next, pf);        // in flight while this page is used
+            const bool interior = page_is_interior(p);
+            unit_scores(k_lds, u, p * PAGE_TOKENS, scale_log2, r, g, interior, pv, alpha);
+            bool moved = false;
+#pragma unroll
+            for (int x = 0; x < PF_UNITS; ++x) moved = moved || alpha[x] != 1.0f;
+            const bool rescale = __any(moved);
             __syncthreads();
             stage_values(pf, v_lds);
             __syncthreads();
+            unit_values(v_lds, u, r, g, pv, alpha, rescale);
+            if (more) prefetch_values(v_cache + next, pf);
         }
-        if (more && !PF_SHARE) prefetch_values(v_cache + next, pf);
-        unit_values(v_lds, u, r, g, pv, alpha, rescale);
-        if (more && PF_SHARE) prefetch_values(v_cache + next, pf);
     }
 
 #pragma unroll
@@ -593,9 +625,12 @@ __global__ __launch_bounds__(PF_THREADS) PF_WAVES_PER_SIMD void attention_prefil
             const float inv = 1.0f / l;
             bf16_t* o = out + (u[x].row * nh + u[x].head) * HD;
 #pragma unroll
-            for (int dt = 0; dt < DTILES; ++dt)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) o[dt * 16 + 4 * g + i] = f32_to_bf16(u[x].c.o[dt][i] * inv);
+            for (int dt = 0; dt < DTILES; ++dt) {               // the lane's four elements of a tile lie side by side: one store
+                uint2 four;
+                four.x = (uint32_t)f32_to_bf16(u[x].c.o[dt][0] * inv).bits | ((uint32_t)f32_to_bf16(u[x].c.o[dt][1] * inv).bits << 16);
+                four.y = (uint32_t)f32_to_bf16(u[x].c.o[dt][2] * inv).bits | ((uint32_t)f32_to_bf16(u[x].c.o[dt][3] * inv).bits << 16);
+                *reinterpret_cast<uint2*>(o + dt * 16 + 4 * g) = four;
+            }
         }
     }
 }

@@ -459,7 +459,7 @@ def attention_decode(q, k_cache, v_cache, block_table, seq_slot, seq_start, nh: 
     B = seq_slot.shape[0]
     _need(q.shape[0] == B and seq_start.shape == (B,), "attention_decode: one query, slot and start for each sequence")
     out = torch.empty_like(q)
-    work = torch.empty((B * nh * n_slices * (hd + 2),), dtype=F32, device=q.device) if n_slices > 1 else None
+    work = torch.empty((B * nh * n_slices * (hd + 4),), dtype=F32, device=q.device) if n_slices > 1 else None
     library.call(attention_lib(hd), "palm_attention_decode", _stream(), _p(q), _p(k_cache), _p(v_cache), _p(block_table),
                  block_table.shape[1], _p(seq_slot), _p(seq_start), B, nh, nkv, hd, float(scale), int(window or 0),
                  int(n_slices), _p(work), _p(out))
