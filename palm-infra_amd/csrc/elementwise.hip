@@ -147,7 +147,11 @@ static bool launch_rmsnorm_fast(hipStream_t stream, void* x, const void* delta, 
                                 const int* rows, int n_out_rows, int width, void* out, int update_x) {
     if (width % 4 != 0 || width > 32768) return false;
     const int quads = width / 4;
-    const int iters = quads <= 256 ? 1 : (quads <= 512 ? 2 : (quads <= 1024 ? 4 : 8));
+    int iters = quads <= 256 ? 1 : (quads <= 512 ? 2 : (quads <= 1024 ? 4 : 8));
+    if (planes > 1 && iters > 4) {                          // eight quads of several planes do not fit a thread's registers:
+        if (quads > 4096) return false;                     // more threads with four quads each, as far as a block goes
+        iters = 4;
+    }
     int threads = (quads + iters - 1) / iters;
     threads = (threads + WAVE - 1) / WAVE * WAVE;
     if (threads > 1024) return false;

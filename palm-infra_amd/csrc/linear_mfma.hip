@@ -269,11 +269,9 @@ __global__ __launch_bounds__(STREAM_WAVES * WAVE) void linear_stream_kernel(cons
                 for (int j = 0; j < 4; ++j) {
                     bf16x8 wj = wv[u][j];
                     bf16x8 xj = AREG ? xa[AREG && t + u < TREG ? t + u : 0][j] : xv[u][j];
-                    if (!EXACT) {
-                        const bool ok = (present[u] >> j) & 1;
-                        wj = ok ? wj : zero_bf16x8();
-                        if (!AREG) xj = ok ? xj : zero_bf16x8();
-                    }
+                    // a chunk beyond K counts as zeros: it is enough that the activations do (held in registers they
+                    // were zeroed when read); the weights read in their place are the row's first, finite if any are
+                    if (!EXACT && !AREG) xj = ((present[u] >> j) & 1) ? xj : zero_bf16x8();
                     acc = mfma_16x16x32(wj, xj, acc);
                 }
                 if (decltype(refill)::value) ask(u);
@@ -339,9 +337,11 @@ static int stream_steps(int n_super, int parts) {
     return (per_part + STREAM_WAVES - 1) / STREAM_WAVES;
 }
 
-// The steps the kernel variants make for a wish of `steps`: 2 or 4 with the activations in registers, else a
-// multiple of 4.
-static int stream_steps_served(int steps) { return steps <= 2 ? 2 : (steps + 3) / 4 * 4; }
+// The steps the kernel variants make for a wish of `steps`: 2, 4, 6 or 8 with the activations in registers
+// (K up to 8192), else a multiple of 4 with the activations read beside the weights, which for more than a few
+// rows is much the slower way (2 against 5 TB/s at 16 rows).
+constexpr int STREAM_MAX_REG_STEPS = 8;
+static int stream_steps_served(int steps) { return steps <= STREAM_MAX_REG_STEPS ? (steps + 1) / 2 * 2 : (steps + 3) / 4 * 4; }
 
 // Into how many ranges K is best cut for an [M, K] x [N, K]^T product whose reader can add planes: enough
 // to give every compute unit two or three blocks, no fewer than two steps for a wave, and no range empty.
@@ -350,6 +350,8 @@ static int stream_parts(int M, int N, int K) {
     if (M > 16 || n_super < 16) return 1;
     const int strips = (N + 15) / 16;
     int parts = max(1, min(min(768 / strips, n_super / (2 * STREAM_WAVES)), 4));
+    // and enough to let a wave keep its share of the activations in registers
+    parts = max(parts, min(4, (n_super + STREAM_MAX_REG_STEPS * STREAM_WAVES - 1) / (STREAM_MAX_REG_STEPS * STREAM_WAVES)));
     for (;;) {      // rounding the steps up can leave the last ranges without work: fewer ranges then
         const int covered = stream_steps_served(stream_steps(n_super, parts)) * STREAM_WAVES;
         const int needed = (n_super + covered - 1) / covered;
@@ -367,7 +369,8 @@ static void launch_stream(hipStream_t stream, const void* a, const void* w, void
     T = (T + U - 1) / U * U;
     if (TREG > 0) T = TREG;
     // every block the same number of strips, as far as that goes
-    const int slots = parts > 1 ? max(1, STREAM_SLOTS_CUT / parts) : STREAM_SLOTS;
+    // (with six or eight steps of activations in registers only one block fits a compute unit)
+    const int slots = TREG > 4 ? max(1, 256 / parts) : (parts > 1 ? max(1, STREAM_SLOTS_CUT / parts) : STREAM_SLOTS);
     const int rounds = (strips + slots - 1) / slots;
     const dim3 grid((strips + rounds - 1) / rounds, parts);
     const bool exact = K % SUPER_K == 0 && parts * T * STREAM_WAVES == n_super;
@@ -389,6 +392,8 @@ static void dispatch_thin(hipStream_t stream, const void* a, const void* w, void
         const int per_wave = stream_steps(n_super, parts);
         if (per_wave <= 2) launch_stream<2, 2, TC, EPI>(stream, a, w, c, M, N, K, parts, norm);
         else if (per_wave <= 4) launch_stream<2, 4, TC, EPI>(stream, a, w, c, M, N, K, parts, norm);
+        else if (per_wave <= 6) launch_stream<2, 6, TC, EPI>(stream, a, w, c, M, N, K, parts, norm);
+        else if (per_wave <= 8) launch_stream<2, 8, TC, EPI>(stream, a, w, c, M, N, K, parts, norm);
         else launch_stream<4, 0, TC, EPI>(stream, a, w, c, M, N, K, parts, norm);
         return;
     }

@@ -318,6 +318,7 @@ def linear_library(a: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
 
 
 THIN_TOKENS = 16      # up to here every wave fetches its own activations; above, a block shares them through LDS
+FOLD_MAX_K = 12288    # up to this K a product of 9 to 16 rows folds a norm in; the thin kernel holds activations in registers up to 8192
 
 
 def thin_serves(a: torch.Tensor, w: torch.Tensor) -> bool:

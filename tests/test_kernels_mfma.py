@@ -24,7 +24,8 @@ def rand(*shape, seed=0, scale=1.0, dtype=BF16):
 
 @pytest.mark.parametrize("M", [1, 8, 16, 17, 33, 64, 70, 150])
 @pytest.mark.parametrize("N,K", [(7, 8), (130, 64), (515, 80), (1000, 224), (96, 4096), (4096, 1536), (300, 12288),
-                                 (1000, 2048), (515, 2056), (130, 5000), (9000, 2048), (8200, 3080)])
+                                 (1000, 2048), (515, 2056), (130, 5000), (9000, 2048), (8200, 3080), (64, 8192), (48, 7000),
+                                 (4200, 5120)])
 def test_linear_thin_against_the_plain_product(ops, M, N, K):
     a, w = rand(M, K, seed=M + K), rand(N, K, seed=N, scale=0.5)
     ref = P.linear(a, w)
@@ -37,7 +38,7 @@ def test_linear_thin_against_the_plain_product(ops, M, N, K):
 
 @pytest.mark.parametrize("M", [1, 8, 16])
 @pytest.mark.parametrize("N,K,planes", [(4096, 4096, 2), (2048, 12288, 3), (1000, 12288, 3), (6144, 4096, 2), (4096, 6000, 2),
-                                        (4096, 2048, 1), (16384, 4096, 1), (515, 520, 1)])
+                                        (4096, 2048, 1), (16384, 4096, 1), (515, 520, 1), (5120, 17408, 3), (2048, 25600, 4)])
 def test_linear_thin_as_planes_of_partial_sums(ops, M, N, K, planes):
     a, w = rand(M, K, seed=M, dtype=BF16), rand(N, K, seed=N + K, dtype=BF16)
     got = ops.linear_thin(a.to(DEV), w.to(DEV), F32, planes_ok=True).cpu()
@@ -123,7 +124,8 @@ def test_linear_thin_orientation(ops):
 
 
 @pytest.mark.parametrize("M", [1, 8, 20, 64])
-@pytest.mark.parametrize("I,K", [(5, 16), (176, 80), (224, 96), (1536, 512), (4500, 2048), (300, 3000), (100, 6000)])
+@pytest.mark.parametrize("I,K", [(5, 16), (176, 80), (224, 96), (1536, 512), (4500, 2048), (300, 3000), (100, 6000), (2200, 5120),
+                                 (40, 8192)])
 def test_linear_thin_gated(ops, M, I, K):
     a, w = rand(M, K, seed=M), rand(2 * I, K, seed=I, scale=0.3)
     g, u = P.linear(a, w[:I]), P.linear(a, w[I:])
