@@ -132,8 +132,10 @@ static void launch_thin(hipStream_t stream, const void* a, const void* w, void* 
 // registers; with TREG == 0 it is read again beside every weight read.  At eight rows the register form is
 // what brings the gated product from 45 to 36 us and the head from 260 to 212 us: an activation read costs
 // the cache path as much as a weight read although it brings nothing new.
-// T: steps a wave makes for one strip, a multiple of U; steps beyond K read nothing and count as zeros
-// (EXACT says there are none, and then nothing is masked).
+// T: steps a wave makes for one strip, a multiple of U; steps beyond K read the row's start and count as zeros
+// (EXACT says there are none, and then nothing is checked: 3% of a decode step at Qwen3-8B's sizes).
+// NW: waves a block, 8, or 4 for a K of fewer than 32 super-steps, which eight waves would share out badly
+// (K = 2560: 20 super-steps are 3 steps for each of eight waves with 12 of 32 turns idle, but 5 for each of four).
 // Few strips and a long K (an output projection: 256 strips) leave most of the chip without work.  Then K is
 // cut into `parts` ranges, blockIdx.y names the range, and the block writes its partial sums to plane
 // blockIdx.y of a [parts, M, N] float32 result; whoever reads the result adds the planes in their order (the
@@ -159,18 +161,18 @@ struct RowNorm {
     float* ss_out;           // [M, strips]
 };
 
-constexpr int STREAM_WAVES = 8;
-constexpr int STREAM_SLOTS = 512;      // blocks that run at once: two on each of 256 compute units
-constexpr int STREAM_SLOTS_CUT = 768;  // with K cut into ranges a block's work is short: three
+constexpr int STREAM_WAVE_SLOTS = 4096;     // waves that run at once in the usual launch: 16 on each of 256 compute units
+constexpr int STREAM_WAVE_SLOTS_CUT = 6144; // with K cut into ranges a block's work is short: 24
 
-template <int U, int TREG, bool EXACT, typename TC, int EPI>
-__global__ __launch_bounds__(STREAM_WAVES * WAVE) void linear_stream_kernel(const bf16_t* __restrict__ A,
-                                                                            const bf16_t* __restrict__ W,
-                                                                            TC* __restrict__ C, int M, int N, int K,
-                                                                            int n_strips, int T_given, RowNorm norm) {
+template <int NW, int U, int TREG, bool EXACT, typename TC, int EPI>
+__global__ __launch_bounds__(NW * WAVE) void linear_stream_kernel(const bf16_t* __restrict__ A,
+                                                                  const bf16_t* __restrict__ W,
+                                                                  TC* __restrict__ C, int M, int N, int K,
+                                                                  int n_strips, int T_given, RowNorm norm) {
     // this block's range of K starts at super-step blockIdx.y * T * NW, its results go to plane blockIdx.y
-    constexpr int NW = STREAM_WAVES;
     constexpr bool AREG = TREG > 0;
+    constexpr int PER = NW * 4;                  // threads that share a row's sum of squares
+    static_assert(NW == 4 || NW == 8, "the epilogues count on 256 or 512 threads");
     __shared__ float part[2][NW][16][17];
     __shared__ float row_factor[16];
     const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
@@ -229,23 +231,23 @@ __global__ __launch_bounds__(STREAM_WAVES * WAVE) void linear_stream_kernel(cons
     }
 
     __builtin_amdgcn_sched_barrier(0);       // the weight reads above go out first, whatever follows
-    // The rows' factors: 32 threads a row add up the pieces, every block in the same order.  The reads go out
+    // The rows' factors: PER threads a row add up the pieces, every block in the same order.  The reads go out
     // here and are used only when the first strip's products are done, so nothing waits for them.
-    const int f_col = min((int)threadIdx.x / 32, M - 1), f_piece = threadIdx.x % 32;
+    const int f_col = min((int)threadIdx.x / PER, M - 1), f_piece = threadIdx.x % PER;
     float piece[8];
     if (norm.ss_in) {
 #pragma unroll
         for (int u = 0; u < 8; ++u)
-            piece[u] = norm.ss_in[(size_t)f_col * norm.pieces_in + min(f_piece + 32 * u, norm.pieces_in - 1)];
+            piece[u] = norm.ss_in[(size_t)f_col * norm.pieces_in + min(f_piece + PER * u, norm.pieces_in - 1)];
     }
     auto publish_row_factors = [&]() {
         float sum = 0.f;
 #pragma unroll
-        for (int u = 0; u < 8; ++u) sum += f_piece + 32 * u < norm.pieces_in ? piece[u] : 0.f;
-        for (int p = 256 + f_piece; p < norm.pieces_in; p += 32) sum += norm.ss_in[(size_t)f_col * norm.pieces_in + p];
+        for (int u = 0; u < 8; ++u) sum += f_piece + PER * u < norm.pieces_in ? piece[u] : 0.f;
+        for (int p = PER * 8 + f_piece; p < norm.pieces_in; p += PER) sum += norm.ss_in[(size_t)f_col * norm.pieces_in + p];
 #pragma unroll
-        for (int off = 16; off > 0; off >>= 1) sum += __shfl_xor(sum, off, WAVE);
-        if (f_piece == 0) row_factor[threadIdx.x / 32] = 1.0f / sqrtf(sum / (float)norm.width_in + norm.eps_in);
+        for (int off = PER / 2; off > 0; off >>= 1) sum += __shfl_xor(sum, off, WAVE);
+        if (f_piece == 0) row_factor[threadIdx.x / PER] = 1.0f / sqrtf(sum / (float)norm.width_in + norm.eps_in);
     };
 
     int buf = 0;
@@ -331,10 +333,14 @@ __global__ __launch_bounds__(STREAM_WAVES * WAVE) void linear_stream_kernel(cons
     }
 }
 
+// waves a block: eight, or four when K has fewer than 32 super-steps
+static int stream_waves(int n_super) { return n_super < 32 ? 4 : 8; }
+
 // steps a wave makes for one strip when K is cut into `parts` ranges
 static int stream_steps(int n_super, int parts) {
     const int per_part = (n_super + parts - 1) / parts;
-    return (per_part + STREAM_WAVES - 1) / STREAM_WAVES;
+    const int nw = stream_waves(n_super);
+    return (per_part + nw - 1) / nw;
 }
 
 // The steps the kernel variants make for a wish of `steps`: 2, 4, 6 or 8 with the activations in registers
@@ -348,19 +354,20 @@ static int stream_steps_served(int steps) { return steps <= STREAM_MAX_REG_STEPS
 static int stream_parts(int M, int N, int K) {
     const int n_super = (K + SUPER_K - 1) / SUPER_K;
     if (M > 16 || n_super < 16) return 1;
+    const int nw = stream_waves(n_super);
     const int strips = (N + 15) / 16;
-    int parts = max(1, min(min(768 / strips, n_super / (2 * STREAM_WAVES)), 4));
+    int parts = max(1, min(min(768 / strips, n_super / (2 * nw)), 4));
     // and enough to let a wave keep its share of the activations in registers
-    parts = max(parts, min(4, (n_super + STREAM_MAX_REG_STEPS * STREAM_WAVES - 1) / (STREAM_MAX_REG_STEPS * STREAM_WAVES)));
+    parts = max(parts, min(4, (n_super + STREAM_MAX_REG_STEPS * nw - 1) / (STREAM_MAX_REG_STEPS * nw)));
     for (;;) {      // rounding the steps up can leave the last ranges without work: fewer ranges then
-        const int covered = stream_steps_served(stream_steps(n_super, parts)) * STREAM_WAVES;
+        const int covered = stream_steps_served(stream_steps(n_super, parts)) * nw;
         const int needed = (n_super + covered - 1) / covered;
         if (needed == parts) return parts;
         parts = needed;
     }
 }
 
-template <int U, int TREG, typename TC, int EPI>
+template <int NW, int U, int TREG, typename TC, int EPI>
 static void launch_stream(hipStream_t stream, const void* a, const void* w, void* c, int M, int N, int K, int parts,
                           const RowNorm& norm) {
     const int strips = EPI == EPI_SWIGLU ? (N / 2 + 7) / 8 : (N + 15) / 16;
@@ -369,32 +376,39 @@ static void launch_stream(hipStream_t stream, const void* a, const void* w, void
     T = (T + U - 1) / U * U;
     if (TREG > 0) T = TREG;
     // every block the same number of strips, as far as that goes
-    // (with six or eight steps of activations in registers only one block fits a compute unit)
-    const int slots = TREG > 4 ? max(1, 256 / parts) : (parts > 1 ? max(1, STREAM_SLOTS_CUT / parts) : STREAM_SLOTS);
+    // (with six or eight steps of activations in registers half as many waves fit a compute unit)
+    const int wave_slots = TREG > 4 ? STREAM_WAVE_SLOTS / 2 : (parts > 1 ? STREAM_WAVE_SLOTS_CUT : STREAM_WAVE_SLOTS);
+    const int slots = max(1, wave_slots / NW / parts);
     const int rounds = (strips + slots - 1) / slots;
     const dim3 grid((strips + rounds - 1) / rounds, parts);
-    const bool exact = K % SUPER_K == 0 && parts * T * STREAM_WAVES == n_super;
-    if (exact)
-        linear_stream_kernel<U, TREG, true, TC, EPI><<<grid, STREAM_WAVES * WAVE, 0, stream>>>(
+    if (K % SUPER_K == 0 && parts * T * NW == n_super)
+        linear_stream_kernel<NW, U, TREG, true, TC, EPI><<<grid, NW * WAVE, 0, stream>>>(
             (const bf16_t*)a, (const bf16_t*)w, (TC*)c, M, N, K, strips, T, norm);
     else
-        linear_stream_kernel<U, TREG, false, TC, EPI><<<grid, STREAM_WAVES * WAVE, 0, stream>>>(
+        linear_stream_kernel<NW, U, TREG, false, TC, EPI><<<grid, NW * WAVE, 0, stream>>>(
             (const bf16_t*)a, (const bf16_t*)w, (TC*)c, M, N, K, strips, T, norm);
+}
+
+template <int NW, typename TC, int EPI>
+static void dispatch_stream(hipStream_t stream, const void* a, const void* w, void* c, int M, int N, int K, int parts,
+                            const RowNorm& norm, int per_wave) {
+    if (per_wave <= 2) launch_stream<NW, 2, 2, TC, EPI>(stream, a, w, c, M, N, K, parts, norm);
+    else if (per_wave <= 4) launch_stream<NW, 2, 4, TC, EPI>(stream, a, w, c, M, N, K, parts, norm);
+    else if (per_wave <= 6) launch_stream<NW, 2, 6, TC, EPI>(stream, a, w, c, M, N, K, parts, norm);
+    else if (per_wave <= 8) launch_stream<NW, 2, 8, TC, EPI>(stream, a, w, c, M, N, K, parts, norm);
+    else launch_stream<NW, 4, 0, TC, EPI>(stream, a, w, c, M, N, K, parts, norm);
 }
 
 template <typename TC, int EPI>
 static void dispatch_thin(hipStream_t stream, const void* a, const void* w, void* c, int M, int N, int K, int parts,
                           const RowNorm& norm) {
     const int n_super = (K + SUPER_K - 1) / SUPER_K;
-    const bool deep = n_super >= 16;                           // enough super-steps to feed eight waves
+    const bool deep = n_super >= 16;                           // enough super-steps to feed a block's waves
     const bool folded = norm.ss_in || norm.resid;              // only the stream kernel folds a norm in
     if (M <= 16 && (deep || folded)) {
         const int per_wave = stream_steps(n_super, parts);
-        if (per_wave <= 2) launch_stream<2, 2, TC, EPI>(stream, a, w, c, M, N, K, parts, norm);
-        else if (per_wave <= 4) launch_stream<2, 4, TC, EPI>(stream, a, w, c, M, N, K, parts, norm);
-        else if (per_wave <= 6) launch_stream<2, 6, TC, EPI>(stream, a, w, c, M, N, K, parts, norm);
-        else if (per_wave <= 8) launch_stream<2, 8, TC, EPI>(stream, a, w, c, M, N, K, parts, norm);
-        else launch_stream<4, 0, TC, EPI>(stream, a, w, c, M, N, K, parts, norm);
+        if (stream_waves(n_super) == 4) dispatch_stream<4, TC, EPI>(stream, a, w, c, M, N, K, parts, norm, per_wave);
+        else dispatch_stream<8, TC, EPI>(stream, a, w, c, M, N, K, parts, norm, per_wave);
         return;
     }
     // a short K: one strip a block, four waves (two strips a block, RT = 2, were measured slower at every size)

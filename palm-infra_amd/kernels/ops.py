@@ -318,7 +318,24 @@ def linear_library(a: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
 
 
 THIN_TOKENS = 16      # up to here every wave fetches its own activations; above, a block shares them through LDS
-FOLD_MAX_K = 12288    # up to this K a product of 9 to 16 rows folds a norm in; the thin kernel holds activations in registers up to 8192
+
+
+COMPUTE_UNITS = 256     # of an MI355X; a folded product's blocks come in rounds of this many
+
+
+def fold_pays(M: int, N: int, K: int) -> bool:
+    """Whether a product of M <= 16 rows that is a branch's output should fold the residual add and the next norm
+    in, or rather be cut along K into planes that the norm's own kernel adds up.  A fold needs all of K in one
+    block.  Up to K = 8192 the block keeps the activations in registers and the fold won at every width measured
+    (N 1024 to 5120: 8 to 28 us against 8 to 36).  Beyond that it reads them beside the weights and wins only
+    where whole rounds of blocks fill the compute units: N 4096 at K 12288 and 14336 (25 to 42 us against 32 to
+    41), not N 2560 or 5120 (a quarter of a second round: 55 to 125 us against 40 to 66), and nowhere measured
+    beyond K 14336."""
+    if K <= 8192:
+        return True
+    strips = (N + 15) // 16
+    rounds = (strips + COMPUTE_UNITS - 1) // COMPUTE_UNITS
+    return K <= 14336 and strips >= 0.75 * rounds * COMPUTE_UNITS
 
 
 def thin_serves(a: torch.Tensor, w: torch.Tensor) -> bool:

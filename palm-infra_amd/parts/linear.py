@@ -54,11 +54,8 @@ class Linear:
 
     def _into(self, x, sink):
         rows = x.values if isinstance(x, Prenormed) else x
-        # (a fold needs the whole of K in one block; beyond what a wave's registers hold of the activations that
-        # costs more than it saves once there are more than eight rows: at 16 rows K = 12288 is still 5% faster
-        # folded, K = 17408 20% slower than cut into ranges whose planes the norm adds up)
         if (sink.foldable and self._folds(rows) and sink.x.shape == (rows.shape[0], self.out_features)
-                and rows.dtype == torch.bfloat16 and (self.in_features <= ops.FOLD_MAX_K or rows.shape[0] <= 8)):
+                and rows.dtype == torch.bfloat16 and ops.fold_pays(rows.shape[0], self.out_features, self.in_features)):
             ss_in, eps_in = (x.ss, x.eps) if isinstance(x, Prenormed) else (None, 0.0)
             values, ss = ops.linear_thin_into_residual(rows, self.weight, sink.x, sink.norm.weight, row_ss=ss_in, row_eps=eps_in)
             return Prenormed(values, ss, sink.norm.eps)
