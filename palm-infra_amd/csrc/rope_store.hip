@@ -17,7 +17,10 @@
 #include <type_traits>
 
 constexpr int MAX_HEAD_DIM = 512;
-constexpr int FAST_MIN_TOKENS = 32;       // from here on the kernels for many tokens run (where they serve the head size)
+// From here on the kernels for many tokens run, where they serve the head size and q/k/v come whole, not as
+// planes.  Measured at 32 heads of 128 over 8 kv heads: 256 tokens 8.6 to 10 us with one wave a head against 10 to
+// 17 us, 512 tokens 14.5 to 18 against 11 to 18 (the slower figures: every token in a sequence of its own).
+constexpr int FAST_MIN_TOKENS = 384;
 
 // One wave per (token, head).  pairing 0: pairs (i, i + rot/2); pairing 1: pairs (2i, 2i + 1).
 // qkv may come as `planes` planes of partial sums (a projection that cut its K into ranges), plane_stride
@@ -171,7 +174,7 @@ constexpr int FAST_HEADS_AT_ONCE = 4;
 
 template <typename TIN, typename T, int E>
 __global__ __launch_bounds__(4 * WAVE) void qk_norm_rope_fast_kernel(
-    const TIN* __restrict__ qkv, int planes, size_t plane_stride, T* __restrict__ q_out, T* __restrict__ k_cache,
+    const TIN* __restrict__ qkv, T* __restrict__ q_out, T* __restrict__ k_cache,
     const int* __restrict__ block_table, int max_pages, const int* __restrict__ tok_slot,
     const int* __restrict__ positions, const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w,
     float eps, const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rotary_dim, int pairing,
@@ -219,14 +222,6 @@ __global__ __launch_bounds__(4 * WAVE) void qk_norm_rope_fast_kernel(
             head[u] = base + (u * 4 + wave) * per_wave + sub;
             read_elems<E>(token + (size_t)min(head[u], n_heads - 1) * hd, x[u]);
         }
-        for (int p = 1; p < planes; ++p)
-#pragma unroll
-            for (int u = 0; u < U; ++u) {
-                float more[E];
-                read_elems<E>(token + p * plane_stride + (size_t)min(head[u], n_heads - 1) * hd, more);
-#pragma unroll
-                for (int e = 0; e < E; ++e) x[u][e] += more[e];
-            }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             if (base + (u * 4 + wave) * per_wave >= n_heads) continue;       // none of the wave's heads of this turn exists
@@ -273,7 +268,7 @@ __global__ __launch_bounds__(4 * WAVE) void qk_norm_rope_fast_kernel(
 // v of 64 consecutive tokens of one kv head into the transposed pages
 template <typename TIN, typename T>
 __global__ __launch_bounds__(4 * WAVE) void v_store_tile_kernel(
-    const TIN* __restrict__ qkv, int planes, size_t plane_stride, T* __restrict__ v_cache,
+    const TIN* __restrict__ qkv, T* __restrict__ v_cache,
     const int* __restrict__ block_table, int max_pages, const int* __restrict__ tok_slot,
     const int* __restrict__ positions, int n_tokens, int nh, int nkv, int hd) {
     __shared__ float tile[PAGE_TOKENS][33];                  // 32 elements of 64 tokens at a time
@@ -285,7 +280,7 @@ __global__ __launch_bounds__(4 * WAVE) void v_store_tile_kernel(
     const int page = block_table[(size_t)tok_slot[t_mine] * max_pages + pos / PAGE_TOKENS];
     T* dst = v_cache + ((size_t)page * nkv + g) * hd * PAGE_TOKENS + pos % PAGE_TOKENS;
     if constexpr (std::is_same<TIN, bf16_t>::value && std::is_same<T, bf16_t>::value) {
-        if (planes == 1 && hd % 8 == 0) {
+        if (hd % 8 == 0) {
             // bfloat16 straight through: 128 elements of the 64 tokens at a time, read 16 bytes a thread, kept in LDS
             // as pairs (rows of 65 words: a lane a token then reads without a bank conflict), written two rows a read
             __shared__ uint32_t pairs[PAGE_TOKENS][65];
@@ -329,7 +324,6 @@ __global__ __launch_bounds__(4 * WAVE) void v_store_tile_kernel(
             if (t0 + tt < n_tokens && d < hd) {
                 const TIN* src = qkv + ((size_t)(t0 + tt) * (nh + 2 * nkv) + nh + nkv + g) * hd + d;
                 v = to_float(*src);
-                for (int p = 1; p < planes; ++p) v += to_float(src[p * plane_stride]);
             }
             tile[tt][i % 32] = v;
         }
@@ -363,14 +357,14 @@ PALM_API int palm_qk_norm_rope_store(hipStream_t stream, const void* qkv, int dt
     dim3 grid(n_tokens, nh + 2 * nkv);
     PALM_CHECK(grid.y <= 65535, "qk_norm_rope_store: %d heads are more than one launch takes", (int)grid.y);
     const size_t plane_stride = (size_t)n_tokens * (nh + 2 * nkv) * hd;
-    if (n_tokens >= FAST_MIN_TOKENS && rope_fast_serves(hd, rotary_dim, pairing, cos_t != nullptr)) {
+    if (planes == 1 && n_tokens >= FAST_MIN_TOKENS && rope_fast_serves(hd, rotary_dim, pairing, cos_t != nullptr)) {
         const int L = fast_lanes(hd);
         const dim3 qk_grid(n_tokens);
         const dim3 v_grid((n_tokens + PAGE_TOKENS - 1) / PAGE_TOKENS, nkv);
         PALM_CHECK(v_grid.y <= 65535, "qk_norm_rope_store: %d kv heads are more than one launch takes", nkv);
 #define PALM_ROPE_FAST_E(TIN, T, EE) case EE: \
         qk_norm_rope_fast_kernel<TIN, T, EE><<<qk_grid, 4 * WAVE, 0, stream>>>( \
-            (const TIN*)qkv, planes, plane_stride, (T*)q_out, (T*)k_cache, block_table, max_pages, tok_slot, positions, \
+            (const TIN*)qkv, (T*)q_out, (T*)k_cache, block_table, max_pages, tok_slot, positions, \
             q_norm_w, k_norm_w, eps, cos_t, sin_t, rotary_dim, pairing, nh, nkv, hd, L, write_cache); break;
 #define PALM_ROPE_FAST(TIN, T) do { \
         switch (hd / L) { \
@@ -378,10 +372,9 @@ PALM_API int palm_qk_norm_rope_store(hipStream_t stream, const void* qkv, int dt
             PALM_ROPE_FAST_E(TIN, T, 5) PALM_ROPE_FAST_E(TIN, T, 6) PALM_ROPE_FAST_E(TIN, T, 7) PALM_ROPE_FAST_E(TIN, T, 8) \
         } \
         if (write_cache) v_store_tile_kernel<TIN, T><<<v_grid, 4 * WAVE, 0, stream>>>( \
-            (const TIN*)qkv, planes, plane_stride, (T*)v_cache, block_table, max_pages, tok_slot, positions, n_tokens, nh, nkv, hd); \
+            (const TIN*)qkv, (T*)v_cache, block_table, max_pages, tok_slot, positions, n_tokens, nh, nkv, hd); \
     } while (0)
-        if (planes > 1) { PALM_DTYPE_SWITCH(dtype, T, PALM_ROPE_FAST(float, T)); }
-        else { PALM_DTYPE_SWITCH(dtype, T, PALM_ROPE_FAST(T, T)); }
+        PALM_DTYPE_SWITCH(dtype, T, PALM_ROPE_FAST(T, T));
 #undef PALM_ROPE_FAST_E
 #undef PALM_ROPE_FAST
         PALM_LAUNCHED();

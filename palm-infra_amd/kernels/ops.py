@@ -35,8 +35,9 @@ _SIGNATURES = {
                          c_void_p, c_int, c_float, c_void_p, c_void_p, c_void_p],
     "palm_scale_rows": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_float, c_int, c_void_p],
     "palm_linear_thin_parts": [c_int, c_int, c_int],
-    "palm_linear_wide": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
-    "palm_linear_wide_splits": [c_int, c_int, c_int, c_int],
+    "palm_linear_wide": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int],
+    "palm_linear_wide_parts": [c_int, c_int, c_int, c_int],
+    "palm_linear_wide_blocks": [c_int, c_int, c_int, c_int, c_int],
     "palm_argmax": [c_void_p, c_void_p, c_int, c_int, c_void_p],
     "palm_apply_penalties": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_float, c_float, c_float],
     "palm_sample": [c_void_p, c_void_p, c_int, c_int, c_void_p, c_float, c_int, c_float, c_float, c_void_p, c_void_p],
@@ -52,7 +53,7 @@ def core():
         lib = library.load("core")
         for name, argtypes in _SIGNATURES.items():
             fn = getattr(lib, name)
-            fn.argtypes, fn.restype = argtypes, c_int      # (palm_linear_wide_splits returns a count, not a status)
+            fn.argtypes, fn.restype = argtypes, c_int      # (the *_parts and *_blocks functions return a count, not a status)
         if lib.palm_page_tokens() != PAGE_TOKENS:
             raise KernelError(f"the kernels were built for pages of {lib.palm_page_tokens()} tokens, "
                               f"the cache uses {PAGE_TOKENS}")
@@ -318,6 +319,7 @@ def linear_library(a: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
 
 
 THIN_TOKENS = 16      # up to here every wave fetches its own activations; above, a block shares them through LDS
+WIDE_TOKENS = 64      # as many rows as that block holds
 
 
 COMPUTE_UNITS = 256     # of an MI355X; a folded product's blocks come in rounds of this many
@@ -336,6 +338,18 @@ def fold_pays(M: int, N: int, K: int) -> bool:
     strips = (N + 15) // 16
     rounds = (strips + COMPUTE_UNITS - 1) // COMPUTE_UNITS
     return K <= 14336 and strips >= 0.75 * rounds * COMPUTE_UNITS
+
+
+WIDE_MIN_BLOCKS = 128   # of 256 compute units
+
+
+def wide_pays(M: int, N: int, K: int, gated: bool = False, planes_ok: bool = False) -> bool:
+    """Whether the kernel for 17 to 64 rows has enough blocks for this product to beat the library: with few
+    weight rows it does only if the reader takes planes of partial sums.  Measured at Qwen3-8B's shapes with 64
+    rows (us, own against library): q/k/v 18 and 18, output projection 14 and 16, down 27 and 37 as planes (76
+    whole), gate/up 45 gated against 46 with the activation's own pass; with 32 rows 14/17, 11/13, 23/26, 40/47."""
+    return THIN_TOKENS < M <= WIDE_TOKENS and core().palm_linear_wide_blocks(
+        M, N, K, 1 if gated else 0, 1 if planes_ok else 0) >= WIDE_MIN_BLOCKS
 
 
 def thin_serves(a: torch.Tensor, w: torch.Tensor) -> bool:
@@ -415,11 +429,16 @@ def linear_thin(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, gated:
         library.call(core(), "palm_linear_thin", _stream(), _p(a), _p(w), _p(out), _code(out, "linear_thin out"), M, N, K,
                      1 if gated else 0, planes, _p(row_ss), pieces, float(row_eps), None, None, None)
         return out
-    # more rows than one block of 16: the kernel that shares the activations through LDS, K split if need be
-    splits = core().palm_linear_wide_splits(M, N, K, 1 if gated else 0)
-    work = torch.empty((splits * M * N,), dtype=F32, device=a.device) if splits > 1 else None
+    if M > WIDE_TOKENS:
+        # the weight goes by once for every 64 rows (a float32 result for many rows: logits at many places)
+        return torch.cat([linear_thin(a[r0:r0 + WIDE_TOKENS], w, out_dtype, gated=gated)
+                          for r0 in range(0, M, WIDE_TOKENS)])
+    # more rows than one block of 16: the kernel that shares the activations through LDS
+    planes = core().palm_linear_wide_parts(M, N, K, 0) if planes_ok and not gated else 1
+    if planes > 1:
+        out = torch.empty((planes, M, N), dtype=F32, device=a.device)
     library.call(core(), "palm_linear_wide", _stream(), _p(a), _p(w), _p(out), _code(out, "linear_wide out"), M, N, K,
-                 1 if gated else 0, splits, _p(work))
+                 1 if gated else 0, planes)
     return out
 
 

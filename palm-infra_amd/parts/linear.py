@@ -1,7 +1,8 @@
 """y = x W^T for a weight in the checkpoint's [out, in] layout: the one place that picks the kernel.
 
   float32 run, or a 32-bit weight under bfloat16 activations   the exact FMA kernel
-  bfloat16 x bfloat16, few rows (decode)                        the matrix-core kernel for thin products
+  bfloat16 x bfloat16, up to 16 rows (decode)                   the matrix-core kernel for thin products
+  bfloat16 x bfloat16, 17 to 64 rows (large decode batches)     the matrix-core kernel that shares the rows through LDS
   bfloat16 x bfloat16, many rows (prompts)                      the BLAS library, as the reference's GPU path
                                                                 does for its products (engine/cuda_matmul.cu:245-260)
 """
@@ -12,9 +13,9 @@ import torch
 from ..kernels import ops
 from .residual import Prenormed
 
-# Up to this many rows the kernel that streams the weight past one block of 16 rows is the fastest; above, the
-# library is (measured at Qwen3-8B's four shapes with 17, 32 and 64 rows: 15 to 49 us against 18 to 66 us of
-# the kernel that shares 64 rows through LDS, which still serves products with a float32 result).
+# Up to this many rows the kernel that streams the weight past one block of 16 rows serves; from there to 64 rows
+# the kernel that shares the rows through LDS, where it has blocks enough to fill the chip (ops.wide_pays), and
+# for every product with a float32 result; else the library.
 THIN_ROWS = 16
 
 
@@ -43,7 +44,8 @@ class Linear:
             x = x.materialize()
         out_dtype = out_dtype or x.dtype
         if x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16:
-            if x.shape[0] <= THIN_ROWS or out_dtype != torch.bfloat16:
+            if (x.shape[0] <= THIN_ROWS or out_dtype != torch.bfloat16
+                    or (ops.thin_serves(x, w) and ops.wide_pays(x.shape[0], self.out_features, self.in_features, planes_ok=planes_ok))):
                 return ops.linear_thin(x, w, out_dtype, planes_ok=planes_ok)
             return ops.linear_library(x, w)
         return ops.linear_exact(x, w, out_dtype)
@@ -68,6 +70,7 @@ class Linear:
             if self._folds(x.values):
                 return ops.linear_thin(x.values, self.weight, x.dtype, gated=True, row_ss=x.ss, row_eps=x.eps)
             x = x.materialize()
-        if x.shape[0] <= THIN_ROWS and ops.thin_serves(x, self.weight):
+        if ops.thin_serves(x, self.weight) and (
+                x.shape[0] <= THIN_ROWS or ops.wide_pays(x.shape[0], self.out_features, self.in_features, gated=True)):
             return ops.linear_thin(x, self.weight, x.dtype, gated=True)
         return ops.swiglu(self(x))

@@ -225,17 +225,17 @@ def test_qk_norm_rope_store(ops, dtype, nh, nkv, hd):
 def test_qk_norm_rope_store_of_many_tokens(ops, dtype, nh, nkv, hd):
     """Prompts go through kernels of their own (heads held in registers, v written tile by tile): three
     sequences that start inside pages, cross page borders, and fill no tile of 64 tokens."""
-    starts, counts, slots = [60, 0, 130], [70, 41, 3], [2, 0, 3]
+    starts, counts, slots = [60, 0, 130], [250, 141, 3], [2, 0, 3]
     n = sum(counts)
     pos = [s + j for s, c in zip(starts, counts) for j in range(c)]
     tslot = [sl for sl, c in zip(slots, counts) for _ in range(c)]
     qkv = rand(n, (nh + 2 * nkv) * hd, seed=hd, dtype=dtype)
     qw, kw = rand(hd, seed=1) + 1.0, rand(hd, seed=2) + 1.0
     eps, theta = 1e-5, 10000.0
-    table = torch.full((4, 3), 9, dtype=torch.int32)
-    table[2] = torch.tensor([5, 1, 7])
-    table[0, :1] = torch.tensor([3])
-    table[3] = torch.tensor([9, 9, 0])
+    table = torch.full((4, 5), 9, dtype=torch.int32)
+    table[2] = torch.tensor([5, 1, 7, 2, 4])
+    table[0, :3] = torch.tensor([3, 6, 8])
+    table[3, 2] = 0
     kc, vc = _paged(10, nkv, hd, dtype)
     inv = torch.from_numpy((1.0 / np.power(np.float32(theta), 2.0 * np.arange(hd // 2, dtype=np.float32) / hd)).astype(np.float32))
     pos_d = torch.tensor(pos, dtype=torch.int32).to(DEV)
@@ -271,11 +271,11 @@ def test_qk_norm_rope_store_of_many_tokens(ops, dtype, nh, nkv, hd):
     assert torch.allclose(kc2.cpu().double(), kc, atol=1e-5 if dtype == F32 else 4e-2) and torch.equal(vc2.cpu().double(), vc)
 
 
-def test_qk_norm_rope_store_of_many_tokens_in_planes_and_other_rotations(ops):
-    nh, nkv, hd, n = 6, 2, 64, 100
+def test_qk_norm_rope_store_of_many_tokens_whole_or_in_planes_and_other_rotations(ops):
+    nh, nkv, hd, n = 6, 2, 64, 430           # enough tokens for the kernels that take many
     i32 = lambda xs: torch.tensor(xs, dtype=torch.int32).to(DEV)
     pos, slot = i32(list(range(30, 30 + n))), i32([1] * n)
-    table = i32([[9, 9, 9], [4, 2, 6]])
+    table = i32([[9] * 8, [4, 2, 6, 1, 8, 3, 7, 5]])
     qw, kw = (rand(hd, seed=1) + 1.0).to(DEV), (rand(hd, seed=2) + 1.0).to(DEV)
     planes = rand(3, n, (nh + 2 * nkv) * hd, seed=11)
     whole = ((planes[0] + planes[1]) + planes[2]).to(BF16)
@@ -288,19 +288,23 @@ def test_qk_norm_rope_store_of_many_tokens_in_planes_and_other_rotations(ops):
         kw_args = dict(q_norm_w=qw if norms else None, k_norm_w=kw if norms else None, eps=1e-6, cos=cos, sin=sin, rotary_dim=rot,
                        pairing=pairing, block_table=table, tok_slot=slot, write_cache=writes)
         results = []
-        # all at once from planes (the kernels for many tokens where they serve), and eleven at a time from one tensor
+        # all at once (the kernels for many tokens where they serve), all at once from planes, and 47 at a time
         kc, vc = _paged(10, nkv, hd, BF16)
-        q = ops.qk_norm_rope_store(planes.to(DEV), nh, nkv, hd, pos, k_cache=kc, v_cache=vc, out_dtype=BF16, **kw_args)
+        q = ops.qk_norm_rope_store(whole.to(DEV), nh, nkv, hd, pos, k_cache=kc, v_cache=vc, **kw_args)
+        kc3, vc3 = _paged(10, nkv, hd, BF16)
+        q3 = ops.qk_norm_rope_store(planes.to(DEV), nh, nkv, hd, pos, k_cache=kc3, v_cache=vc3, out_dtype=BF16, **kw_args)
         kc2, vc2 = _paged(10, nkv, hd, BF16)
         qs = []
-        for a in range(0, n, 11):
-            sl = slice(a, a + 11)
+        for a in range(0, n, 47):
+            sl = slice(a, a + 47)
             args = dict(kw_args, cos=None if cos is None else cos[sl].contiguous(), sin=None if sin is None else sin[sl].contiguous(),
                         tok_slot=slot[sl].contiguous())
             qs.append(ops.qk_norm_rope_store(whole[sl].contiguous().to(DEV), nh, nkv, hd, pos[sl].contiguous(), k_cache=kc2, v_cache=vc2, **args))
         case = (pairing, rot, norms, writes)
         assert torch.allclose(q.float(), torch.cat(qs).float(), atol=6e-2, rtol=2e-2), case
         assert torch.allclose(kc.float(), kc2.float(), atol=6e-2, rtol=2e-2) and torch.allclose(vc.float(), vc2.float(), atol=2e-2, rtol=1e-2), case
+        assert torch.allclose(q3.float(), torch.cat(qs).float(), atol=6e-2, rtol=2e-2), case
+        assert torch.allclose(kc3.float(), kc2.float(), atol=6e-2, rtol=2e-2) and torch.allclose(vc3.float(), vc2.float(), atol=2e-2, rtol=1e-2), case
         assert (float(kc.abs().max()) > 0.5) == writes, case
 
 
