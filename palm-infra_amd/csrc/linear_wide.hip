@@ -236,7 +236,7 @@ static WidePlan wide_plan(int N, int K, int epilogue, int max_parts) {
     for (int parts = 1; parts <= max_parts; ++parts) {
         const int per = (n_chunks + parts - 1) / parts;
         if (parts > 1 && (per < WIDE_MIN_CHUNKS || (parts - 1) * per >= n_chunks)) continue;   // short, or an empty range
-        for (int waves = 4; waves <= 8; waves += 2) {
+        for (int waves = 8; waves >= 4; waves -= 2) {       // of equals the larger block: it shares the rows among more strips
             const long blocks = (long)((strips + waves - 1) / waves) * parts;
             const long cost = ((blocks + WIDE_UNITS - 1) / WIDE_UNITS) * (per + 2) * waves;
             if (best_cost < 0 || cost < best_cost) { best_cost = cost; best = WidePlan{waves, parts, per}; }
