@@ -120,123 +120,188 @@ PALM_API int palm_apply_penalties(hipStream_t stream, float* logits, int V, cons
 }
 
 // ---- sampling -------------------------------------------------------------------------------------
-// Thread t owns the contiguous chunk [t * chunk, (t + 1) * chunk) of the row, so that sums and ranks
-// "in index order" are a scan over threads.  All sums are added in a fixed order: the result for a row
-// is the same whatever else is in the batch.
+// One block of 16 waves for each row.  Wave w owns the contiguous range [w * per, (w + 1) * per) of the row and
+// walks it 64 elements at a time, a lane an element: reads are contiguous, and "index order" is the order
+// (wave, step, lane).  A weight is w = exp((l - l_max) / T), at most 1; sums of weights are 64-bit sums of the
+// integers floor(w * 2^31).  Integer sums do not depend on the order of their terms: a row's result is the same
+// bits whatever else is in the batch, however the atomic additions below fall, and a part's sum is exactly the
+// sum of its parts' (so a search that goes from waves to threads to elements never misses its target).
+
+constexpr int SAMPLE_WAVES = SAMPLE_THREADS / WAVE;
+constexpr float FIXED_ONE = 2147483648.0f;           // 2^31: a weight fits 32 bits, a row's sum 64
+constexpr int HIST_STRIDE = 257;                     // a wave's histogram starts one bank on from its neighbour's
+typedef unsigned long long mass_t;
 
 struct SampleShared {
-    BestPair best[SAMPLE_THREADS / WAVE];
-    float part[SAMPLE_THREADS];      // per-thread partial sums
-    int cnt[SAMPLE_THREADS];         // per-thread counts
-    unsigned int hist[256];
+    BestPair best[SAMPLE_WAVES];
+    union {
+        mass_t mass[SAMPLE_WAVES][HIST_STRIDE];          // a histogram for each wave: weights by a byte of the key
+        unsigned int count[SAMPLE_WAVES][HIST_STRIDE];   //                            elements by a byte of the key
+    } hist;
+    mass_t bin_mass[256];
+    mass_t wave_mass[SAMPLE_WAVES];              // weights above the threshold, by wave; then by wave of threads
+    int wave_ties[SAMPLE_WAVES];                 // elements at the threshold
     float cand_v[TOPK_MAX];
     int cand_i[TOPK_MAX];
     float cand_w[TOPK_MAX];
     int n_cand;
     // results of the serial parts, broadcast
-    uint32_t prefix; int remaining; int owner; float base; int n_ties; float total;
+    uint32_t prefix; int remaining; int owner; int owner_ties; mass_t base; mass_t above; float total; int result;
 };
 
-// fixed-order sum of part[0..n): a tree over the block
-__device__ float block_tree_sum(float* part, int n) {
-    __syncthreads();
-    for (int stride = SAMPLE_THREADS / 2; stride > 0; stride >>= 1) {
-        if ((int)threadIdx.x < stride && (int)threadIdx.x + stride < n) part[threadIdx.x] += part[threadIdx.x + stride];
-        __syncthreads();
+__device__ inline uint32_t fixed_weight(float l, float l_max, float inv_t, float min_w) {
+    const float w = __expf((l - l_max) * inv_t);
+    return w >= min_w ? (uint32_t)(w * FIXED_ONE) : 0u;       // (a NaN fails the comparison)
+}
+__device__ inline float key_value(uint32_t key) {             // the float whose ordered_key is key
+    return __uint_as_float((key & 0x80000000u) ? (key & 0x7fffffffu) : ~key);
+}
+__device__ inline mass_t wave_sum(mass_t v) {
+#pragma unroll
+    for (int off = WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, WAVE);
+    return v;
+}
+__device__ inline int wave_sum(int v) {
+#pragma unroll
+    for (int off = WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, WAVE);
+    return v;
+}
+// how many lanes below this one have the flag set
+__device__ inline int lanes_before(bool flag) {
+    const unsigned long long m = __ballot(flag);
+    return __popcll(m & ((1ull << (threadIdx.x % WAVE)) - 1ull));
+}
+
+// The wave's range of the row, and f(i, l) for its elements in index order (every lane takes part in every
+// step; a lane beyond the range gets i = -1 and l = -inf).
+struct Range { int begin, end; };
+__device__ inline Range wave_range(int V) {
+    const int per = ((V + SAMPLE_WAVES - 1) / SAMPLE_WAVES + WAVE - 1) / WAVE * WAVE;
+    const int begin = min(V, (int)(threadIdx.x / WAVE) * per);
+    return Range{begin, min(V, begin + per)};
+}
+constexpr int RANGE_AHEAD = 16;          // steps whose reads are on their way together: the row comes from L2, a read takes long
+template <typename F>
+__device__ inline void for_range(const float* __restrict__ row, Range rg, F&& f) {
+    const int lane = threadIdx.x % WAVE;
+    for (int base = rg.begin; base < rg.end; base += RANGE_AHEAD * WAVE) {
+        float l[RANGE_AHEAD];
+#pragma unroll
+        for (int u = 0; u < RANGE_AHEAD; ++u) {
+            const int i = base + u * WAVE + lane;
+            l[u] = i < rg.end ? row[i] : -INFINITY;
+        }
+#pragma unroll
+        for (int u = 0; u < RANGE_AHEAD; ++u) {
+            const int i = base + u * WAVE + lane;
+            if (base + u * WAVE < rg.end) f(i < rg.end ? i : -1, l[u]);
+        }
     }
-    const float r = part[0];
-    __syncthreads();
-    return r;
 }
 
-// The weight of element i of the row if it is kept, else 0.  kept: key > tau, or key == tau and the
-// element is among the first n_ties elements equal to tau (rank counted in index order).
-__device__ inline float kept_weight(float l, float l_max, float inv_t, float min_w) {
-    const float w = expf((l - l_max) * inv_t);
-    return w >= min_w ? w : 0.f;
+// wave_mass[w] = the weights of wave w's elements with key > tau (all of them if `all`), wave_ties[w] = how many
+// of its elements have key == tau; then a barrier
+template <bool WEIGHTS = true>     // false: wave_mass[w] counts the elements instead of weighing them
+__device__ void masses_by_wave(const float* __restrict__ row, int V, float l_max, float inv_t, float min_w, uint32_t tau,
+                               bool all, SampleShared& sh) {
+    mass_t mine = 0ull;
+    int ties = 0;
+    for_range(row, wave_range(V), [&](int i, float l) {
+        const uint32_t key = ordered_key(l);
+        if (i >= 0 && (all || key > tau)) mine += WEIGHTS ? fixed_weight(l, l_max, inv_t, min_w) : 1u;
+        ties += i >= 0 && !all && key == tau;
+    });
+    mine = wave_sum(mine);
+    ties = wave_sum(ties);
+    if (threadIdx.x % WAVE == 0) { sh.wave_mass[threadIdx.x / WAVE] = mine; sh.wave_ties[threadIdx.x / WAVE] = ties; }
+    __syncthreads();
 }
 
-// Draw in index order over the kept set: the first kept element whose cumulative weight reaches target.
-// `tau`/`n_ties` describe the kept set (tau == 0 keeps every key, since ordered keys of finite floats
-// are > 0 ... see ordered_key: only NaN patterns could be smaller, and they carry no weight).
-__device__ int draw_index_order(const float* __restrict__ row, int V, int chunk, float l_max, float inv_t,
-                                float min_w, uint32_t tau, int n_ties, float target, SampleShared& sh,
-                                float* __restrict__ probs_out, float total) {
-    const int begin = threadIdx.x * chunk, end = min(V, begin + chunk);
-    // ranks of ties: how many elements equal to tau lie before this thread's chunk
-    int my_ties = 0;
-    for (int i = begin; i < end; ++i) my_ties += ordered_key(row[i]) == tau;
-    sh.cnt[threadIdx.x] = my_ties;
-    __syncthreads();
+// The element in which the weights of the kept set, added up in index order, pass `target` (< their sum).
+// The kept set: key > tau, and the first n_ties elements with key == tau (`all`: every element).  Needs
+// masses_by_wave(tau).  Three levels: the wave's range, a thread's piece of that range, the element.
+__device__ int draw_index_order(const float* __restrict__ row, int V, float l_max, float inv_t, float min_w, uint32_t tau,
+                                bool all, int n_ties, mass_t w_tau, mass_t target, SampleShared& sh) {
     if (threadIdx.x == 0) {
-        int run = 0;
-        for (int t = 0; t < SAMPLE_THREADS; ++t) { const int c = sh.cnt[t]; sh.cnt[t] = run; run += c; }
+        mass_t run = 0ull;
+        int ties_before = 0, owner = SAMPLE_WAVES - 1, owner_ties = 0;
+        mass_t base = 0ull;
+        bool found = false;
+        for (int w = 0; w < SAMPLE_WAVES; ++w) {
+            const int kept_ties = all ? 0 : max(0, min(sh.wave_ties[w], n_ties - ties_before));
+            const mass_t kept = sh.wave_mass[w] + (mass_t)kept_ties * w_tau;
+            if (!found && target < run + kept) { found = true; owner = w; base = run; owner_ties = ties_before; }
+            run += kept;
+            ties_before += sh.wave_ties[w];
+        }
+        sh.owner = owner; sh.base = base; sh.owner_ties = owner_ties;
     }
     __syncthreads();
-    int tie_rank = sh.cnt[threadIdx.x];
-    float mine = 0.f;
+    // the owner's range, a piece a thread
+    const int per = ((V + SAMPLE_WAVES - 1) / SAMPLE_WAVES + WAVE - 1) / WAVE * WAVE;
+    const int r_begin = min(V, sh.owner * per), r_end = min(V, r_begin + per);
+    const int piece = (r_end - r_begin + SAMPLE_THREADS - 1) / SAMPLE_THREADS;
+    const int begin = min(r_end, r_begin + (int)threadIdx.x * piece), end = min(r_end, begin + piece);
+    const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
+    mass_t above = 0ull;
+    int ties = 0;
     for (int i = begin; i < end; ++i) {
         const float l = row[i];
         const uint32_t key = ordered_key(l);
-        bool keep = key > tau;
-        if (key == tau) { keep = tie_rank < n_ties; ++tie_rank; }
-        const float w = keep ? kept_weight(l, l_max, inv_t, min_w) : 0.f;
-        mine += w;
-        if (probs_out) probs_out[i] = w / total;
+        if (all || key > tau) above += fixed_weight(l, l_max, inv_t, min_w);
+        ties += !all && key == tau;
     }
-    sh.part[threadIdx.x] = mine;
+    // ties before this thread's piece: a scan over the lanes, then over the waves
+    int tie_scan = ties;
+#pragma unroll
+    for (int off = 1; off < WAVE; off <<= 1) { const int o = __shfl_up(tie_scan, off, WAVE); if (lane >= off) tie_scan += o; }
+    if (lane == WAVE - 1) sh.wave_ties[wave] = tie_scan;
     __syncthreads();
-    if (threadIdx.x == 0) {
-        float run = 0.f;
-        int owner = -1, last_nonzero = -1;
-        float base = 0.f;
-        for (int t = 0; t < SAMPLE_THREADS; ++t) {
-            const float p = sh.part[t];
-            if (p > 0.f) last_nonzero = t;
-            if (owner < 0 && p > 0.f && target <= run + p) { owner = t; base = run; }
-            run += p;
-        }
-        // rounding can leave the target a hair above the total: then the last kept element is taken
-        sh.n_ties = owner < 0;
-        if (owner < 0) owner = last_nonzero;
-        sh.owner = owner; sh.base = base;
-    }
+    int ties_before = sh.owner_ties + tie_scan - ties;
+    for (int w = 0; w < wave; ++w) ties_before += sh.wave_ties[w];
+    const int kept_ties = all ? 0 : max(0, min(ties, n_ties - ties_before));
+    const mass_t kept = above + (mass_t)kept_ties * w_tau;
+    mass_t scan = kept;
+#pragma unroll
+    for (int off = 1; off < WAVE; off <<= 1) { const mass_t o = __shfl_up(scan, off, WAVE); if (lane >= off) scan += o; }
+    if (lane == WAVE - 1) sh.wave_mass[wave] = scan;
+    if (threadIdx.x == 0) sh.result = -1;
     __syncthreads();
-    int result = -1;
-    if ((int)threadIdx.x == sh.owner) {
-        float run = sh.base;
-        int rank = sh.cnt[threadIdx.x], last_kept = -1;
+    mass_t before = sh.base + scan - kept;
+    for (int w = 0; w < wave; ++w) before += sh.wave_mass[w];
+    if (target >= before && target < before + kept) {          // one thread at most: the pieces' sums tile the range's
+        mass_t run = before;
+        int rank = ties_before;
         for (int i = begin; i < end; ++i) {
             const float l = row[i];
             const uint32_t key = ordered_key(l);
-            bool keep = key > tau;
-            if (key == tau) { keep = rank < n_ties; ++rank; }
-            const float w = keep ? kept_weight(l, l_max, inv_t, min_w) : 0.f;
-            if (w > 0.f) {
-                last_kept = i;
-                run += w;
-                if (!sh.n_ties && target <= run) { result = i; break; }
+            bool keep = all || key > tau;
+            if (!all && key == tau) { keep = rank < n_ties; ++rank; }
+            if (keep) {
+                run += fixed_weight(l, l_max, inv_t, min_w);
+                if (target < run) { sh.result = i; break; }
             }
         }
-        if (result < 0) result = last_kept;
-        sh.remaining = result;
     }
     __syncthreads();
-    return sh.remaining;
+    return sh.result;
 }
 
-// mass and count of the elements with key >= tau (fixed-order sums)
-__device__ float mass_at_least(const float* __restrict__ row, int V, int chunk, float l_max, float inv_t,
-                               float min_w, uint32_t tau, bool strict, SampleShared& sh) {
-    const int begin = threadIdx.x * chunk, end = min(V, begin + chunk);
-    float mine = 0.f;
-    for (int i = begin; i < end; ++i) {
-        const float l = row[i];
+// probs_out[i] = the element's share of the kept set's weight (needs masses_by_wave(tau) for the ties' ranks)
+__device__ void write_probabilities(const float* __restrict__ row, int V, float l_max, float inv_t, float min_w, uint32_t tau,
+                                    bool all, int n_ties, mass_t total, const SampleShared& sh, float* __restrict__ probs_out) {
+    int rank = 0;
+    for (int w = 0; w < (int)(threadIdx.x / WAVE); ++w) rank += sh.wave_ties[w];
+    const float inv_total = 1.0f / (float)total;
+    for_range(row, wave_range(V), [&](int i, float l) {
         const uint32_t key = ordered_key(l);
-        if (strict ? key > tau : key >= tau) mine += kept_weight(l, l_max, inv_t, min_w);
-    }
-    sh.part[threadIdx.x] = mine;
-    return block_tree_sum(sh.part, SAMPLE_THREADS);
+        const bool tie = i >= 0 && !all && key == tau;
+        bool keep = i >= 0 && (all || key > tau);
+        const int before = lanes_before(tie);
+        if (tie) keep = rank + before < n_ties;
+        rank += __popcll(__ballot(tie));
+        if (i >= 0) probs_out[i] = keep ? (float)fixed_weight(l, l_max, inv_t, min_w) * inv_total : 0.f;
+    });
 }
 
 // One block per row.  out[row] = the token; probs_out (optional, [rows, V]) = the distribution drawn from.
@@ -246,6 +311,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     __shared__ SampleShared sh;
     const float* row = logits + (size_t)blockIdx.x * V;
     float* probs_out = probs_all ? probs_all + (size_t)blockIdx.x * V : nullptr;
+    const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
     const BestPair best = block_argmax(row, V, sh.best);
     if (temperature <= 0.f || top_k == 1) {
         if (probs_out) for (int i = threadIdx.x; i < V; i += blockDim.x) probs_out[i] = i == best.i ? 1.f : 0.f;
@@ -255,61 +321,126 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     const float l_max = best.v, inv_t = 1.0f / temperature;
     const float min_w = min_p > 0.f ? min_p : 0.f;          // w_best = exp(0) = 1
     const float u = uniforms[blockIdx.x];
-    const int chunk = (V + SAMPLE_THREADS - 1) / SAMPLE_THREADS;
     const bool use_top_p = top_p > 0.f && top_p < 1.f;
+    const Range mine = wave_range(V);
 
     if (top_k <= 0 || top_k >= V) {
-        // ---- no top-k: thresholds on the logit, draw in index order ----
-        float total = mass_at_least(row, V, chunk, l_max, inv_t, min_w, 0u, false, sh);
-        uint32_t tau = 0u;
-        int n_ties = 0x7fffffff;
-        if (use_top_p) {
-            const float cutoff = top_p * total;
-            // the largest tau whose mass(key >= tau) still reaches the cutoff
-            uint32_t lo = 0u, hi = 0xffffffffu;              // invariant: mass(>= lo) >= cutoff
-            while (lo < hi) {
-                const uint32_t mid = lo + (hi - lo) / 2u + 1u;
-                const float mass = mass_at_least(row, V, chunk, l_max, inv_t, min_w, mid, false, sh);
-                if (mass >= cutoff) lo = mid; else hi = mid - 1u;
-            }
-            tau = lo;
-            const float above = mass_at_least(row, V, chunk, l_max, inv_t, min_w, tau, true, sh);
-            // all elements equal to tau weigh the same; take as many (in index order) as the cutoff needs
-            float w_tau = 0.f;
-            {
-                union { uint32_t u; float f; } c;
-                c.u = (tau & 0x80000000u) ? (tau & 0x7fffffffu) : ~tau;
-                w_tau = kept_weight(c.f, l_max, inv_t, min_w);
-            }
-            n_ties = 1;
-            float cum = above + w_tau;
-            while (cum < cutoff && w_tau > 0.f && n_ties < V) { cum += w_tau; ++n_ties; }
-            // the count of ties that exist bounds n_ties inside draw_index_order (rank < n_ties)
-            total = cum;
+        // ---- no top-k: a threshold on the logit, the draw in index order ----
+        masses_by_wave(row, V, l_max, inv_t, min_w, 0u, true, sh);
+        mass_t total = 0ull;
+        for (int w = 0; w < SAMPLE_WAVES; ++w) total += sh.wave_mass[w];
+        if (total == 0ull) {                                 // nothing has weight (a row of -inf or NaN): the first maximum
+            if (probs_out) for (int i = threadIdx.x; i < V; i += blockDim.x) probs_out[i] = i == best.i ? 1.f : 0.f;
+            if (threadIdx.x == 0) out[blockIdx.x] = best.i;
+            return;
         }
-        const int tok = draw_index_order(row, V, chunk, l_max, inv_t, min_w, tau, n_ties, u * total, sh, probs_out, total);
-        if (threadIdx.x == 0) out[blockIdx.x] = tok;
+        uint32_t tau = 0u;
+        bool all = true;
+        int n_ties = 0;
+        mass_t w_tau = 0ull;
+        if (use_top_p) {
+            // The largest tau whose elements with key >= tau weigh at least the cutoff, a byte of the key at a time
+            // from the top: the weights of the elements that match the bytes found so far, by their next byte.
+            mass_t cutoff = (mass_t)((double)top_p * (double)total);
+            if (cutoff < 1ull) cutoff = 1ull;
+            uint32_t prefix = 0u, mask = 0u;
+            mass_t above = 0ull;                             // the weight of the keys above the bytes found so far
+            __syncthreads();
+            // The top byte of a float's key is its sign and most of its exponent: most of a row shares one or two
+            // values of it, and as many additions to one histogram bin take as many turns.  Usually the elements
+            // that share the maximum's top byte already weigh as much as the cutoff: then that byte is the answer.
+            const uint32_t top = ordered_key(l_max) & 0xff000000u;
+            int first_shift = 24;
+            if (top) {
+                masses_by_wave(row, V, l_max, inv_t, min_w, top - 1u, false, sh);
+                mass_t with_top = 0ull;
+                for (int w = 0; w < SAMPLE_WAVES; ++w) with_top += sh.wave_mass[w];
+                if (with_top >= cutoff) { prefix = top; mask = 0xff000000u; first_shift = 16; }
+                __syncthreads();
+            }
+            for (int shift = first_shift; shift >= 0; shift -= 8) {
+                for (int i = threadIdx.x; i < SAMPLE_WAVES * HIST_STRIDE; i += blockDim.x) (&sh.hist.mass[0][0])[i] = 0ull;
+                __syncthreads();
+                for_range(row, mine, [&](int i, float l) {
+                    const uint32_t key = ordered_key(l);
+                    const uint32_t w = i >= 0 && (key & mask) == prefix ? fixed_weight(l, l_max, inv_t, min_w) : 0u;
+                    const int bin = w ? (int)((key >> shift) & 0xffu) : -1;
+                    if (bin >= 0) atomicAdd(&sh.hist.mass[wave][bin], (mass_t)w);
+                });
+                __syncthreads();
+                if (threadIdx.x < 256) {
+                    mass_t sum = 0ull;
+                    for (int w = 0; w < SAMPLE_WAVES; ++w) sum += sh.hist.mass[w][threadIdx.x];
+                    sh.bin_mass[threadIdx.x] = sum;
+                }
+                __syncthreads();
+                if (threadIdx.x == 0) {
+                    mass_t run = above;
+                    int bin = 255;
+                    for (; bin > 0; --bin) {
+                        if (run + sh.bin_mass[bin] >= cutoff) break;
+                        run += sh.bin_mass[bin];
+                    }
+                    sh.prefix = prefix | ((uint32_t)bin << shift);
+                    sh.above = run;
+                }
+                __syncthreads();
+                prefix = sh.prefix;
+                above = sh.above;
+                mask |= 0xffu << shift;
+            }
+            tau = prefix;
+            all = false;
+            // the elements equal to tau weigh the same; as many of them (in index order) as the cutoff needs
+            w_tau = (mass_t)fixed_weight(key_value(tau), l_max, inv_t, min_w);
+            n_ties = w_tau ? (int)min((mass_t)V, (cutoff - above + w_tau - 1ull) / w_tau) : 0;
+            total = above + (mass_t)n_ties * w_tau;
+            masses_by_wave(row, V, l_max, inv_t, min_w, tau, false, sh);
+        }
+        mass_t target = (mass_t)((double)u * (double)total);
+        if (target >= total) target = total - 1ull;
+        if (probs_out) write_probabilities(row, V, l_max, inv_t, min_w, tau, all, n_ties, total, sh, probs_out);
+        const int tok = draw_index_order(row, V, l_max, inv_t, min_w, tau, all, n_ties, w_tau, target, sh);
+        if (threadIdx.x == 0) out[blockIdx.x] = tok >= 0 ? tok : best.i;
         return;
     }
 
     // ---- top-k (k <= TOPK_MAX): select, sort, then the reference's serial walk ----
     const int k = top_k;
-    // radix select of the k-th largest key, 8 bits at a time from the top
+    // the key of the k-th largest element, a byte at a time from the top: how many of the elements that match the
+    // bytes found so far have which next byte
     uint32_t prefix = 0u, mask = 0u;
     int remaining = k;                                       // how many of the wanted lie at or below the prefix bin
-    for (int shift = 24; shift >= 0; shift -= 8) {
-        for (int i = threadIdx.x; i < 256; i += blockDim.x) sh.hist[i] = 0u;
+    // (the top byte: if k elements or more share the maximum's, it is the answer; see the search for top-p above)
+    const uint32_t top = ordered_key(best.v) & 0xff000000u;
+    int first_shift = 24;
+    if (top) {
+        masses_by_wave<false>(row, V, 0.f, 0.f, 0.f, top - 1u, false, sh);
+        mass_t with_top = 0ull;
+        for (int w = 0; w < SAMPLE_WAVES; ++w) with_top += sh.wave_mass[w];
+        if (with_top >= (mass_t)k) { prefix = top; mask = 0xff000000u; first_shift = 16; }
         __syncthreads();
-        for (int i = threadIdx.x; i < V; i += blockDim.x) {
-            const uint32_t key = ordered_key(row[i]);
-            if ((key & mask) == prefix) atomicAdd(&sh.hist[(key >> shift) & 0xffu], 1u);
+    }
+    for (int shift = first_shift; shift >= 0; shift -= 8) {
+        for (int i = threadIdx.x; i < SAMPLE_WAVES * HIST_STRIDE; i += blockDim.x) (&sh.hist.count[0][0])[i] = 0u;
+        __syncthreads();
+        for_range(row, mine, [&](int i, float l) {
+            const uint32_t key = ordered_key(l);
+            const int bin = i >= 0 && (key & mask) == prefix ? (int)((key >> shift) & 0xffu) : -1;
+            if (bin >= 0) atomicAdd(&sh.hist.count[wave][bin], 1u);
+        });
+        __syncthreads();
+        if (threadIdx.x < 256) {
+            unsigned int sum = 0u;
+            for (int w = 0; w < SAMPLE_WAVES; ++w) sum += sh.hist.count[w][threadIdx.x];
+            sh.bin_mass[threadIdx.x] = sum;
         }
         __syncthreads();
         if (threadIdx.x == 0) {
             int need = remaining;
             int bin = 255;
             for (; bin > 0; --bin) {
-                const int c = (int)sh.hist[bin];
+                const int c = (int)sh.bin_mass[bin];
                 if (c >= need) break;
                 need -= c;
             }
@@ -320,35 +451,29 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
         prefix = sh.prefix;
         remaining = sh.remaining;
         mask |= 0xffu << shift;
-        __syncthreads();
     }
     const uint32_t tau = prefix;                             // key of the k-th largest
     const int ties_wanted = remaining;                       // how many elements equal to tau belong to the k
 
-    // gather: everything above tau, and the first `ties_wanted` elements equal to tau in index order
-    const int begin = threadIdx.x * chunk, end = min(V, begin + chunk);
-    int my_ties = 0;
-    for (int i = begin; i < end; ++i) my_ties += ordered_key(row[i]) == tau;
-    sh.cnt[threadIdx.x] = my_ties;
-    if (threadIdx.x == 0) sh.n_cand = 0;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        int run = 0;
-        for (int t = 0; t < SAMPLE_THREADS; ++t) { const int c = sh.cnt[t]; sh.cnt[t] = run; run += c; }
-    }
-    __syncthreads();
+    // gather: everything above tau, and the first `ties_wanted` elements equal to tau in index order; the last
+    // histogram holds, for each wave, how many of its elements equal tau
     {
-        int rank = sh.cnt[threadIdx.x];
-        for (int i = begin; i < end; ++i) {
-            const float l = row[i];
+        int rank = 0;
+        for (int w = 0; w < wave; ++w) rank += (int)sh.hist.count[w][tau & 0xffu];
+        if (threadIdx.x == 0) sh.n_cand = 0;
+        __syncthreads();
+        for_range(row, mine, [&](int i, float l) {
             const uint32_t key = ordered_key(l);
-            bool keep = key > tau;
-            if (key == tau) { keep = rank < ties_wanted; ++rank; }
+            const bool tie = i >= 0 && key == tau;
+            bool keep = i >= 0 && key > tau;
+            const int before = lanes_before(tie);
+            if (tie) keep = rank + before < ties_wanted;
+            rank += __popcll(__ballot(tie));
             if (keep) {
                 const int slot = atomicAdd(&sh.n_cand, 1);
                 if (slot < TOPK_MAX) { sh.cand_v[slot] = l; sh.cand_i[slot] = i; }
             }
-        }
+        });
     }
     __syncthreads();
     const int n_cand = min(sh.n_cand, TOPK_MAX);
