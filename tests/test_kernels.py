@@ -513,6 +513,18 @@ def test_rows_are_sampled_independently(ops):
     together = ops.sample(lg.to(DEV), u.to(DEV), 1.0, 20, 0.9, 0.0).cpu().tolist()
     alone = [ops.sample(lg[r:r + 1].to(DEV), u[r:r + 1].to(DEV), 1.0, 20, 0.9, 0.0).item() for r in range(4)]
     assert together == alone
+    # without top-k, on a wide row of an odd width, and again and again: weights are added as integers, so not
+    # a bit depends on the order in which the block's waves arrive
+    lg = rand(4, 151937, seed=9, scale=3.0)
+    for args in ((0.8, 0, 0.9, 0.0), (1.2, 0, 1.0, 0.02), (1.0, 0, 1.0, 0.0)):
+        together = ops.sample(lg.to(DEV), u.to(DEV), *args).cpu().tolist()
+        alone = [ops.sample(lg[r:r + 1].to(DEV), u[r:r + 1].to(DEV), *args).item() for r in range(4)]
+        assert together == alone and together == ops.sample(lg.to(DEV), u.to(DEV), *args).cpu().tolist(), args
+        probs = ops.sample(lg.to(DEV), u.to(DEV), *args, want_probs=True)[1].cpu().double()
+        assert all(float(probs[r, together[r]]) > 0 for r in range(4)), args
+        for r in range(4):           # the token is where the kept weights, added up in index order, pass u
+            cdf = torch.cumsum(probs[r], 0)
+            assert float(cdf[together[r]] - probs[r, together[r]]) - 1e-4 <= float(u[r]) <= float(cdf[together[r]]) + 1e-4, (args, r)
 
 
 def test_penalties(ops):
