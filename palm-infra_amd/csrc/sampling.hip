@@ -130,6 +130,18 @@ PALM_API int palm_apply_penalties(hipStream_t stream, float* logits, int V, cons
 constexpr int SAMPLE_WAVES = SAMPLE_THREADS / WAVE;
 constexpr float FIXED_ONE = 2147483648.0f;           // 2^31: a weight fits 32 bits, a row's sum 64
 constexpr int HIST_STRIDE = 257;                     // a wave's histogram starts one bank on from its neighbour's
+constexpr int SEG_CAP = 256;                         // elements a wave can set aside for the later passes of top-k
+constexpr int COARSE_BINS = 1024;
+static_assert(COARSE_BINS == SAMPLE_THREADS, "a thread a bin in the scan over the bins");
+
+// 0 for the row's maximum, growing with the distance below it: 64 bins for each doubling of (distance + 1), so
+// the few elements near the top have bins to themselves, and the many far below still spread over some dozen bins
+// (additions to one bin take turns).  Monotone: an element in a lower bin is at least as large as one in a higher.
+__device__ inline int coarse_bin(float l, float l_max) {
+    const float f = (l_max - l) + 1.0f;                        // at least 1, or NaN
+    const uint32_t b = (__float_as_uint(f) - 0x3f800000u) >> 17;
+    return f >= 1.0f ? (int)min(b, (uint32_t)COARSE_BINS - 1u) : COARSE_BINS - 1;
+}
 typedef unsigned long long mass_t;
 
 struct SampleShared {
@@ -137,7 +149,13 @@ struct SampleShared {
     union {
         mass_t mass[SAMPLE_WAVES][HIST_STRIDE];          // a histogram for each wave: weights by a byte of the key
         unsigned int count[SAMPLE_WAVES][HIST_STRIDE];   //                            elements by a byte of the key
+        struct {                                         // or: the few elements still in the running, by wave
+            uint32_t key[SAMPLE_WAVES][SEG_CAP];
+            int idx[SAMPLE_WAVES][SEG_CAP];
+        } seg;
     } hist;
+    unsigned int small[256];                     // one histogram for the block, where few elements are counted
+    unsigned int coarse[COARSE_BINS];            // elements by their distance below the maximum
     mass_t bin_mass[256];
     mass_t wave_mass[SAMPLE_WAVES];              // weights above the threshold, by wave; then by wave of threads
     int wave_ties[SAMPLE_WAVES];                 // elements at the threshold
@@ -411,28 +429,70 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     // bytes found so far have which next byte
     uint32_t prefix = 0u, mask = 0u;
     int remaining = k;                                       // how many of the wanted lie at or below the prefix bin
-    // (the top byte: if k elements or more share the maximum's, it is the answer; see the search for top-p above)
-    const uint32_t top = ordered_key(best.v) & 0xff000000u;
-    int first_shift = 24;
-    if (top) {
-        masses_by_wave<false>(row, V, 0.f, 0.f, 0.f, top - 1u, false, sh);
-        mass_t with_top = 0ull;
-        for (int w = 0; w < SAMPLE_WAVES; ++w) with_top += sh.wave_mass[w];
-        if (with_top >= (mass_t)k) { prefix = top; mask = 0xff000000u; first_shift = 16; }
+    // First a coarse cut: count the elements by their distance below the maximum, find the bin in which the k-th
+    // largest lies, and set the elements of the bins up to it aside, by wave and in index order.  If every wave's
+    // fit, the exact search and the gathering walk them instead of the row.
+    int seg_n = 0;
+    bool compact = false;
+    {
+        sh.coarse[threadIdx.x] = 0u;
+        __syncthreads();
+        for_range(row, mine, [&](int i, float l) { if (i >= 0) atomicAdd(&sh.coarse[coarse_bin(l, best.v)], 1u); });
+        __syncthreads();
+        // a scan over the bins, a thread a bin: the bin where the running count reaches k
+        const int mine_c = (int)sh.coarse[threadIdx.x];
+        int scan = mine_c;
+#pragma unroll
+        for (int off = 1; off < WAVE; off <<= 1) { const int o = __shfl_up(scan, off, WAVE); if (lane >= off) scan += o; }
+        if (lane == WAVE - 1) sh.wave_ties[wave] = scan;
+        if (threadIdx.x == 0) sh.owner = COARSE_BINS - 1;
+        __syncthreads();
+        for (int w = 0; w < wave; ++w) scan += sh.wave_ties[w];
+        if (scan - mine_c < k && k <= scan) sh.owner = threadIdx.x;
+        __syncthreads();
+        const int cut = sh.owner;
+        int n = 0;
+        for_range(row, mine, [&](int i, float l) {
+            const bool match = i >= 0 && coarse_bin(l, best.v) <= cut;
+            const int at = n + lanes_before(match);
+            if (match && at < SEG_CAP) { sh.hist.seg.key[wave][at] = ordered_key(l); sh.hist.seg.idx[wave][at] = i; }
+            n += __popcll(__ballot(match));
+        });
+        __syncthreads();                                     // (wave_ties is read above)
+        if (lane == 0) sh.wave_ties[wave] = n;
+        __syncthreads();
+        bool fits = true;
+        for (int w = 0; w < SAMPLE_WAVES; ++w) fits = fits && sh.wave_ties[w] <= SEG_CAP;
+        compact = fits;
+        seg_n = compact ? n : 0;
         __syncthreads();
     }
+    const int first_shift = 24;
+    // f(i, l) for the elements in the running, in index order within the wave
+    auto each = [&](auto&& f) {
+        if (compact) {
+            for (int j0 = 0; j0 < seg_n; j0 += WAVE) {
+                const bool valid = j0 + lane < seg_n;
+                f(valid ? sh.hist.seg.idx[wave][j0 + lane] : -1, valid ? key_value(sh.hist.seg.key[wave][j0 + lane]) : -INFINITY);
+            }
+        } else {
+            for_range(row, mine, f);
+        }
+    };
     for (int shift = first_shift; shift >= 0; shift -= 8) {
-        for (int i = threadIdx.x; i < SAMPLE_WAVES * HIST_STRIDE; i += blockDim.x) (&sh.hist.count[0][0])[i] = 0u;
+        if (compact) { if (threadIdx.x < 256) sh.small[threadIdx.x] = 0u; }
+        else for (int i = threadIdx.x; i < SAMPLE_WAVES * HIST_STRIDE; i += blockDim.x) (&sh.hist.count[0][0])[i] = 0u;
         __syncthreads();
-        for_range(row, mine, [&](int i, float l) {
+        each([&](int i, float l) {
             const uint32_t key = ordered_key(l);
             const int bin = i >= 0 && (key & mask) == prefix ? (int)((key >> shift) & 0xffu) : -1;
-            if (bin >= 0) atomicAdd(&sh.hist.count[wave][bin], 1u);
+            if (bin >= 0) atomicAdd(compact ? &sh.small[bin] : &sh.hist.count[wave][bin], 1u);
         });
         __syncthreads();
         if (threadIdx.x < 256) {
             unsigned int sum = 0u;
-            for (int w = 0; w < SAMPLE_WAVES; ++w) sum += sh.hist.count[w][threadIdx.x];
+            if (compact) sum = sh.small[threadIdx.x];
+            else for (int w = 0; w < SAMPLE_WAVES; ++w) sum += sh.hist.count[w][threadIdx.x];
             sh.bin_mass[threadIdx.x] = sum;
         }
         __syncthreads();
@@ -455,14 +515,22 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     const uint32_t tau = prefix;                             // key of the k-th largest
     const int ties_wanted = remaining;                       // how many elements equal to tau belong to the k
 
-    // gather: everything above tau, and the first `ties_wanted` elements equal to tau in index order; the last
-    // histogram holds, for each wave, how many of its elements equal tau
+    // gather: everything above tau, and the first `ties_wanted` elements equal to tau in index order
     {
         int rank = 0;
-        for (int w = 0; w < wave; ++w) rank += (int)sh.hist.count[w][tau & 0xffu];
+        if (compact) {
+            int ties = 0;
+            each([&](int i, float l) { ties += i >= 0 && ordered_key(l) == tau; });
+            ties = wave_sum(ties);
+            if (lane == 0) sh.wave_ties[wave] = ties;
+            __syncthreads();
+            for (int w = 0; w < wave; ++w) rank += sh.wave_ties[w];
+        } else {                                             // the last histogram holds each wave's count of them
+            for (int w = 0; w < wave; ++w) rank += (int)sh.hist.count[w][tau & 0xffu];
+        }
         if (threadIdx.x == 0) sh.n_cand = 0;
         __syncthreads();
-        for_range(row, mine, [&](int i, float l) {
+        each([&](int i, float l) {
             const uint32_t key = ordered_key(l);
             const bool tie = i >= 0 && key == tau;
             bool keep = i >= 0 && key > tau;

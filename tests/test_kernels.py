@@ -507,6 +507,22 @@ def test_draws_walk_the_kept_set_and_follow_u(ops):
         assert tok == P.draw(lg[0].double().numpy(), u, temperature=0.9, top_k=40, top_p=0.95), u
 
 
+def test_top_k_where_the_candidates_do_not_stand_out(ops):
+    """Rows whose k largest are not a few elements near the top: all equal, half of them equal to the maximum, and
+    a maximum far above a flat rest (the kernel's coarse cut does not thin these out, so its slow way runs)."""
+    V = 9001
+    flat = torch.zeros(V)
+    half = rand(V, seed=3, dtype=F32)
+    half[::2] = float(half.max()) + 1.0
+    spike = rand(V, seed=4, dtype=F32) * 1e-3
+    spike[4321] = 500.0
+    for lg in (flat, half, spike):
+        for k in (1, 5, 300):
+            for u in (0.0, 0.3, 0.77, 0.9999):
+                tok = ops.sample(lg.reshape(1, -1).to(DEV), torch.tensor([u], dtype=F32).to(DEV), 0.9, k, 1.0, 0.0).item()
+                assert tok == P.draw(lg.double().numpy(), u, temperature=0.9, top_k=k), (k, u)
+
+
 def test_rows_are_sampled_independently(ops):
     lg = rand(4, 2000, seed=8)
     u = torch.tensor([0.1, 0.5, 0.9, 0.3])
