@@ -21,7 +21,7 @@ import sys
 import tempfile
 import threading
 import time
-from concurrent.futures import ThreadPoolExecutor
+from concurrent.futures import ThreadPoolExecutor, wait
 from pathlib import Path
 
 CSRC = Path(__file__).resolve().parent.parent / "csrc"
@@ -32,9 +32,10 @@ FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-fno-gpu-rdc",
          "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option"]
 
 CORE_SOURCES = ["elementwise.hip", "linear.hip", "rope_store.hip", "attention_simple.hip", "sampling.hip",
-                "linear_mfma.hip", "linear_wide.hip"]
+                "linear_mfma.hip", "linear_wide.hip", "linear_wide_store_32.hip", "linear_wide_store_64.hip",
+                "linear_wide_gated_32.hip", "linear_wide_gated_64.hip"]
 ATTENTION_SOURCES = ["attention_mfma.hip"]
-HEADERS = ["common.h", "mfma.h"]
+HEADERS = ["common.h", "mfma.h", "linear_wide.h"]
 
 
 class KernelBuildError(RuntimeError):
@@ -130,7 +131,13 @@ def _compile(name: str, sources, defines, force: bool) -> Path:
 
     try:
         with ThreadPoolExecutor(max_workers=min(8, len(sources))) as pool:
-            objs = list(pool.map(one, sources))
+            jobs = [pool.submit(one, src) for src in sources]
+            pending = set(jobs)
+            while pending:                               # a line now and then, so that a long compile is seen to be alive
+                done, pending = wait(pending, timeout=15)
+                if pending and not done:
+                    _say(f"  still compiling, {len(pending)} of {len(jobs)} files to go ({time.time() - t0:.0f} s)")
+            objs = [j.result() for j in jobs]
         tmp = out.with_suffix(f".tmp{os.getpid()}")
         r = subprocess.run([hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-fno-gpu-rdc",
                             *[str(o) for o in objs], "-o", str(tmp)], capture_output=True, text=True, env=env)
