@@ -429,6 +429,7 @@ def linear_thin(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, gated:
         library.call(core(), "palm_linear_thin", _stream(), _p(a), _p(w), _p(out), _code(out, "linear_thin out"), M, N, K,
                      1 if gated else 0, planes, _p(row_ss), pieces, float(row_eps), None, None, None)
         return out
+    _need(row_ss is None, f"linear_thin: rows that lack their norm's factor come at most {THIN_TOKENS} at a time, not {M}")
     if M > WIDE_TOKENS:
         # the weight goes by once for every 64 rows (a float32 result for many rows: logits at many places)
         return torch.cat([linear_thin(a[r0:r0 + WIDE_TOKENS], w, out_dtype, gated=gated)

@@ -123,6 +123,8 @@ def test_the_folded_norm_refuses_what_it_does_not_serve(ops):
         ops.linear_thin_into_residual(a[:4].contiguous(), w, x[:4, :8].contiguous(), nw)
     with pytest.raises(KernelError, match="sums of squares"):
         ops.linear_thin(a[:4].contiguous(), w, F32, row_ss=torch.zeros(5, 2, device=DEV), row_eps=1e-6)
+    with pytest.raises(KernelError, match="at most 16"):          # the kernel for 17 to 64 rows applies no row factor
+        ops.linear_thin(a, w, F32, row_ss=torch.ones(17, 2, device=DEV), row_eps=1e-6)
 
 
 def test_linear_thin_orientation(ops):
