@@ -315,13 +315,20 @@ PALM_API int palm_attention_decode(hipStream_t stream, const void* q, const void
 constexpr int PF_WAVES = 4;
 constexpr int PF_THREADS = PF_WAVES * WAVE;
 constexpr int PF_UNITS = 2;                                // units of 16 columns held by a wave
+constexpr float PF_LAZY_LOG2 = 8.0f;                       // how far (in powers of two) a maximum may rise before the outputs are rescaled
 // K rows in LDS are a multiple of eight 16-byte chunks long and a row's chunks are permuted by its number
 // (chunk ^ swizzle(row)): the eight lanes that LDS serves together read one chunk column of keys
 // {0..3, 8..11} (or {4..7, 12..15}, ..), which the permutation sends to eight different bank groups.
 constexpr int K_CHUNKS = (CHUNKS + 7) / 8 * 8;
 constexpr int K_STRIDE = K_CHUNKS * 8;
 __device__ inline int k_swizzle(int row) { return (row & 3) | (((row >> 3) & 1) << 2); }
-constexpr int V_STRIDE = PAGE_TOKENS + 8;
+// Head sizes whose key rows are whole multiples of 128 bytes (64, 128) take their pages from memory straight into
+// LDS (global_load_lds: no registers in between, no write instruction); a wave's instruction fills 1 KB of LDS
+// in lane order, so rows cannot be padded there and V^T's chunks are permuted like K's instead (row d's chunk c
+// at c ^ v_swizzle(d): the 16 rows that lanes read together then start in 16 different groups of four banks).
+constexpr bool PF_DMA = CHUNKS % 8 == 0 && (PAGE_TOKENS * K_STRIDE + HD * PAGE_TOKENS) * 2 <= 60 * 1024;
+constexpr int V_STRIDE = PF_DMA ? PAGE_TOKENS : PAGE_TOKENS + 8;
+__device__ inline int v_swizzle(int row) { return PF_DMA ? (row >> 1) & 7 : 0; }
 constexpr int PAGE_CHUNKS = PAGE_TOKENS * HD / 8;          // 16-byte chunks in a page of K (and of V^T)
 constexpr int PF_LOADS = (PAGE_CHUNKS + PF_THREADS - 1) / PF_THREADS;
 constexpr bool PF_SHARE = (PAGE_TOKENS * K_STRIDE + HD * V_STRIDE) * 2 > 60 * 1024;   // too big for 64 KB: V reuses K's space
@@ -353,8 +360,41 @@ __device__ inline void stage_values(const PagePrefetch& pf, bf16_t* v_lds) {
 #pragma unroll
     for (int i = 0; i < PF_LOADS; ++i) {
         const int c = i * PF_THREADS + threadIdx.x;
-        if (c < PAGE_CHUNKS) *reinterpret_cast<bf16x8*>(v_lds + (c / 8) * V_STRIDE + (c % 8) * 8) = pf.v[i];
+        if (c < PAGE_CHUNKS) *reinterpret_cast<bf16x8*>(v_lds + (c / 8) * V_STRIDE + ((c % 8) ^ v_swizzle(c / 8)) * 8) = pf.v[i];
     }
+}
+
+// A page of K and of V^T from memory into LDS without a stop in registers.  An instruction of a wave fills 1 KB
+// in lane order: for K that is 64 / CHUNKS key rows, for V^T eight rows of 64 tokens; a lane asks for the chunk
+// that belongs at its place.  k_from / v_from: the lane's places in a page, as page_sources() gives them.
+struct PageSources { uint32_t k[PF_LOADS], v[PF_LOADS]; };       // byte offsets into a page of K and of V^T
+__device__ inline PageSources page_sources() {
+    PageSources src;
+    const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
+    constexpr int K_ROWS = WAVE / (CHUNKS > 0 ? CHUNKS : 1);     // key rows an instruction covers
+#pragma unroll
+    for (int i = 0; i < PF_LOADS; ++i) {
+        const int inst = i * PF_WAVES + wave;
+        const int k_row = inst * K_ROWS + lane / CHUNKS, v_row = inst * 8 + lane / 8;
+        src.k[i] = (uint32_t)(k_row * HD + ((lane % CHUNKS) ^ k_swizzle(k_row)) * 8) * sizeof(bf16_t);
+        src.v[i] = (uint32_t)(v_row * PAGE_TOKENS + ((lane % 8) ^ v_swizzle(v_row)) * 8) * sizeof(bf16_t);
+    }
+    return src;
+}
+__device__ inline void page_into_lds(const bf16_t* __restrict__ kp, const bf16_t* __restrict__ vp, const PageSources& src,
+                                     bf16_t* k_lds, bf16_t* v_lds) {
+    typedef const __attribute__((address_space(1))) void* global_ptr;
+    typedef __attribute__((address_space(3))) void* lds_ptr;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
+    constexpr int KB = 1024 / sizeof(bf16_t);                    // elements of 1 KB
+#pragma unroll
+    for (int i = 0; i < PF_LOADS; ++i)
+        __builtin_amdgcn_global_load_lds((global_ptr)(reinterpret_cast<const char*>(kp) + src.k[i]),
+                                         (lds_ptr)(k_lds + (i * PF_WAVES + wave) * KB), 16, 0, 0);
+#pragma unroll
+    for (int i = 0; i < PF_LOADS; ++i)
+        __builtin_amdgcn_global_load_lds((global_ptr)(reinterpret_cast<const char*>(vp) + src.v[i]),
+                                         (lds_ptr)(v_lds + (i * PF_WAVES + wave) * KB), 16, 0, 0);
 }
 
 struct Unit {                 // one (head, 16 query positions): the wave's share of it
@@ -366,7 +406,8 @@ struct Unit {                 // one (head, 16 query positions): the wave's shar
     size_t row;               // the column's row in q and out
     int head;
     bf16x8 qv[KSTEPS];
-    Columns c;
+    Columns c;                // (c.l is not used here: see weights)
+    f32x4 weights;            // the sum of the column's softmax weights, four times
 };
 
 __device__ inline void read_key_fragments(const bf16_t* k_lds, int t, int r, int g, bf16x8 (&kf)[KSTEPS]) {
@@ -393,12 +434,12 @@ __device__ inline void unit_scores(const bf16_t* k_lds, Unit (&u)[PF_UNITS], int
     for (int t = 0; t < 4; ++t) {
         if (t < 3) read_key_fragments(k_lds, t + 1, r, g, kf[(t + 1) & 1]);
 #pragma unroll
-        for (int x = 0; x < PF_UNITS; ++x) s[x][t] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
         for (int x = 0; x < PF_UNITS; ++x) {
-            if (!u[x].active) continue;
+            if (!u[x].active) continue;                         // (its scores stay unset and unused)
+            f32x4 acc = mfma_16x16x32(kf[t & 1][0], u[x].qv[0], f32x4{0.f, 0.f, 0.f, 0.f});
 #pragma unroll
-            for (int j = 0; j < KSTEPS; ++j) s[x][t] = mfma_16x16x32(kf[t & 1][j], u[x].qv[j], s[x][t]);
+            for (int j = 1; j < KSTEPS; ++j) acc = mfma_16x16x32(kf[t & 1][j], u[x].qv[j], acc);
+            s[x][t] = acc;
         }
     }
 #pragma unroll
@@ -427,20 +468,20 @@ __device__ inline void unit_scores(const bf16_t* k_lds, Unit (&u)[PF_UNITS], int
         mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
         mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
         mx *= scale_log2;                                           // the scale is positive: the maximum commutes with it
-        const float m_new = fmaxf(c.m, mx);
-        const float m_sub = m_new == -INFINITY ? 0.f : m_new;       // see score_page
-        alpha[x] = exp2_weight(c.m - m_sub);
-        float sum = 0.f;
+        // c.m is the reference the weights are taken against, not the running maximum itself: it follows the
+        // maximum only when that has risen by more than PF_LAZY_LOG2 above it (from -inf: at the first key).
+        // Until then the weights are at most 2^PF_LAZY_LOG2 instead of at most 1, which 32-bit sums and the
+        // bfloat16 operand hold as well, and the outputs need no rescaling.
+        const bool jump = mx > c.m + PF_LAZY_LOG2;
+        const float m_ref = jump ? mx : c.m;
+        const float m_sub = m_ref == -INFINITY ? 0.f : m_ref;       // see score_page
+        alpha[x] = jump ? exp2_weight(c.m - m_sub) : 1.0f;
 #pragma unroll
         for (int h = 0; h < 2; ++h)
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const float p = exp2_weight(fmaf(s[x][2 * h + e / 4][e % 4], scale_log2, -m_sub));
-                sum += p;
-                pv[x][h][e] = (__bf16)p;
-            }
-        c.l = c.l * alpha[x] + sum;
-        c.m = m_new;
+            for (int e = 0; e < 8; ++e)
+                pv[x][h][e] = (__bf16)exp2_weight(fmaf(s[x][2 * h + e / 4][e % 4], scale_log2, -m_sub));
+        c.m = m_ref;
     }
 }
 
@@ -454,17 +495,30 @@ __device__ inline void unit_values(const bf16_t* v_lds, Unit (&u)[PF_UNITS], int
             if (!u[x].active) continue;
 #pragma unroll
             for (int dt = 0; dt < DTILES; ++dt) u[x].c.o[dt] = u[x].c.o[dt] * alpha[x];
+            u[x].weights = u[x].weights * alpha[x];
         }
+    }
+    // the sum of a column's weights comes from the matrix cores too: a row of ones in place of a row of V^T (every
+    // row of the tile is that row: each of a lane's four elements is the whole sum over the page's keys)
+    bf16x8 ones;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ones[e] = (__bf16)1.0f;
+#pragma unroll
+    for (int x = 0; x < PF_UNITS; ++x) {
+        if (!u[x].active) continue;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) u[x].weights = mfma_16x16x32(ones, pv[x][h], u[x].weights);
     }
     bf16x8 vf[2][2];
 #pragma unroll
-    for (int h = 0; h < 2; ++h) vf[0][h] = *reinterpret_cast<const bf16x8*>(v_lds + r * V_STRIDE + h * 32 + g * 8);
+    for (int h = 0; h < 2; ++h) vf[0][h] = *reinterpret_cast<const bf16x8*>(v_lds + r * V_STRIDE + ((h * 4 + g) ^ v_swizzle(r)) * 8);
 #pragma unroll
     for (int dt = 0; dt < DTILES; ++dt) {
         if (dt + 1 < DTILES) {
             const bf16_t* vrow = v_lds + ((dt + 1) * 16 + r) * V_STRIDE;
 #pragma unroll
-            for (int h = 0; h < 2; ++h) vf[(dt + 1) & 1][h] = *reinterpret_cast<const bf16x8*>(vrow + h * 32 + g * 8);
+            for (int h = 0; h < 2; ++h)
+                vf[(dt + 1) & 1][h] = *reinterpret_cast<const bf16x8*>(vrow + ((h * 4 + g) ^ v_swizzle((dt + 1) * 16 + r)) * 8);
         }
 #pragma unroll
         for (int x = 0; x < PF_UNITS; ++x) {
@@ -538,6 +592,7 @@ __global__ __launch_bounds__(PF_THREADS) PF_WAVES_PER_SIMD void attention_prefil
         load_query(q + (u[x].row * nh + u[x].head) * HD, true, g, u[x].qv);
         u[x].c.m = -INFINITY;
         u[x].c.l = 0.f;
+        u[x].weights = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int dt = 0; dt < DTILES; ++dt) u[x].c.o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
@@ -551,10 +606,16 @@ __global__ __launch_bounds__(PF_THREADS) PF_WAVES_PER_SIMD void attention_prefil
         p_lo = min(p_lo, window > 0 ? max(0, start + tile16 * 16 - window + 1) / PAGE_TOKENS : 0);
     }
     PagePrefetch pf;
+    PageSources sources;
     {
         const size_t base = ((size_t)pages[p_lo] * nkv + kvh) * PAGE_TOKENS * HD;
-        prefetch_keys(k_cache + base, pf);
-        prefetch_values(v_cache + base, pf);
+        if constexpr (PF_DMA) {
+            sources = page_sources();
+            page_into_lds(k_cache + base, v_cache + base, sources, k_lds, v_lds);
+        } else {
+            prefetch_keys(k_cache + base, pf);
+            prefetch_values(v_cache + base, pf);
+        }
     }
     // is every key of page p visible to every column of this wave that takes part?  (also marks who does)
     auto page_is_interior = [&](int p) -> bool {
@@ -566,17 +627,23 @@ __global__ __launch_bounds__(PF_THREADS) PF_WAVES_PER_SIMD void attention_prefil
         }
         return __all(inside);
     };
-    if (!PF_SHARE) {
-        stage_keys(pf, k_lds);
-        stage_values(pf, v_lds);
+    if constexpr (!PF_SHARE) {
+        if constexpr (!PF_DMA) {
+            stage_keys(pf, k_lds);
+            stage_values(pf, v_lds);
+        }
         __syncthreads();
         for (int p = p_lo; p <= p_hi; ++p) {
             const int buf = (p - p_lo) & 1;
             const bool more = p < p_hi;
             if (more) {                                         // in flight while this page is used
                 const size_t next = ((size_t)pages[p + 1] * nkv + kvh) * PAGE_TOKENS * HD;
-                prefetch_keys(k_cache + next, pf);
-                prefetch_values(v_cache + next, pf);
+                if constexpr (PF_DMA) {     // straight into the other buffer, whose last readers passed the barrier a page ago
+                    page_into_lds(k_cache + next, v_cache + next, sources, k_lds + (buf ^ 1) * K_TILE, v_lds + (buf ^ 1) * V_TILE);
+                } else {
+                    prefetch_keys(k_cache + next, pf);
+                    prefetch_values(v_cache + next, pf);
+                }
             }
             bf16x8 pv[PF_UNITS][2];
             float alpha[PF_UNITS];
@@ -586,11 +653,13 @@ __global__ __launch_bounds__(PF_THREADS) PF_WAVES_PER_SIMD void attention_prefil
 #pragma unroll
             for (int x = 0; x < PF_UNITS; ++x) moved = moved || alpha[x] != 1.0f;
             unit_values(v_lds + buf * V_TILE, u, r, g, pv, alpha, __any(moved));
-            if (more) {                                         // the other buffer's last readers passed the barrier a page ago
-                stage_keys(pf, k_lds + (buf ^ 1) * K_TILE);
-                stage_values(pf, v_lds + (buf ^ 1) * V_TILE);
+            if constexpr (!PF_DMA) {
+                if (more) {                                     // the other buffer's last readers passed the barrier a page ago
+                    stage_keys(pf, k_lds + (buf ^ 1) * K_TILE);
+                    stage_values(pf, v_lds + (buf ^ 1) * V_TILE);
+                }
             }
-            __syncthreads();
+            __syncthreads();                                    // (waits for the reads into LDS, too)
         }
     } else {
         for (int p = p_lo; p <= p_hi; ++p) {
@@ -618,9 +687,7 @@ __global__ __launch_bounds__(PF_THREADS) PF_WAVES_PER_SIMD void attention_prefil
 
 #pragma unroll
     for (int x = 0; x < PF_UNITS; ++x) {
-        float l = u[x].c.l;
-        l += __shfl_xor(l, 16, WAVE);
-        l += __shfl_xor(l, 32, WAVE);
+        const float l = u[x].weights[0];
         if (u[x].valid) {
             const float inv = 1.0f / l;
             bf16_t* o = out + (u[x].row * nh + u[x].head) * HD;
