@@ -155,7 +155,10 @@ struct SampleShared {
         } seg;
     } hist;
     unsigned int small[256];                     // one histogram for the block, where few elements are counted
-    unsigned int coarse[COARSE_BINS];            // elements by their distance below the maximum
+    union {                                      // by the distance below the maximum:
+        unsigned int coarse[COARSE_BINS];        //   elements (top-k)
+        mass_t coarse_mass[COARSE_BINS];         //   weights (top-p)
+    };
     mass_t bin_mass[256];
     mass_t wave_mass[SAMPLE_WAVES];              // weights above the threshold, by wave; then by wave of threads
     int wave_ties[SAMPLE_WAVES];                 // elements at the threshold
@@ -344,9 +347,25 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
 
     if (top_k <= 0 || top_k >= V) {
         // ---- no top-k: a threshold on the logit, the draw in index order ----
-        masses_by_wave(row, V, l_max, inv_t, min_w, 0u, true, sh);
+        // the weight of the whole row: by wave for the draw, or (top-p, which first looks for its threshold) by distance
+        // below the maximum, see below
+        const bool coarse_first = use_top_p && !probs_out;
         mass_t total = 0ull;
-        for (int w = 0; w < SAMPLE_WAVES; ++w) total += sh.wave_mass[w];
+        if (coarse_first) {
+            sh.coarse_mass[threadIdx.x] = 0ull;
+            __syncthreads();
+            for_range(row, mine, [&](int i, float l) {
+                const uint32_t w = i >= 0 ? fixed_weight(l, l_max, inv_t, min_w) : 0u;
+                if (w) atomicAdd(&sh.coarse_mass[coarse_bin(l, l_max)], (mass_t)w);
+            });
+            __syncthreads();
+            mass_t part = 0ull;
+            for (int b = lane; b < COARSE_BINS; b += WAVE) part += sh.coarse_mass[b];
+            total = wave_sum(part);
+        } else {
+            masses_by_wave(row, V, l_max, inv_t, min_w, 0u, true, sh);
+            for (int w = 0; w < SAMPLE_WAVES; ++w) total += sh.wave_mass[w];
+        }
         if (total == 0ull) {                                 // nothing has weight (a row of -inf or NaN): the first maximum
             if (probs_out) for (int i = threadIdx.x; i < V; i += blockDim.x) probs_out[i] = i == best.i ? 1.f : 0.f;
             if (threadIdx.x == 0) out[blockIdx.x] = best.i;
@@ -364,6 +383,130 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
             uint32_t prefix = 0u, mask = 0u;
             mass_t above = 0ull;                             // the weight of the keys above the bytes found so far
             __syncthreads();
+            // First a coarse cut, as for top-k: the weights by their distance below the maximum (added up above), the bin in
+            // which they reach the cutoff, the elements of the bins up to it set aside.  If they fit, the threshold, the
+            // ties and the draw are found among them.  (The probabilities are written from the row: not here.)
+            if (coarse_first) {
+                const mass_t mine_m = sh.coarse_mass[threadIdx.x];
+                mass_t scan = mine_m;
+#pragma unroll
+                for (int off = 1; off < WAVE; off <<= 1) { const mass_t o = __shfl_up(scan, off, WAVE); if (lane >= off) scan += o; }
+                if (lane == WAVE - 1) sh.wave_mass[wave] = scan;
+                if (threadIdx.x == 0) sh.owner = COARSE_BINS - 1;
+                __syncthreads();
+                for (int w = 0; w < wave; ++w) scan += sh.wave_mass[w];
+                if (scan - mine_m < cutoff && cutoff <= scan) sh.owner = threadIdx.x;
+                __syncthreads();
+                const int cut = sh.owner;
+                // How many elements that is at least: a bin's weight over the largest weight an element of it can
+                // have.  A flat row keeps most of its elements; then setting them aside is a pass for nothing.
+                if (threadIdx.x == 0) sh.n_cand = 0;
+                __syncthreads();
+                if ((int)threadIdx.x <= cut && mine_m) {
+                    const float nearest = __uint_as_float(((uint32_t)threadIdx.x << 17) + 0x3f800000u) - 1.0f;   // coarse_bin, backwards
+                    const mass_t heaviest = (mass_t)fixed_weight(l_max - nearest, l_max, inv_t, 0.f) + 1ull;
+                    atomicAdd(&sh.n_cand, (int)min(mine_m / heaviest, (mass_t)(1 << 20)));
+                }
+                __syncthreads();
+                bool fits = sh.n_cand <= SEG_CAP * SAMPLE_WAVES;
+                int seg_n = 0;
+                if (fits) {
+                    for_range(row, mine, [&](int i, float l) {
+                        const bool match = i >= 0 && coarse_bin(l, l_max) <= cut;
+                        const int at = seg_n + lanes_before(match);
+                        if (match && at < SEG_CAP) { sh.hist.seg.key[wave][at] = ordered_key(l); sh.hist.seg.idx[wave][at] = i; }
+                        seg_n += __popcll(__ballot(match));
+                    });
+                    if (lane == 0) sh.wave_ties[wave] = seg_n;
+                    __syncthreads();
+                    for (int w = 0; w < SAMPLE_WAVES; ++w) fits = fits && sh.wave_ties[w] <= SEG_CAP;
+                    __syncthreads();
+                }
+                if (fits) {
+                    // f(key, index) for the wave's elements set aside, in index order; every lane takes part in every step
+                    auto each = [&](auto&& f) {
+                        for (int j0 = 0; j0 < seg_n; j0 += WAVE) {
+                            const bool valid = j0 + lane < seg_n;
+                            f(valid ? sh.hist.seg.key[wave][j0 + lane] : 0u, valid ? sh.hist.seg.idx[wave][j0 + lane] : -1);
+                        }
+                    };
+                    for (int shift = 24; shift >= 0; shift -= 8) {
+                        if (threadIdx.x < 256) sh.bin_mass[threadIdx.x] = 0ull;
+                        __syncthreads();
+                        each([&](uint32_t key, int i) {
+                            if (i >= 0 && (key & mask) == prefix) {
+                                const uint32_t w = fixed_weight(key_value(key), l_max, inv_t, min_w);
+                                if (w) atomicAdd(&sh.bin_mass[(key >> shift) & 0xffu], (mass_t)w);
+                            }
+                        });
+                        __syncthreads();
+                        if (threadIdx.x == 0) {
+                            mass_t run = above;
+                            int bin = 255;
+                            for (; bin > 0; --bin) {
+                                if (run + sh.bin_mass[bin] >= cutoff) break;
+                                run += sh.bin_mass[bin];
+                            }
+                            sh.prefix = prefix | ((uint32_t)bin << shift);
+                            sh.above = run;
+                        }
+                        __syncthreads();
+                        prefix = sh.prefix;
+                        above = sh.above;
+                        mask |= 0xffu << shift;
+                    }
+                    tau = prefix;
+                    w_tau = (mass_t)fixed_weight(key_value(tau), l_max, inv_t, min_w);
+                    n_ties = w_tau ? (int)min((mass_t)V, (cutoff - above + w_tau - 1ull) / w_tau) : 0;
+                    total = above + (mass_t)n_ties * w_tau;
+                    mass_t target = (mass_t)((double)u * (double)total);
+                    if (target >= total) target = total - 1ull;
+                    // the kept weights by wave, then the wave in which they pass the target, then the element
+                    mass_t kept = 0ull;
+                    int ties = 0;
+                    each([&](uint32_t key, int i) {
+                        if (i >= 0 && key > tau) kept += fixed_weight(key_value(key), l_max, inv_t, min_w);
+                        ties += i >= 0 && key == tau;
+                    });
+                    kept = wave_sum(kept);
+                    ties = wave_sum(ties);
+                    if (lane == 0) { sh.wave_mass[wave] = kept; sh.wave_ties[wave] = ties; }
+                    if (threadIdx.x == 0) sh.result = -1;
+                    __syncthreads();
+                    mass_t before = 0ull;
+                    int ties_before = 0;
+                    for (int w = 0; w < wave; ++w) {
+                        before += sh.wave_mass[w] + (mass_t)max(0, min(sh.wave_ties[w], n_ties - ties_before)) * w_tau;
+                        ties_before += sh.wave_ties[w];
+                    }
+                    const mass_t here = kept + (mass_t)max(0, min(ties, n_ties - ties_before)) * w_tau;
+                    if (target >= before && target < before + here) {        // one wave at most
+                        mass_t run = before;
+                        int rank = ties_before;
+                        bool found = false;
+                        each([&](uint32_t key, int i) {
+                            const bool tie = i >= 0 && key == tau;
+                            bool keep = i >= 0 && key > tau;
+                            const int at = rank + lanes_before(tie);
+                            if (tie) keep = at < n_ties;
+                            rank += __popcll(__ballot(tie));
+                            const mass_t w = keep ? (mass_t)fixed_weight(key_value(key), l_max, inv_t, min_w) : 0ull;
+                            mass_t scan = w;
+#pragma unroll
+                            for (int off = 1; off < WAVE; off <<= 1) { const mass_t o = __shfl_up(scan, off, WAVE); if (lane >= off) scan += o; }
+                            const unsigned long long hit = __ballot(w > 0ull && target < run + scan);
+                            if (!found && hit) {
+                                found = true;
+                                if (lane == __ffsll((long long)hit) - 1) sh.result = i;
+                            }
+                            run += __shfl(scan, WAVE - 1, WAVE);
+                        });
+                    }
+                    __syncthreads();
+                    if (threadIdx.x == 0) out[blockIdx.x] = sh.result >= 0 ? sh.result : best.i;
+                    return;
+                }
+            }
             // The top byte of a float's key is its sign and most of its exponent: most of a row shares one or two
             // values of it, and as many additions to one histogram bin take as many turns.  Usually the elements
             // that share the maximum's top byte already weigh as much as the cutoff: then that byte is the answer.
