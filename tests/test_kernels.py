@@ -501,6 +501,15 @@ def test_draws_walk_the_kept_set_and_follow_u(ops):
         assert ref[tok] > 0
         lo = cdf[tok] - ref[tok]
         assert lo - 1e-4 <= u <= cdf[tok] + 1e-4, (u, tok)
+    # many ties at the threshold (logits on a grid of halves): the draw, which searches among a few elements set
+    # aside, lands where the kernel's own probabilities (written from the whole row) put u
+    tied = torch.round(rand(1, 5003, seed=6, scale=2.0, dtype=F32) * 2) / 2
+    for top_p, t in ((0.8, 1.0), (0.35, 0.7), (0.97, 1.3)):
+        probs = ops.sample(tied.to(DEV), torch.zeros(1).to(DEV), t, 0, top_p, 0.0, want_probs=True)[1].cpu().double()[0]
+        cdf = torch.cumsum(probs, 0)
+        for u in (0.0, 0.123, 0.5, 0.77, 0.9999):
+            tok = ops.sample(tied.to(DEV), torch.tensor([u], dtype=F32).to(DEV), t, 0, top_p, 0.0).item()
+            assert float(probs[tok]) > 0 and float(cdf[tok] - probs[tok]) - 1e-4 <= u <= float(cdf[tok]) + 1e-4, (top_p, t, u, tok)
     # with top-k the walk is over the sorted candidates, as the reference's (engine/sampler.cpp:180-187)
     for u in (0.0, 0.2, 0.55, 0.93, 0.9999):
         tok = ops.sample(lg.to(DEV), torch.tensor([u], dtype=F32).to(DEV), 0.9, 40, 0.95, 0.0).item()
