@@ -381,20 +381,29 @@ __device__ inline PageSources page_sources() {
     }
     return src;
 }
+// The load itself is written out in assembly.  Through the compiler's builtin every later read of LDS, of either
+// buffer, would first wait for all such loads, and the page on its way would never overlap the arithmetic on the
+// page at hand.  This way the compiler does not know of the loads: lds_loads_done() waits for them before the
+// barrier after which their buffer is read (a wait of the compiler's own for other loads can only wait for these
+// too, since loads come back in order).
+__device__ __forceinline__ void load_16_bytes_a_lane_into_lds(const void* from, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(from), "s"(lds_base) : "m0");
+}
+// s_waitcnt vmcnt(0), as an instruction that the compiler knows (it then also knows that its own loads are done)
+__device__ __forceinline__ void lds_loads_done() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+__device__ __forceinline__ uint32_t lds_address(const bf16_t* p) {       // the same in every lane of a wave
+    return __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)p);
+}
 __device__ inline void page_into_lds(const bf16_t* __restrict__ kp, const bf16_t* __restrict__ vp, const PageSources& src,
                                      bf16_t* k_lds, bf16_t* v_lds) {
-    typedef const __attribute__((address_space(1))) void* global_ptr;
-    typedef __attribute__((address_space(3))) void* lds_ptr;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
     constexpr int KB = 1024 / sizeof(bf16_t);                    // elements of 1 KB
 #pragma unroll
     for (int i = 0; i < PF_LOADS; ++i)
-        __builtin_amdgcn_global_load_lds((global_ptr)(reinterpret_cast<const char*>(kp) + src.k[i]),
-                                         (lds_ptr)(k_lds + (i * PF_WAVES + wave) * KB), 16, 0, 0);
+        load_16_bytes_a_lane_into_lds(reinterpret_cast<const char*>(kp) + src.k[i], lds_address(k_lds + (i * PF_WAVES + wave) * KB));
 #pragma unroll
     for (int i = 0; i < PF_LOADS; ++i)
-        __builtin_amdgcn_global_load_lds((global_ptr)(reinterpret_cast<const char*>(vp) + src.v[i]),
-                                         (lds_ptr)(v_lds + (i * PF_WAVES + wave) * KB), 16, 0, 0);
+        load_16_bytes_a_lane_into_lds(reinterpret_cast<const char*>(vp) + src.v[i], lds_address(v_lds + (i * PF_WAVES + wave) * KB));
 }
 
 struct Unit {                 // one (head, 16 query positions): the wave's share of it
@@ -628,7 +637,9 @@ __global__ __launch_bounds__(PF_THREADS) PF_WAVES_PER_SIMD void attention_prefil
         return __all(inside);
     };
     if constexpr (!PF_SHARE) {
-        if constexpr (!PF_DMA) {
+        if constexpr (PF_DMA) {
+            lds_loads_done();
+        } else {
             stage_keys(pf, k_lds);
             stage_values(pf, v_lds);
         }
@@ -659,7 +670,8 @@ __global__ __launch_bounds__(PF_THREADS) PF_WAVES_PER_SIMD void attention_prefil
                     stage_values(pf, v_lds + (buf ^ 1) * V_TILE);
                 }
             }
-            __syncthreads();                                    // (waits for the reads into LDS, too)
+            if constexpr (PF_DMA) lds_loads_done();
+            __syncthreads();
         }
     } else {
         for (int p = p_lo; p <= p_hi; ++p) {
