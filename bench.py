@@ -26,11 +26,10 @@ if ROOT not in sys.path:
 PEAK_HBM_GBS = 8000.0
 PEAK_FLOPS = {"bf16": 2.5e15, "fp16": 2.5e15, "fp8": 5.0e15, "fp32": 157.3e12}
 
-# BASELINE.json configs[2]: Qwen3-8B sizes
-QWEN3_8B = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_size=151936, hidden_size=4096,
-                num_hidden_layers=36, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
-                intermediate_size=12288, rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=False,
-                max_position_embeddings=40960)
+# BASELINE.json configs[2]: Qwen3-8B sizes, kept as data beside the configuration code
+from palm_infra_amd.config import preset_dict  # noqa: E402
+
+QWEN3_8B = preset_dict("qwen3-8b")
 CONTEXT = 2048          # tokens every sequence holds when decoding starts
 PREFILL_TOKENS = 2048
 BATCH = 8

@@ -56,3 +56,31 @@ def config_from_dir(model_dir):
     if not path.is_file():
         raise FileNotFoundError(f"no config.json in {model_dir}")
     return config_from_dict(json.loads(path.read_text()))
+
+
+# ---- named sizes -------------------------------------------------------------------------------------
+# config.json files kept as data beside this module: the sizes that measurements and examples name
+# (the reference names models by package file; its benchmark protocol is examples/bench.cpp:564-590).
+PRESET_DIR = Path(__file__).resolve().parent / "presets"
+
+
+def preset_names() -> list[str]:
+    return sorted(p.stem for p in PRESET_DIR.glob("*.json"))
+
+
+def preset_dict(name: str) -> dict:
+    """The config.json of a named size, as a dict."""
+    path = PRESET_DIR / f"{name}.json"
+    if not path.is_file():
+        raise ConfigError(f"unknown size {name!r}; known: {', '.join(preset_names())}")
+    return json.loads(path.read_text())
+
+
+def config_source(name_or_path) -> dict:
+    """A config.json given as a path to the file (or to its folder), or as a named size."""
+    path = Path(name_or_path)
+    if path.is_dir():
+        path = path / "config.json"
+    if path.is_file():
+        return json.loads(path.read_text())
+    return preset_dict(str(name_or_path))

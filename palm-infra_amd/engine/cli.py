@@ -4,7 +4,8 @@ tokens, ``bench`` times a run and prints ``key=value`` lines.
 Options keep the reference's names and meanings where it has them (examples/cli_common.cpp:44-347):
 ``--prompt``, ``--prompt-file``, ``--prompt-tokens``, ``--max-new-tokens``, ``--n-ctx``, ``--warmup``,
 ``--temperature``, ``--top-k``, ``--top-p``, ``--min-p``, ``--repeat-penalty``, ``--repeat-last-n``,
-``--presence-penalty``, ``--frequency-penalty``, ``--seed``, ``--output kv|human``.  ``--package`` names a
+``--presence-penalty``, ``--frequency-penalty``, ``--seed``, ``--output kv|human``, ``--profile``,
+``--trace``.  ``--package`` names a
 model folder here (``--model`` is the same): there is no packaging step.  New: ``--dtype``, ``--batch``,
 ``--prompt-ids``, ``--random-config`` (random weights from a config.json or a named size).  Options of
 the reference that select a backend, offload, vision or speculation have no meaning here and are
@@ -17,18 +18,19 @@ as in the reference (examples/bench.cpp:564-583).
 from __future__ import annotations
 
 import argparse
-import json
 import sys
 import time
 from pathlib import Path
 
+from ..config import config_source
 from ..sampling import SamplingError, SamplingParams
 
 
 def build_parser(prog: str, bench: bool) -> argparse.ArgumentParser:
     ap = argparse.ArgumentParser(prog=prog, description=__doc__.split("\n\n")[0])
     ap.add_argument("--package", "--model", dest="model", help="model folder: config.json + safetensors")
-    ap.add_argument("--random-config", help="instead of --package: a config.json to fill with random weights")
+    ap.add_argument("--random-config", "--random", dest="random_config",
+                    help="instead of --package: a config.json, or a named size, to fill with random weights")
     ap.add_argument("--prompt", action="append", default=[], help="prompt text (needs tokenizer.json); may repeat")
     ap.add_argument("--prompt-file", help="read prompt text from a file")
     ap.add_argument("--prompt-ids", action="append", default=[], help="prompt as comma-separated token ids; may repeat")
@@ -49,6 +51,9 @@ def build_parser(prog: str, bench: bool) -> argparse.ArgumentParser:
     ap.add_argument("--frequency-penalty", type=float, default=0.0)
     ap.add_argument("--seed", type=int, default=42)
     ap.add_argument("--output", default="kv", choices=["kv", "human"], help="bench output format")
+    ap.add_argument("--profile", action="store_true", help="print time per kernel entry point, prefill and decode apart "
+                                                            "(steps then launch kernel by kernel, without HIP graphs)")
+    ap.add_argument("--trace", metavar="PATH.json", help="write the steps and kernel launches as a Chrome trace")
     return ap
 
 
@@ -98,8 +103,7 @@ def make_engine(args):
     if args.model:
         return Engine.from_dir(args.model, dtype=args.dtype, max_tokens=args.n_ctx)
     if args.random_config:
-        raw = json.loads(Path(args.random_config).read_text())
-        return Engine.from_config(raw, seed=args.seed, dtype=args.dtype, max_tokens=args.n_ctx)
+        return Engine.from_config(config_source(args.random_config), seed=args.seed, dtype=args.dtype, max_tokens=args.n_ctx)
     raise SystemExit("--package <model folder> (or --random-config <config.json>) is required")
 
 
@@ -139,6 +143,9 @@ def run(argv, bench: bool) -> int:
     if args.max_new_tokens < 1:
         print(f"{ap.prog}: max_new_tokens must be >= 1", file=sys.stderr)
         return 1
+    if args.trace is not None and not args.trace:
+        print(f"{ap.prog}: --trace path must not be empty", file=sys.stderr)
+        return 1
     t0 = time.perf_counter()
     engine = make_engine(args)
     load_ms = (time.perf_counter() - t0) * 1000.0
@@ -153,6 +160,11 @@ def run(argv, bench: bool) -> int:
     if bench:
         for _ in range(max(0, args.warmup)):
             engine.generate(prompts, sampling, args.max_new_tokens, ignore_eos=no_stop, max_batch=max(1, args.batch))
+    recorder = None
+    if args.profile or args.trace:
+        # after the warm-up, so that what is timed has loaded its libraries and the tables show the timed run alone
+        from ..kernels.profile import KernelProfile
+        recorder = KernelProfile().install()
     t1 = time.perf_counter()
 
     def stream(i, tok):
@@ -163,9 +175,15 @@ def run(argv, bench: bool) -> int:
     results, metrics = engine.generate(prompts, sampling, args.max_new_tokens, ignore_eos=no_stop,
                                        max_batch=max(1, args.batch), on_token=stream)
     total_ms = (time.perf_counter() - t1) * 1000.0
+    if recorder is not None:
+        recorder.remove()
+        if args.trace:
+            recorder.write_chrome_trace(args.trace)
     if bench:
         (print_human if args.output == "human" else print_kv)(load_ms, metrics, total_ms, len(prompts),
                                                                [r.finish_reason for r in results])
+        if args.profile:
+            print(recorder.format())
         return 0
     if len(prompts) == 1:
         print()
@@ -173,6 +191,8 @@ def run(argv, bench: bool) -> int:
         for i, r in enumerate(results):
             text = tokenizer.decode(r.token_ids) if tokenizer else " ".join(map(str, r.token_ids))
             print(f"[{i}] {text}")
+    if args.profile:
+        print(recorder.format(), file=sys.stderr)
     print(f"ttft {metrics.ttft_ms:.1f} ms | tpot {metrics.tpot_ms:.2f} ms | prefill {metrics.prefill_tps:.1f} tok/s | "
           f"decode {metrics.decode_tps:.1f} tok/s | tokens {metrics.generated_tokens}", file=sys.stderr)
     return 0

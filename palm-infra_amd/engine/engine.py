@@ -16,6 +16,7 @@ import torch
 
 from ..cache import ModelCache
 from ..config import config_from_dict, config_from_dir
+from ..kernels import profile
 from ..parts import make_context
 from ..weights import ModelFiles, load_weights, random_weights
 from .model import DecoderModel
@@ -170,7 +171,7 @@ class Engine:
 
     def _graph_serves(self, entries) -> bool:
         return (self.graphs_enabled and self.model.capturable and len(entries) <= self.GRAPH_MAX_BATCH
-                and all(len(e.tokens) == 1 for e in entries))
+                and all(len(e.tokens) == 1 for e in entries) and profile.active() is None)
 
     def _run_decode_graph(self, entries) -> torch.Tensor:
         from ..parts import StepContext
@@ -219,8 +220,18 @@ class Engine:
         return logits[torch.tensor(wanted, dtype=torch.long, device=self.device)] if wanted else logits[:0]
 
     def _run(self, entries) -> torch.Tensor:
+        recorder = profile.active()
+        if recorder is not None:
+            # a step with a recorder installed launches kernel by kernel (no graph) and is filed as a whole
+            single = all(len(e.tokens) == 1 and self.cache.lengths[e.slot] > 0 for e in entries)
+            label = f"{'decode' if single else 'prefill'} {len(entries)} x {max(len(e.tokens) for e in entries)}"
+            with recorder.step("decode" if single else "prefill", label):
+                return self._run_plain(entries)
         if self._graph_serves(entries):
             return self._run_decode_graph(entries)
+        return self._run_plain(entries)
+
+    def _run_plain(self, entries) -> torch.Tensor:
         cache = self.cache
         growth = [(e.slot, len(e.tokens)) for e in entries]
         cache.reserve(growth)

@@ -24,6 +24,8 @@ import time
 from concurrent.futures import ThreadPoolExecutor, wait
 from pathlib import Path
 
+from . import profile
+
 CSRC = Path(__file__).resolve().parent.parent / "csrc"
 ARCH = "gfx950"
 FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-fno-gpu-rdc",
@@ -194,6 +196,7 @@ def loaded_paths() -> list[str]:
 
 def call(lib: ctypes.CDLL, fn_name: str, *args) -> None:
     fn = getattr(lib, fn_name)
-    rc = fn(*args)
+    recorder = profile.active()
+    rc = fn(*args) if recorder is None else recorder.around(fn_name, lambda: fn(*args))
     if rc != 0:
         raise KernelError(f"{fn_name}: {lib.palm_last_error().decode(errors='replace')}")

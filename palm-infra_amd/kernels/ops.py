@@ -11,7 +11,7 @@ from ctypes import c_float, c_int, c_longlong, c_void_p
 
 import torch
 
-from . import library
+from . import library, profile
 from .library import KernelError
 
 F32, BF16 = torch.float32, torch.bfloat16
@@ -315,6 +315,9 @@ def linear_library(a: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     _need(a.dtype == BF16 and w.dtype == BF16, "linear_library serves bfloat16 operands only")
     _need(a.dim() == 2 and w.dim() == 2 and a.shape[1] == w.shape[1],
           f"linear: a {tuple(a.shape)} and w {tuple(w.shape)} do not share the inner size")
+    recorder = profile.active()
+    if recorder is not None:
+        return recorder.around("library_matmul", lambda: torch.matmul(a, w.t()))
     return torch.matmul(a, w.t())
 
 

@@ -14,7 +14,7 @@ from pathlib import Path
 
 import torch
 
-from ..config.registry import config_from_dict
+from ..config.registry import config_from_dict, config_source
 from .safetensors_io import write_safetensors
 
 _STORE = {"bfloat16": torch.bfloat16, "float32": torch.float32, "float16": torch.float16}
@@ -61,12 +61,12 @@ def main(argv=None) -> int:
     import argparse
     ap = argparse.ArgumentParser(prog="palm_random_model",
                                  description="Write a model folder (config.json, model.safetensors) with random weights.")
-    ap.add_argument("--config", required=True, help="a config.json of a registered architecture")
+    ap.add_argument("--config", required=True, help="a config.json of a registered architecture, or a named size")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--out", required=True, help="folder to write")
     ap.add_argument("--dtype", default="bfloat16", choices=sorted(_STORE), help="how the tensors are stored")
     args = ap.parse_args(argv)
-    raw = json.loads(Path(args.config).read_text())
+    raw = config_source(args.config)
     out = write_random_model(raw, args.seed, args.out, args.dtype)
     print(out)
     return 0

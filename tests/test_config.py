@@ -124,3 +124,21 @@ def test_run_order_is_data_and_is_checked():
         dataclasses.replace(spec, order=(LayerCall(5),))
     with pytest.raises(ValueError, match="holds none"):
         dataclasses.replace(spec, order=(LayerCall(0), LayerCall(1, cache_of=0), LayerCall(0, cache_of=1)))
+
+
+def test_named_sizes_are_data_and_load():
+    from palm_infra_amd.config import ConfigError, config_source, preset_dict, preset_names
+    assert {"tiny-a", "tiny-b", "qwen3-8b", "qwen3-14b", "qwen3-32b"} <= set(preset_names())
+    for name in preset_names():
+        cfg = config_from_dict(preset_dict(name))
+        assert cfg.spec().vocab_size == preset_dict(name)["vocab_size"]
+    assert config_source("tiny-b")["head_dim"] == 32
+    with pytest.raises(ConfigError, match="unknown size 'qwen9'.*tiny-a"):
+        config_source("qwen9")
+
+
+def test_config_source_reads_a_file_or_a_folder(tmp_path):
+    import json
+    from palm_infra_amd.config import config_source
+    (tmp_path / "config.json").write_text(json.dumps(tiny.CONFIGS["A"]))
+    assert config_source(tmp_path) == tiny.CONFIGS["A"] == config_source(tmp_path / "config.json")

@@ -131,3 +131,32 @@ def test_command_line_generates_and_reports(model_dirs):
     bad = subprocess.run([str(ROOT / "bin" / "palm_chat"), "--package", str(model_dirs["A"]["float32"]), "--temperature", "3"],
                          capture_output=True, text=True, timeout=120)
     assert bad.returncode == 1 and "temperature must be between 0 and 2" in bad.stderr
+
+
+def test_command_line_profile_and_trace(tmp_path):
+    """``--profile`` prints a table per phase whose launches are the timed run's; ``--trace`` writes them as a
+    Chrome trace; the model is a named size with random weights."""
+    import json
+    trace = tmp_path / "t.json"
+    b = subprocess.run([str(ROOT / "bin" / "palm_bench"), "--random", "tiny-b", "--prompt-tokens", "20", "--batch", "2",
+                        "--max-new-tokens", "4", "--temperature", "0", "--n-ctx", "512", "--warmup", "1", "--profile",
+                        "--trace", str(trace)], capture_output=True, text=True, timeout=120)
+    assert b.returncode == 0, b.stderr[-2000:]
+    out = b.stdout
+    assert "[prefill_profile]" in out and "[decode_profile]" in out and "generated_tokens=8" in out
+    decode = out.split("[decode_profile]")[1]
+    rows = {line.split()[0]: int(line.split()[1]) for line in decode.strip().splitlines()[2:]}
+    # tiny-b has three layers; three decode steps of two sequences follow the prompts' step
+    assert rows["palm_attention_decode"] == 3 * 3 and rows["palm_argmax"] == 3
+    events = json.loads(trace.read_text())["traceEvents"]
+    steps = [e for e in events if e.get("ph") == "X" and e["tid"] == 0]
+    assert [e["cat"] for e in steps] == ["prefill", "decode", "decode", "decode"]
+    kernels = [e for e in events if e.get("ph") == "X" and e["tid"] == 1]
+    assert all(e["dur"] >= 0 for e in kernels) and sum(e["name"] == "palm_attention_decode" for e in kernels) == 9
+    # every launch of a step lies inside the step
+    first = steps[0]
+    inside = [e for e in kernels if first["ts"] <= e["ts"] and e["ts"] + e["dur"] <= first["ts"] + first["dur"] + 1.0]
+    assert len(inside) >= 3 * 4
+    empty = subprocess.run([str(ROOT / "bin" / "palm_bench"), "--random", "tiny-b", "--trace", ""], capture_output=True,
+                           text=True, timeout=120)
+    assert empty.returncode == 1 and "--trace path must not be empty" in empty.stderr
