@@ -7,7 +7,7 @@ Options keep the reference's names and meanings where it has them (examples/cli_
 ``--presence-penalty``, ``--frequency-penalty``, ``--seed``, ``--output kv|human``, ``--profile``,
 ``--trace``.  ``--package`` names a
 model folder here (``--model`` is the same): there is no packaging step.  New: ``--dtype``, ``--batch``,
-``--prompt-ids``, ``--random-config`` (random weights from a config.json or a named size).  Options of
+``--prompt-ids``, ``--prompt-lengths``, ``--random-config`` (random weights from a config.json or a named size).  Options of
 the reference that select a backend, offload, vision or speculation have no meaning here and are
 refused by the parser.
 
@@ -35,6 +35,8 @@ def build_parser(prog: str, bench: bool) -> argparse.ArgumentParser:
     ap.add_argument("--prompt-file", help="read prompt text from a file")
     ap.add_argument("--prompt-ids", action="append", default=[], help="prompt as comma-separated token ids; may repeat")
     ap.add_argument("--prompt-tokens", type=int, default=0, help="use N dummy tokens (no stop token)")
+    ap.add_argument("--prompt-lengths", metavar="LO:HI", help="like --prompt-tokens, the length of each of --batch prompts "
+                                                              "drawn uniformly from LO..HI (by --seed) and the ids at random")
     ap.add_argument("--batch", type=int, default=1, help="with --prompt-tokens: how many such prompts; else the most "
                                                           "requests in one batch")
     ap.add_argument("--max-new-tokens", type=int, default=2048)
@@ -81,6 +83,17 @@ def load_tokenizer(model_dir):
 
 def collect_prompts(args, tokenizer, vocab_size: int):
     """Returns (prompts as id lists, stopping disabled?)."""
+    if args.prompt_lengths:
+        import random
+        try:
+            lo, hi = (int(x) for x in args.prompt_lengths.split(":"))
+        except ValueError:
+            raise SystemExit("--prompt-lengths takes LO:HI, two whole numbers")
+        if not 1 <= lo <= hi:
+            raise SystemExit("--prompt-lengths needs 1 <= LO <= HI")
+        rng = random.Random(args.seed)
+        lengths = [rng.randint(lo, hi) for _ in range(max(1, args.batch))]
+        return [[rng.randrange(vocab_size) for _ in range(n)] for n in lengths], True
     if args.prompt_tokens > 0:
         # token 0 is always valid (examples/bench.cpp:564-567)
         return [[0] * args.prompt_tokens for _ in range(max(1, args.batch))], True
