@@ -104,14 +104,14 @@ class ModelCache:
     reads another entry's cache: ``shares[i]`` is that entry's index)."""
 
     def __init__(self, needs: list[list], shares: list[int | None], max_tokens: int, max_seqs: int | None,
-                 max_positions: int, dtype: torch.dtype, device):
+                 max_positions: int | None, dtype: torch.dtype, device):
         if max_tokens <= 0:
             raise ValueError(f"max_tokens = {max_tokens} must be positive")
         self.device, self.dtype = device, dtype
         n_pages = pages_for(max_tokens)
         self.max_seqs = int(max_seqs) if max_seqs else min(n_pages, 1024)
         self.max_tokens = n_pages * PAGE_TOKENS
-        self.max_seq_tokens = min(max_positions, self.max_tokens)
+        self.max_seq_tokens = min(max_positions, self.max_tokens) if max_positions else self.max_tokens
         max_pages_per_slot = pages_for(self.max_seq_tokens)
         self.pad_slot = self.max_seqs
         self.slots = FreeList(self.max_seqs, "slot")

@@ -147,7 +147,9 @@ class Qwen3Config:
         head_ref = embed_ref if tied else tensor("lm_head.weight", (V, H), "matrix")
         return ModelSpec(
             architecture=self.architecture, vocab_size=V, hidden_size=H,
-            max_positions=self.max_position_embeddings,
+            # the reference never reads max_position_embeddings (models/qwen3.py:175-184): its limit is the cache's
+            # rows (engine/engine.cpp:969-976), and rotation angles are computed, not looked up
+            max_positions=None,
             embedding=PartSpec("embedding", "token_table", {"vocab_size": V, "hidden_size": H}, {"table": embed_ref}),
             layers=tuple(layers),
             order=tuple(LayerCall(i) for i in range(self.num_hidden_layers)),

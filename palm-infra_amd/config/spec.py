@@ -80,7 +80,9 @@ class ModelSpec:
     architecture: str
     vocab_size: int
     hidden_size: int
-    max_positions: int
+    # the longest sequence the model itself can take (a learned position table has a last row); None if only the
+    # cache bounds it, as with rotation, whose angles are computed from the position
+    max_positions: int | None
     embedding: PartSpec
     layers: tuple[PartSpec, ...]
     order: tuple[LayerCall, ...]

@@ -85,6 +85,7 @@ def test_a_step_that_does_not_fit_takes_nothing():
 def test_longest_sequence_is_bounded_by_positions_and_by_the_cache():
     assert _cache(max_tokens=64 * 12, max_positions=100).max_seq_tokens == 100
     assert _cache(max_tokens=64 * 2, max_positions=4096).max_seq_tokens == 128
+    assert _cache(max_tokens=64 * 5, max_positions=None).max_seq_tokens == 320      # a model without a limit of its own
     assert _cache(max_tokens=65).max_tokens == 128   # rounded up to whole pages
 
 

@@ -176,11 +176,25 @@ def test_a_refused_step_changes_nothing(model_dirs):
     eng.step([StepEntry(s, ids[:4], [])])
     for bad, err in (([StepEntry(s, [256], [0])], StepError), ([StepEntry(s, [1], [1])], StepError),
                      ([StepEntry(s, [], [])], StepError), ([StepEntry(s, [1], []), StepEntry(s, [2], [])], StepError),
-                     ([StepEntry(31, [1], [])], StepError), ([StepEntry(s, [1] * 200, [])], CacheFull), ([], StepError)):
+                     ([StepEntry(31, [1], [])], StepError), ([StepEntry(s, [1] * 2000, [])], CacheFull), ([], StepError)):
         with pytest.raises(err):
             eng.step(bad)
         assert eng.length(s) == 4
-    got = eng.step([StepEntry(s, ids[4:], list(range(6)))])           # max_position_embeddings is 128: 200 more do not fit
+    got = eng.step([StepEntry(s, ids[4:], list(range(6)))])           # the cache has 24 pages: 2,000 more do not fit
     tiny.assert_logits_close(got, reference(model_dirs, "A", "float32", ids)[4:], "float32", "after refused steps")
     eng.close(s)
     eng.cache.check()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_sequence_longer_than_max_position_embeddings(model_dirs, dtype):
+    """The reference never reads ``max_position_embeddings`` (models/qwen3.py:175-184); a sequence is bounded by
+    the cache alone.  Configuration A names 128 positions; 150 tokens run, the last 10 one by one."""
+    from palm_infra_amd.engine import StepEntry
+    eng = engine_for(model_dirs, "A", dtype)
+    ids = tiny.prompts("A", [150], seed=21)[0]
+    s = eng.open()
+    got = [eng.step([StepEntry(s, ids[:140], list(range(140)))])]
+    got += [eng.step([StepEntry(s, [t], [0])]) for t in ids[140:]]
+    eng.close(s)
+    tiny.assert_logits_close(torch.cat(got), reference(model_dirs, "A", dtype, ids), dtype, "150 tokens with 128 positions named")
