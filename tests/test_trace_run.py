@@ -87,16 +87,23 @@ def schedule_steps(reqs):
     return steps, checks
 
 
-@pytest.mark.parametrize("name,dtype", [("A", "float32"), ("A", "bfloat16"), ("B", "float32"), ("B", "bfloat16")])
-def test_replay_schedules(model_dirs, tmp_path, name, dtype):
+# the last three: a folder stored in one precision and run in the other (a tensor stored in 32-bit stays so in
+# the bfloat16 mode; bfloat16 and float16 widen exactly for the float32 mode; float16 is re-rounded for bfloat16)
+@pytest.mark.parametrize("name,dtype,store", [("A", "float32", None), ("A", "bfloat16", None), ("B", "float32", None),
+                                              ("B", "bfloat16", None), ("B", "bfloat16", "float32"),
+                                              ("A", "float32", "bfloat16"), ("B", "float32", "float16"),
+                                              ("A", "bfloat16", "float16")])
+def test_replay_schedules(model_dirs, tmp_path, name, dtype, store):
     lengths = {"A": [5, 17, 9, 70, 40, 33], "B": [1, 31, 12, 64, 100, 45]}[name]
     reqs = tiny.prompts(name, lengths, seed=8)
     steps, checks = schedule_steps(reqs)
     # the most that is live at once: the second batch, each request rounded up to 64
     max_tokens = max(sum(-(-len(reqs[i]) // 64) * 64 for i in m) for m in ([0, 1, 2], [3, 4, 5, 0]))
     out = tmp_path / "out"
-    run_trace(model_dirs[name][dtype], dtype, steps, out, max_tokens)
-    cfg, w = P.read_model(model_dirs[name][dtype])
+    store = store or dtype
+    model_dir = model_dirs[name][store] if store in model_dirs[name] else tiny.write_model(name, tmp_path / "model", store)
+    run_trace(model_dir, dtype, steps, out, max_tokens)
+    cfg, w = P.read_model(model_dir)
     V = cfg["vocab_size"]
     refs = [P.logits(cfg, w, r) for r in reqs]
     files = {}

@@ -45,7 +45,7 @@ def sharpened_tensors(name: str, store: str) -> dict[str, torch.Tensor]:
             t = t * 4.0
         elif k.endswith("q_norm.weight"):
             t = t * 4.0
-        out[k] = t.to(torch.bfloat16 if store == "bfloat16" else torch.float32)
+        out[k] = t.to({"bfloat16": torch.bfloat16, "float16": torch.float16, "float32": torch.float32}[store])
     return out
 
 
