@@ -52,11 +52,15 @@ class Qwen3Config:
         eos = raw.get("eos_token_id")
         eos_ids = () if eos is None else tuple(int(e) for e in (eos if isinstance(eos, (list, tuple)) else [eos]))
         tie = raw.get("tie_word_embeddings")
+        # newer checkpoints keep the rotation's base in a ``rope_parameters`` table; the top-level key, which the
+        # reference reads (models/qwen3.py:179), comes first
+        nested = raw.get("rope_parameters") if isinstance(raw.get("rope_parameters"), dict) else {}
+        theta = raw.get("rope_theta", nested.get("rope_theta", 1000000.0))
         cfg = cls(
             vocab_size=_need(raw, "vocab_size"), hidden_size=hidden,
             num_hidden_layers=_need(raw, "num_hidden_layers"), num_attention_heads=nh,
             num_key_value_heads=nkv, head_dim=hd, intermediate_size=_need(raw, "intermediate_size"),
-            rms_norm_eps=float(raw.get("rms_norm_eps", 1e-6)), rope_theta=float(raw.get("rope_theta", 1000000.0)),
+            rms_norm_eps=float(raw.get("rms_norm_eps", 1e-6)), rope_theta=float(theta),
             max_position_embeddings=int(raw.get("max_position_embeddings", 32768)),
             tie_word_embeddings=None if tie is None else bool(tie), eos_token_ids=eos_ids,
         )
@@ -69,6 +73,8 @@ class Qwen3Config:
                               f"(use_sliding_window=true, sliding_window={raw['sliding_window']})")
         if raw.get("rope_scaling") not in (None, {}):
             raise ConfigError(f"config.json: rope_scaling={raw['rope_scaling']!r} is not supported (plain rotation only)")
+        if nested.get("rope_type", nested.get("type", "default")) not in (None, "default"):
+            raise ConfigError(f"config.json: rope_parameters={nested!r} is not supported (plain rotation only)")
         if raw.get("hidden_act", "silu") != "silu":
             raise ConfigError(f"config.json: hidden_act={raw['hidden_act']!r}; the feed-forward of this architecture uses silu")
         return cfg

@@ -142,3 +142,12 @@ def test_config_source_reads_a_file_or_a_folder(tmp_path):
     from palm_infra_amd.config import config_source
     (tmp_path / "config.json").write_text(json.dumps(tiny.CONFIGS["A"]))
     assert config_source(tmp_path) == tiny.CONFIGS["A"] == config_source(tmp_path / "config.json")
+
+
+def test_rotation_base_in_a_rope_parameters_table():
+    raw = {k: v for k, v in tiny.CONFIGS["B"].items() if k != "rope_theta"}
+    assert config_from_dict(dict(raw, rope_parameters={"rope_type": "default", "rope_theta": 12345.0})).rope_theta == 12345.0
+    assert config_from_dict(dict(raw, rope_theta=7.0, rope_parameters={"rope_theta": 12345.0})).rope_theta == 7.0
+    assert config_from_dict(raw).rope_theta == 1000000.0
+    with pytest.raises(ConfigError, match="plain rotation only"):
+        config_from_dict(dict(raw, rope_parameters={"rope_type": "yarn", "rope_theta": 1e6, "factor": 4.0}))
