@@ -78,3 +78,40 @@ def test_a_model_with_a_part_that_plans_on_the_host_is_not_recorded(model_dirs):
                          {("toy.w_in",): torch.zeros(24, 64, device="cuda:0"), ("toy.w_out",): torch.zeros(64, 24, device="cuda:0")})
     eng = Engine(config, toy.toy_spec(base), w, torch.float32, max_tokens=256)
     assert not eng.model.capturable
+
+
+@pytest.mark.parametrize("name", ["B", "C"])
+def test_replays_of_steps_with_17_to_64_sequences(model_dirs, name):
+    """From 17 sequences on a tiny model's products go to the BLAS library (its matrices have too few rows for
+    the kernel that shares the activations through LDS), so these recorded steps hold library calls: every
+    replay is checked against plain launches, with other work and synchronisations between the replays."""
+    from palm_infra_amd.engine import Engine, StepEntry
+    dtype = "bfloat16"
+    g = Engine.from_dir(model_dirs[name][dtype], dtype=dtype, max_tokens=64 * 64, graphs=True)
+    e = Engine.from_dir(model_dirs[name][dtype], dtype=dtype, max_tokens=64 * 64, graphs=False)
+    n_req = 40
+    reqs = tiny.prompts(name, [2 + (5 * i) % 23 for i in range(n_req)], seed=40)
+    decoded = tiny.prompts(name, [30] * n_req, seed=41)
+    sg = [g.open() for _ in reqs]
+    se = [e.open() for _ in reqs]
+    g.step([StepEntry(s, r, []) for s, r in zip(sg, reqs)])
+    e.step([StepEntry(s, r, []) for s, r in zip(se, reqs)])
+    live = list(range(n_req))
+    for t in range(30):
+        if t in (6, 12, 18, 24):                                    # 40 -> 33 -> 26 -> 19 -> 12 sequences
+            for _ in range(7):
+                gone = live.pop((3 * t) % len(live))
+                g.close(sg[gone]); e.close(se[gone])
+        a = g.step([StepEntry(sg[i], [decoded[i][t]], [0]) for i in live])
+        b = e.step([StepEntry(se[i], [decoded[i][t]], [0]) for i in live])
+        if t % 5 == 2:
+            torch.cuda.synchronize()
+            extra = g.open()
+            g.step([StepEntry(extra, reqs[3], [0])])
+            g.close(extra)
+        tiny.assert_logits_close(a, b.double().cpu(), dtype, f"{name} {len(live)} sequences, step {t}")
+        assert float((a - b).abs().max()) < 0.05 * float(b.abs().max()), (len(live), t)
+    for i in live:
+        g.close(sg[i]); e.close(se[i])
+    g.cache.check(); e.cache.check()
+    assert sum(st["graph"] is not None for st in g._decode_graphs.values()) >= 4
