@@ -55,7 +55,20 @@ def config_from_dir(model_dir):
     path = Path(model_dir) / "config.json"
     if not path.is_file():
         raise FileNotFoundError(f"no config.json in {model_dir}")
-    return config_from_dict(json.loads(path.read_text()))
+    raw = json.loads(path.read_text())
+    # a checkpoint's generation_config.json may name more stop tokens than config.json (a chat model's end-of-turn
+    # token beside the end-of-text one); generation stops at any of them
+    extra = Path(model_dir) / "generation_config.json"
+    if extra.is_file():
+        more = json.loads(extra.read_text()).get("eos_token_id")
+        if more is not None:
+            ids = []
+            for group in (raw.get("eos_token_id"), more):
+                for t in ([] if group is None else group if isinstance(group, (list, tuple)) else [group]):
+                    if int(t) not in ids:
+                        ids.append(int(t))
+            raw = dict(raw, eos_token_id=ids)
+    return config_from_dict(raw)
 
 
 # ---- named sizes -------------------------------------------------------------------------------------

@@ -6,7 +6,7 @@ Options keep the reference's names and meanings where it has them (examples/cli_
 ``--temperature``, ``--top-k``, ``--top-p``, ``--min-p``, ``--repeat-penalty``, ``--repeat-last-n``,
 ``--presence-penalty``, ``--frequency-penalty``, ``--seed``, ``--output kv|human``, ``--profile``,
 ``--trace``.  ``--package`` names a
-model folder here (``--model`` is the same): there is no packaging step.  New: ``--dtype``, ``--batch``,
+model folder here (``--model`` is the same): there is no packaging step.  New: ``--dtype``, ``--batch``, ``--stop-token-ids``, ``--ignore-eos``,
 ``--prompt-ids``, ``--prompt-lengths``, ``--random-config`` (random weights from a config.json or a named size).  Options of
 the reference that select a backend, offload, vision or speculation have no meaning here and are
 refused by the parser.
@@ -40,6 +40,9 @@ def build_parser(prog: str, bench: bool) -> argparse.ArgumentParser:
     ap.add_argument("--batch", type=int, default=1, help="with --prompt-tokens: how many such prompts; else the most "
                                                           "requests in one batch")
     ap.add_argument("--max-new-tokens", type=int, default=2048)
+    ap.add_argument("--stop-token-ids", help="comma-separated token ids that end a sequence (default: the model's "
+                                             "eos_token_id of config.json and generation_config.json)")
+    ap.add_argument("--ignore-eos", action="store_true", help="never stop before --max-new-tokens")
     ap.add_argument("--n-ctx", type=int, default=16384, help="tokens the cache holds for all live sequences together")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--warmup", type=int, default=1, help="warm-up runs before the timed run (bench)")
@@ -165,14 +168,23 @@ def run(argv, bench: bool) -> int:
     tokenizer = load_tokenizer(args.model)
     prompts, no_stop = collect_prompts(args, tokenizer, engine.vocab_size)
 
+    no_stop = no_stop or args.ignore_eos
+    stop_ids = None
+    if args.stop_token_ids is not None:
+        try:
+            stop_ids = tuple(int(t) for t in args.stop_token_ids.replace(",", " ").split())
+        except ValueError:
+            print(f"{ap.prog}: --stop-token-ids takes comma-separated whole numbers", file=sys.stderr)
+            return 1
     if not bench and not prompts:
-        return repl(engine, sampling, tokenizer, args)
+        return repl(engine, sampling, tokenizer, args, stop_ids)
     if not prompts:
         prompts = [[0] * 16]
         no_stop = True
     if bench:
         for _ in range(max(0, args.warmup)):
-            engine.generate(prompts, sampling, args.max_new_tokens, ignore_eos=no_stop, max_batch=max(1, args.batch))
+            engine.generate(prompts, sampling, args.max_new_tokens, stop_token_ids=stop_ids, ignore_eos=no_stop,
+                            max_batch=max(1, args.batch))
     recorder = None
     if args.profile or args.trace:
         # after the warm-up, so that what is timed has loaded its libraries and the tables show the timed run alone
@@ -185,7 +197,7 @@ def run(argv, bench: bool) -> int:
             piece = tokenizer.decode([tok]) if tokenizer else f"{tok} "
             print(piece, end="", flush=True)
 
-    results, metrics = engine.generate(prompts, sampling, args.max_new_tokens, ignore_eos=no_stop,
+    results, metrics = engine.generate(prompts, sampling, args.max_new_tokens, stop_token_ids=stop_ids, ignore_eos=no_stop,
                                        max_batch=max(1, args.batch), on_token=stream)
     total_ms = (time.perf_counter() - t1) * 1000.0
     if recorder is not None:
@@ -211,7 +223,7 @@ def run(argv, bench: bool) -> int:
     return 0
 
 
-def repl(engine, sampling, tokenizer, args) -> int:
+def repl(engine, sampling, tokenizer, args, stop_ids=None) -> int:
     """Prompts from standard input, one a line (text with a tokenizer, else token ids); ``/quit`` ends,
     ``/reset`` is accepted for the reference's users: every line starts a fresh sequence here."""
     print("one prompt a line; /quit to end", file=sys.stderr)
@@ -226,7 +238,7 @@ def repl(engine, sampling, tokenizer, args) -> int:
         except ValueError:
             print("without a tokenizer a prompt is a list of token ids", file=sys.stderr)
             continue
-        results, _ = engine.generate([ids], sampling, args.max_new_tokens)
+        results, _ = engine.generate([ids], sampling, args.max_new_tokens, stop_token_ids=stop_ids, ignore_eos=args.ignore_eos)
         out = results[0].token_ids
         print(tokenizer.decode(out) if tokenizer else " ".join(map(str, out)), flush=True)
     return 0

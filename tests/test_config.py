@@ -151,3 +151,14 @@ def test_rotation_base_in_a_rope_parameters_table():
     assert config_from_dict(raw).rope_theta == 1000000.0
     with pytest.raises(ConfigError, match="plain rotation only"):
         config_from_dict(dict(raw, rope_parameters={"rope_type": "yarn", "rope_theta": 1e6, "factor": 4.0}))
+
+
+def test_stop_tokens_of_generation_config_join_those_of_config(tmp_path):
+    import json
+    (tmp_path / "config.json").write_text(json.dumps(dict(tiny.CONFIGS["A"], eos_token_id=7)))
+    assert config_from_dir(tmp_path).eos_token_ids == (7,)
+    (tmp_path / "generation_config.json").write_text(json.dumps({"eos_token_id": [9, 7], "temperature": 0.6}))
+    assert config_from_dir(tmp_path).eos_token_ids == (7, 9)
+    assert config_from_dir(tmp_path).spec().stop_token_ids == (7, 9)
+    (tmp_path / "generation_config.json").write_text(json.dumps({"top_k": 20}))
+    assert config_from_dir(tmp_path).eos_token_ids == (7,)

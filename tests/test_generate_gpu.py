@@ -128,6 +128,14 @@ def test_command_line_generates_and_reports(model_dirs):
     kv = dict(line.split("=", 1) for line in b.stdout.strip().splitlines())
     assert kv["prompt_tokens"] == "60" and kv["generated_tokens"] == "15" and kv["decode_tokens"] == "12" and kv["hit_eos"] == "0"
     assert float(kv["decode_tps"]) > 0 and float(kv["prefill_tps"]) > 0
+    # stop tokens given on the command line, and stopping switched off
+    free = P.greedy(cfg, w, prompt, 12)
+    common = [str(ROOT / "bin" / "palm_chat"), "--package", str(model_dirs["A"]["float32"]), "--dtype", "float32", "--prompt-ids",
+              ",".join(map(str, prompt)), "--max-new-tokens", "12", "--temperature", "0", "--n-ctx", "256"]
+    r = subprocess.run(common + ["--ignore-eos"], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0 and [int(t) for t in r.stdout.split()] == free, r.stderr[-2000:]
+    r = subprocess.run(common + ["--stop-token-ids", f"{free[4]},999"], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0 and [int(t) for t in r.stdout.split()] == free[:free.index(free[4]) + 1], r.stderr[-2000:]
     bad = subprocess.run([str(ROOT / "bin" / "palm_chat"), "--package", str(model_dirs["A"]["float32"]), "--temperature", "3"],
                          capture_output=True, text=True, timeout=120)
     assert bad.returncode == 1 and "temperature must be between 0 and 2" in bad.stderr
