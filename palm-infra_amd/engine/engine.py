@@ -255,14 +255,23 @@ class Engine:
 
     # ---- generation --------------------------------------------------------------------------
     def generate(self, prompts, sampling=None, max_new_tokens: int = 2048, stop_token_ids=None, ignore_eos: bool = False,
-                 max_batch: int = 64, on_token=None):
+                 max_batch: int = 64, on_token=None, **sampling_options):
         """Token ids in, token ids out: ``prompts`` is a list of lists of ids; returns (results, metrics),
-        the results in the order of the prompts.  ``stop_token_ids`` defaults to config.json's
-        ``eos_token_id``; ``ignore_eos`` switches stopping off, as the reference's benchmark does
-        (examples/bench.cpp:583)."""
+        the results in the order of the prompts.  ``sampling`` is a ``SamplingParams``; its fields may also be
+        given by name (``temperature=0.7, seed=1``) and then replace those of ``sampling`` or of the defaults.
+        ``stop_token_ids`` defaults to the model's ``eos_token_id``; ``ignore_eos`` switches stopping off, as
+        the reference's benchmark does (examples/bench.cpp:583)."""
+        import dataclasses
         from ..sampling import DeviceSampler, SamplingParams
         from .generate import generate
-        sampler = DeviceSampler(sampling or SamplingParams())
+        sampling = sampling or SamplingParams()
+        if sampling_options:
+            unknown = sorted(set(sampling_options) - {f.name for f in dataclasses.fields(SamplingParams)})
+            if unknown:
+                raise TypeError(f"generate() got unknown options {unknown}; sampling options are "
+                                f"{[f.name for f in dataclasses.fields(SamplingParams)]}")
+            sampling = dataclasses.replace(sampling, **sampling_options)
+        sampler = DeviceSampler(sampling)
         if ignore_eos:
             stop = ()
         else:

@@ -31,6 +31,11 @@ def test_greedy_generation_equals_the_plain_implementation(model_dirs, engine_a)
     assert metrics.prefill_tps > 0 and metrics.decode_tps > 0
     engine_a.cache.check()
     assert engine_a.cache.slots.held_count == 0
+    # sampling options by name: temperature 0 is the greedy choice whatever the other options say
+    named, _ = engine_a.generate(prompts, temperature=0.0, seed=3, max_new_tokens=8, ignore_eos=True)
+    assert [r.token_ids for r in named] == [r.token_ids for r in results]
+    with pytest.raises(TypeError, match="unknown options \\['temprature'\\]"):
+        engine_a.generate(prompts, temprature=0.0)
 
 
 def test_stop_tokens_end_sequences_early_and_batches_follow(model_dirs, engine_a):
