@@ -22,6 +22,7 @@ import sys
 import time
 from pathlib import Path
 
+from ..cache import CacheFull
 from ..config import config_source
 from ..sampling import SamplingError, SamplingParams
 
@@ -163,7 +164,12 @@ def run(argv, bench: bool) -> int:
         print(f"{ap.prog}: --trace path must not be empty", file=sys.stderr)
         return 1
     t0 = time.perf_counter()
-    engine = make_engine(args)
+    try:
+        engine = make_engine(args)
+    except (ValueError, FileNotFoundError, RuntimeError) as e:
+        # a config.json, a checkpoint or a build that cannot be used: the message says what and where
+        print(f"{ap.prog}: {type(e).__name__}: {e}", file=sys.stderr)
+        return 1
     load_ms = (time.perf_counter() - t0) * 1000.0
     tokenizer = load_tokenizer(args.model)
     prompts, no_stop = collect_prompts(args, tokenizer, engine.vocab_size)
@@ -181,6 +187,15 @@ def run(argv, bench: bool) -> int:
     if not prompts:
         prompts = [[0] * 16]
         no_stop = True
+    try:
+        return _generate_and_report(ap, args, engine, sampling, tokenizer, prompts, stop_ids, no_stop, load_ms, bench)
+    except (ValueError, CacheFull) as e:
+        # a prompt that does not fit the cache, a token outside the vocabulary
+        print(f"{ap.prog}: {type(e).__name__}: {e}", file=sys.stderr)
+        return 1
+
+
+def _generate_and_report(ap, args, engine, sampling, tokenizer, prompts, stop_ids, no_stop, load_ms, bench) -> int:
     if bench:
         for _ in range(max(0, args.warmup)):
             engine.generate(prompts, sampling, args.max_new_tokens, stop_token_ids=stop_ids, ignore_eos=no_stop,
@@ -197,13 +212,15 @@ def run(argv, bench: bool) -> int:
             piece = tokenizer.decode([tok]) if tokenizer else f"{tok} "
             print(piece, end="", flush=True)
 
-    results, metrics = engine.generate(prompts, sampling, args.max_new_tokens, stop_token_ids=stop_ids, ignore_eos=no_stop,
-                                       max_batch=max(1, args.batch), on_token=stream)
+    try:
+        results, metrics = engine.generate(prompts, sampling, args.max_new_tokens, stop_token_ids=stop_ids,
+                                           ignore_eos=no_stop, max_batch=max(1, args.batch), on_token=stream)
+    finally:
+        if recorder is not None:
+            recorder.remove()
     total_ms = (time.perf_counter() - t1) * 1000.0
-    if recorder is not None:
-        recorder.remove()
-        if args.trace:
-            recorder.write_chrome_trace(args.trace)
+    if args.trace:
+        recorder.write_chrome_trace(args.trace)
     if bench:
         (print_human if args.output == "human" else print_kv)(load_ms, metrics, total_ms, len(prompts),
                                                                [r.finish_reason for r in results])
@@ -238,7 +255,12 @@ def repl(engine, sampling, tokenizer, args, stop_ids=None) -> int:
         except ValueError:
             print("without a tokenizer a prompt is a list of token ids", file=sys.stderr)
             continue
-        results, _ = engine.generate([ids], sampling, args.max_new_tokens, stop_token_ids=stop_ids, ignore_eos=args.ignore_eos)
+        try:
+            results, _ = engine.generate([ids], sampling, args.max_new_tokens, stop_token_ids=stop_ids,
+                                         ignore_eos=args.ignore_eos)
+        except (ValueError, CacheFull) as e:
+            print(f"{type(e).__name__}: {e}", file=sys.stderr)
+            continue
         out = results[0].token_ids
         print(tokenizer.decode(out) if tokenizer else " ".join(map(str, out)), flush=True)
     return 0

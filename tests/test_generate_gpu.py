@@ -141,6 +141,14 @@ def test_command_line_generates_and_reports(model_dirs):
     assert r.returncode == 0 and [int(t) for t in r.stdout.split()] == free, r.stderr[-2000:]
     r = subprocess.run(common + ["--stop-token-ids", f"{free[4]},999"], capture_output=True, text=True, timeout=120)
     assert r.returncode == 0 and [int(t) for t in r.stdout.split()] == free[:free.index(free[4]) + 1], r.stderr[-2000:]
+    # what cannot run ends with one line and status 1, not with a traceback
+    for extra, says in ((["--prompt-ids", "1,2,900"], "outside the vocabulary"), (["--prompt-ids", ",".join(["1"] * 300)], "300")):
+        r = subprocess.run([str(ROOT / "bin" / "palm_chat"), "--package", str(model_dirs["A"]["float32"]), "--n-ctx", "128",
+                            "--max-new-tokens", "4"] + extra, capture_output=True, text=True, timeout=120)
+        assert r.returncode == 1 and says in r.stderr and "Traceback" not in r.stderr, r.stderr[-2000:]
+    r = subprocess.run([str(ROOT / "bin" / "palm_chat"), "--package", str(ROOT / "no_such_folder"), "--prompt-ids", "1"],
+                       capture_output=True, text=True, timeout=120)
+    assert r.returncode == 1 and "no config.json" in r.stderr and "Traceback" not in r.stderr
     bad = subprocess.run([str(ROOT / "bin" / "palm_chat"), "--package", str(model_dirs["A"]["float32"]), "--temperature", "3"],
                          capture_output=True, text=True, timeout=120)
     assert bad.returncode == 1 and "temperature must be between 0 and 2" in bad.stderr
