@@ -60,11 +60,22 @@ def main(argv=None) -> int:
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="the most tokens that live requests hold at any time (each rounded up to 64)")
     args = ap.parse_args(argv)
+    from ..cache import CacheFull
     from .engine import Engine
-    engine = Engine.from_dir(args.model, dtype=args.dtype, max_tokens=args.max_tokens)
+    try:
+        engine = Engine.from_dir(args.model, dtype=args.dtype, max_tokens=args.max_tokens)
+    except (ValueError, FileNotFoundError, RuntimeError) as e:
+        print(f"trace_run: {type(e).__name__}: {e}", file=sys.stderr)
+        return 1
 
     def report(msg):
         print(msg, flush=True)
 
-    replay(engine, sys.stdin, args.out, report)
+    try:
+        replay(engine, sys.stdin, args.out, report)
+    except (ValueError, KeyError, CacheFull) as e:
+        # a line that is no JSON object of the form above, a token outside the vocabulary, more tokens than
+        # --max-tokens holds: the steps before it are done and reported, this one changed nothing
+        print(f"trace_run: {type(e).__name__}: {e}", file=sys.stderr)
+        return 1
     return 0

@@ -138,3 +138,14 @@ def test_replay_drives_the_framework_s_own_step(model_dirs, tmp_path):
     s1 = eng.step([StepEntry(x, reqs[0][15:16], [0])]).cpu()
     assert torch.equal(read_logits(out, 0, 256), s0) and torch.equal(read_logits(out, 1, 256), s1)
     assert not (out / "2.f32").exists()
+
+
+def test_a_step_that_cannot_run_ends_the_replay_with_one_line(model_dirs, tmp_path):
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": [1, 2, 3], "want": [2]}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": [1] * 200, "want": []}], "end": []}]
+    proc = subprocess.run([str(ROOT / "bin" / "trace_run"), "--model", str(model_dirs["A"]["float32"]), "--dtype", "float32",
+                           "--out", str(tmp_path / "o"), "--max-tokens", "128"], input="".join(json.dumps(s) + "\n" for s in steps),
+                          capture_output=True, text=True, timeout=120)
+    assert proc.returncode == 1 and proc.stdout.strip() == "done 0"
+    assert "CacheFull" in proc.stderr and "Traceback" not in proc.stderr
+    assert (tmp_path / "o" / "0.f32").exists()
