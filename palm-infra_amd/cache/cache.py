@@ -158,9 +158,10 @@ class ModelCache:
         self.lengths[slot] = 0
         self.slots.give_back(slot)
 
-    def reserve(self, growth: list[tuple[int, int]]) -> None:
-        """Make room for ``n_new`` more tokens in each ``(slot, n_new)``; nothing is taken if the
-        whole step does not fit."""
+    def check_room(self, growth: list[tuple[int, int]], in_pieces: bool = False) -> None:
+        """Raise ``CacheFull`` (or ``CacheMisuse``) if the step does not fit; take nothing.  ``in_pieces``: the
+        tokens will go through in several steps, between which a windowed group gives pages back, so only the
+        groups that keep every key are asked for the whole growth."""
         for slot, n_new in growth:
             if not self.slots.is_held(slot):
                 raise CacheMisuse(f"slot {slot} is used but not open")
@@ -168,10 +169,17 @@ class ModelCache:
                 raise CacheFull(f"slot {slot}: {self.lengths[slot]} + {n_new} tokens exceed the longest sequence "
                                 f"the cache takes ({self.max_seq_tokens})")
         for g in self.kv_groups:
+            if in_pieces and g.need.window:
+                continue
             need = sum(g.table.pages_needed(slot, self.lengths[slot] + n) for slot, n in growth)
             if need > g.table.pages.free_count:
                 raise CacheFull(f"the step needs {need} more pages of {PAGE_TOKENS} tokens; "
                                 f"{g.table.pages.free_count} of {g.n_pages} are free")
+
+    def reserve(self, growth: list[tuple[int, int]]) -> None:
+        """Make room for ``n_new`` more tokens in each ``(slot, n_new)``; nothing is taken if the
+        whole step does not fit."""
+        self.check_room(growth)
         for g in self.kv_groups:
             for slot, n in growth:
                 g.table.grow(slot, self.lengths[slot] + n)

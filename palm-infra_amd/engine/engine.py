@@ -49,7 +49,7 @@ def resolve_dtype(dtype) -> torch.dtype:
 
 class Engine:
     def __init__(self, config, spec, weights, dtype: torch.dtype, max_tokens: int, max_seqs: int | None = None,
-                 device="cuda:0", graphs: bool = True):
+                 device="cuda:0", graphs: bool = True, max_step_tokens: int = 32768):
         self.device = torch.device(device)
         if self.device.type != "cuda":
             raise RuntimeError(f"the engine runs on a GPU; device {device!r} was asked for and there is no CPU path")
@@ -66,6 +66,11 @@ class Engine:
         # a windowed group gives pages back only between steps, so long prompts go through it in pieces
         windows = [g.need.window for g in self.cache.kv_groups if g.need.window]
         self.step_tokens_per_seq = max(1024, 2 * max(windows)) if windows else None
+        # the most tokens that run through the layers at once: longer steps go through in pieces, so that a step's
+        # activations (the widest: tokens x twice the feed-forward width) stay within a few gigabytes
+        if max_step_tokens < 1:
+            raise ValueError(f"max_step_tokens = {max_step_tokens} must be positive")
+        self.max_step_tokens = int(max_step_tokens)
 
     # ---- construction ------------------------------------------------------------------------
     @classmethod
@@ -127,21 +132,30 @@ class Engine:
         order of the entries and of each entry's ``want``.  Nothing changes if the step is refused."""
         entries = [e if isinstance(e, StepEntry) else StepEntry(*e) for e in entries]
         self._validate(entries)
-        limit = self.step_tokens_per_seq
-        if limit is None or all(len(e.tokens) <= limit for e in entries):
+        per_seq, per_step = self.step_tokens_per_seq, self.max_step_tokens
+        total = sum(len(e.tokens) for e in entries)
+        if (per_seq is None or all(len(e.tokens) <= per_seq for e in entries)) and total <= per_step:
             return self._run(entries)
-        # pieces of at most `limit` tokens per sequence, one after the other
+        # Pieces: a sequence's tokens go through in order, at most `per_seq` of them a step (a windowed group gives
+        # pages back between steps) and at most `per_step` tokens of all sequences together (what bounds the memory
+        # of a step's activations).  A sequence's result does not depend on how its tokens are cut.
+        self.cache.check_room([(e.slot, len(e.tokens)) for e in entries], in_pieces=True)
+        per_seq = per_seq or per_step
+        fed = [0] * len(entries)
         results = {}
-        n_pieces = max((len(e.tokens) + limit - 1) // limit for e in entries)
-        for c in range(n_pieces):
-            piece, back = [], []
+        while any(fed[i] < len(e.tokens) for i, e in enumerate(entries)):
+            piece, back, room = [], [], per_step
             for i, e in enumerate(entries):
-                toks = e.tokens[c * limit:(c + 1) * limit]
-                if not toks:
+                if room == 0:
+                    break
+                n = min(len(e.tokens) - fed[i], per_seq, room)
+                if n <= 0:
                     continue
-                want = [w - c * limit for w in e.want if c * limit <= w < (c + 1) * limit]
-                piece.append(StepEntry(e.slot, toks, want))
-                back.extend((i, w + c * limit) for w in want)
+                lo, hi = fed[i], fed[i] + n
+                want = [w - lo for w in e.want if lo <= w < hi]
+                piece.append(StepEntry(e.slot, e.tokens[lo:hi], want))
+                back.extend((i, w + lo) for w in want)
+                fed[i], room = hi, room - n
             logits = self._run(piece)
             for r, key in enumerate(back):
                 results[key] = logits[r]

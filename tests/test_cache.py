@@ -77,6 +77,10 @@ def test_a_step_that_does_not_fit_takes_nothing():
     assert c.kv_groups[0].table.pages.free_count == free and c.lengths[a] == 64
     with pytest.raises(CacheFull, match="longest sequence"):
         c.reserve([(b, 64 * 4 + 1)])
+    with pytest.raises(CacheFull, match="more pages"):
+        c.check_room([(a, 65), (b, 100)])            # the same question without taking anything
+    c.check_room([(a, 64), (b, 100)])
+    assert c.kv_groups[0].table.pages.free_count == free and c.lengths[a] == 64 and c.lengths[b] == 0
     with pytest.raises(CacheMisuse, match="not open"):
         c.reserve([(3, 1)])
     c.check()
