@@ -110,14 +110,17 @@ class Qwen3Config:
 
     # ------------------------------------------------------------------------------------------
     def spec(self, tensor_names=None) -> ModelSpec:
-        """The model as parts.  ``tensor_names`` (the names a checkpoint holds) settles the head when
-        config.json does not say whether it is tied."""
+        """The model as parts.  ``tensor_names`` (the names a checkpoint holds) settles the head as the reference
+        does (models/qwen3.py:89-95, 162-165): ``lm_head.weight`` if the checkpoint has it, else the embedding,
+        whatever ``tie_word_embeddings`` says (the reference never reads that key).  Without a checkpoint
+        (random weights) the key decides."""
         H, nh, nkv, hd, I, V = (self.hidden_size, self.num_attention_heads, self.num_key_value_heads,
                                 self.head_dim, self.intermediate_size, self.vocab_size)
         eps = self.rms_norm_eps
-        tied = self.tie_word_embeddings
-        if tied is None:
-            tied = tensor_names is not None and "lm_head.weight" not in tensor_names
+        if tensor_names is not None:
+            tied = "lm_head.weight" not in tensor_names
+        else:
+            tied = bool(self.tie_word_embeddings)
 
         def norm(name: str, width: int) -> PartSpec:
             return PartSpec("norm", "rms", {"width": width, "eps": eps},

@@ -105,11 +105,11 @@ def test_head_is_tied_by_key_or_by_what_the_checkpoint_holds():
     assert "lm_head.weight" not in config_from_dict(raw).spec().expected_tensors()
     raw["tie_word_embeddings"] = False
     assert "lm_head.weight" in config_from_dict(raw).spec().expected_tensors()
-    raw.pop("tie_word_embeddings")
-    cfg = config_from_dict(raw)
-    # models/qwen3.py:89-95, 162-165: lm_head.weight if the file has it, else the embedding
-    assert "lm_head.weight" in cfg.spec(["lm_head.weight", "model.embed_tokens.weight"]).expected_tensors()
-    assert "lm_head.weight" not in cfg.spec(["model.embed_tokens.weight"]).expected_tensors()
+    # models/qwen3.py:89-95, 162-165: lm_head.weight if the file has it, else the embedding, whatever the key says
+    for tie in (True, False, None):
+        cfg = config_from_dict({k: v for k, v in dict(raw, tie_word_embeddings=tie).items() if v is not None})
+        assert "lm_head.weight" in cfg.spec(["lm_head.weight", "model.embed_tokens.weight"]).expected_tensors()
+        assert "lm_head.weight" not in cfg.spec(["model.embed_tokens.weight"]).expected_tensors()
 
 
 def test_run_order_is_data_and_is_checked():

@@ -78,15 +78,27 @@ def test_one_error_lists_missing_unexpected_and_misshapen(tmp_path):
         assert word in text, word
 
 
-def test_tied_config_with_a_stored_head_is_reported(tmp_path):
+def test_a_stored_head_is_used_whatever_the_config_says(tmp_path):
+    """models/qwen3.py:89-95, 162-165: lm_head.weight if the checkpoint has it, else the embedding; the reference
+    never reads tie_word_embeddings."""
     tensors = tiny.sharpened_tensors("A", "float32")
-    tensors["lm_head.weight"] = torch.zeros(256, 64)
+    tensors["lm_head.weight"] = torch.full((256, 64), 0.5)
     (tmp_path / "config.json").write_text(json.dumps(tiny.CONFIGS["A"]))      # tie_word_embeddings: true
     write_safetensors(tmp_path / "model.safetensors", tensors)
     files = ModelFiles(tmp_path)
-    with pytest.raises(WeightError) as e:
-        load_weights(config_from_dir(tmp_path).spec(files.names()), files, torch.float32, "cpu")
-    assert e.value.unexpected == ["lm_head.weight"]
+    spec = config_from_dir(tmp_path).spec(files.names())
+    w = load_weights(spec, files, torch.float32, "cpu")
+    assert torch.equal(w.get(spec.head.tensors["weight"]), tensors["lm_head.weight"])
+    # and the other way round: the key says untied, the checkpoint has no head of its own
+    d = tmp_path / "b"
+    d.mkdir()
+    tensors = {k: v for k, v in tiny.sharpened_tensors("B", "float32").items() if k != "lm_head.weight"}
+    (d / "config.json").write_text(json.dumps(tiny.CONFIGS["B"]))             # tie_word_embeddings: false
+    write_safetensors(d / "model.safetensors", tensors)
+    files = ModelFiles(d)
+    spec = config_from_dir(d).spec(files.names())
+    w = load_weights(spec, files, torch.float32, "cpu")
+    assert w.get(spec.head.tensors["weight"]).data_ptr() == w.get(spec.embedding.tensors["table"]).data_ptr()
 
 
 def test_what_is_kept_in_which_precision(tmp_path):
