@@ -20,8 +20,6 @@ import json
 import sys
 from pathlib import Path
 
-import numpy as np
-
 
 def replay(engine, lines, out_dir, report=print) -> None:
     out_dir = Path(out_dir)

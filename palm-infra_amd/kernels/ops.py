@@ -6,7 +6,6 @@ are only memory here: no torch operator computes on the product path.
 """
 from __future__ import annotations
 
-import ctypes
 from ctypes import c_float, c_int, c_longlong, c_void_p
 
 import torch

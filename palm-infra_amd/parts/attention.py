@@ -9,8 +9,6 @@ h // (heads / kv_heads) (kernels/attention.cpp:1161); output projection.  No bia
 """
 from __future__ import annotations
 
-import torch
-
 from ..cache import KVNeed
 from ..kernels import ops
 from .base import register_part

@@ -2,8 +2,6 @@
 joined into one [2I, H] product (models/qwen3.py:276-287; kernels/elementwise.cpp:529-583)."""
 from __future__ import annotations
 
-import torch
-
 from .base import register_part
 from .linear import Linear
 

@@ -4,8 +4,8 @@ import random
 import pytest
 import torch
 
-from palm_infra_amd.cache import (PAGE_TOKENS, CacheFull, CacheMisuse, FreeList, KVNeed, ModelCache, PageTable,
-                                  StateNeed, pages_for)
+from palm_infra_amd.cache import (PAGE_TOKENS, CacheFull, CacheMisuse, FreeList, KVNeed, ModelCache, StateNeed,
+                                  pages_for)
 
 
 def test_free_list_hands_out_each_number_once_and_lowest_first():

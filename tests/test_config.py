@@ -113,7 +113,7 @@ def test_head_is_tied_by_key_or_by_what_the_checkpoint_holds():
 
 
 def test_run_order_is_data_and_is_checked():
-    from palm_infra_amd.config import LayerCall, ModelSpec
+    from palm_infra_amd.config import LayerCall
     spec = config_from_dict(tiny.CONFIGS["A"]).spec()
     import dataclasses
     twice = dataclasses.replace(spec, order=(LayerCall(0), LayerCall(1), LayerCall(0), LayerCall(1, cache_of=1)))

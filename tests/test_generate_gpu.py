@@ -1,7 +1,6 @@
 """Generation through the entry points: greedy tokens equal the plain implementation's; temperature
 sampling is reproducible and a sequence's tokens do not depend on its batch companions."""
 import subprocess
-import sys
 from pathlib import Path
 
 import pytest

@@ -1,6 +1,5 @@
 """The matrix-core kernels alone against their plain references: the thin linear product (with and
 without the gated epilogue) and the bfloat16 attention kernels, at sizes other than the tiny models'."""
-import math
 
 import pytest
 import torch

@@ -186,7 +186,6 @@ def test_embedding_and_head_parts(dtype):
 def test_block_part_is_a_plain_decoder_layer(dtype, n_rows, model_dirs):
     """One layer of tiny model C, built as a block from the model's description and run alone: with many rows
     (the norms run as kernels of their own) and with few (in bfloat16 the products fold them in)."""
-    import tiny
     from palm_infra_amd.cache import ModelCache
     from palm_infra_amd.config import config_from_dir
     from palm_infra_amd.parts import Builder, Prenormed, ResidualSink, as_tensor, cache_needs, make_context

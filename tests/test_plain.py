@@ -10,7 +10,6 @@ import torch.nn.functional as F
 
 import plain_qwen3 as P
 import tiny
-from palm_infra_amd.config import config_from_dict
 
 F64 = torch.float64
 

@@ -1,7 +1,6 @@
 """Sampling options and the host side of the sampler (no GPU)."""
 import pytest
 
-import plain_qwen3 as P
 from palm_infra_amd.sampling import GREEDY, SamplingError, SamplingParams, SequenceSampling, penalty_counts, uniform
 
 

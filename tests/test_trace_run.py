@@ -3,7 +3,6 @@ requests are replayed whole, with the last 32 tokens one by one, and in batches 
 float32 and in bfloat16, and compared with the plain implementation."""
 import json
 import subprocess
-import sys
 from pathlib import Path
 
 import numpy as np
