@@ -4,11 +4,16 @@
 //
 // This is the exact path: plain FMA in 32-bit, no matrix-core mode of reduced precision.  Every output
 // element adds its products in the same order of k whatever M and N are, so a row's result does not
-// depend on how many rows are computed with it.  It serves the float32 mode and any mix of element
+// depend on how many rows are computed with it.  The sum goes in two levels, runs of SUM_RUN products and then
+// the runs' sums: a 32-bit sum of K terms one after the other is off by about sqrt(K) roundings, which at
+// K = 12288 and 36 layers adds up to more than 1e-4 on logits of order one; two levels leave
+// sqrt(SUM_RUN) + sqrt(K / SUM_RUN).  It serves the float32 mode and any mix of element
 // types (a 32-bit matrix under bfloat16 activations).
 #include "common.h"
 
 constexpr int TILE_M = 64, TILE_N = 64, TILE_K = 16;
+constexpr int SUM_RUN = 256;          // products added one after the other before their sum joins the total
+static_assert(SUM_RUN % TILE_K == 0, "a run is a whole number of tiles");
 
 template <typename TA, typename TW, typename TC>
 __global__ __launch_bounds__(256) void linear_tiled_kernel(const TA* __restrict__ A, const TW* __restrict__ W,
@@ -20,7 +25,7 @@ __global__ __launch_bounds__(256) void linear_tiled_kernel(const TA* __restrict_
     const int tx = tid % 16, ty = tid / 16;          // thread computes rows ty*4.., columns tx*4..
     const int m0 = blockIdx.y * TILE_M, n0 = blockIdx.x * TILE_N;
     const int lrow = tid / 4, lk = (tid % 4) * 4;    // what this thread loads: one row, four k
-    float acc[4][4] = {};
+    float acc[4][4] = {}, total[4][4] = {};
     for (int k0 = 0; k0 < K; k0 += TILE_K) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -40,6 +45,12 @@ __global__ __launch_bounds__(256) void linear_tiled_kernel(const TA* __restrict_
 #pragma unroll
                 for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], w[j], acc[i][j]);
         }
+        if ((k0 + TILE_K) % SUM_RUN == 0 || k0 + TILE_K >= K) {      // the run is over: its sum joins the total
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) { total[i][j] += acc[i][j]; acc[i][j] = 0.f; }
+        }
         __syncthreads();
     }
 #pragma unroll
@@ -50,7 +61,7 @@ __global__ __launch_bounds__(256) void linear_tiled_kernel(const TA* __restrict_
         for (int j = 0; j < 4; ++j) {
             const int n = n0 + tx * 4 + j;
             if (n >= N) continue;
-            float v = acc[i][j];
+            float v = total[i][j];
             if (accumulate) v += to_float(C[(size_t)m * N + n]);
             C[(size_t)m * N + n] = from_float<TC>(v);
         }
