@@ -383,6 +383,14 @@ def test_attention_exact_prompts_decode_and_mixed_lengths(ops, dtype, nh, nkv, h
         assert torch.allclose(got, ref, atol=1e-5 if dtype == F32 else 2e-2), lens
 
 
+def test_attention_exact_over_thousands_of_keys(ops):
+    """The float32 path's attention keeps its 1e-5 where a query sees thousands of keys (a prompt's continuation
+    far into a sequence, single queries)."""
+    for lens in ([(3000, 40)], [(2048, 1), (4500, 1), (70, 70)]):
+        got, ref = _attention_case(ops, ops.attention_exact, F32, 8, 2, 64, lens, None, seed=len(lens))
+        assert torch.allclose(got, ref, atol=1e-5), (lens, float((got - ref).abs().max()))
+
+
 @pytest.mark.parametrize("dtype", [F32, BF16])
 def test_attention_exact_window(ops, dtype):
     for window in (1, 5, 64, 100):

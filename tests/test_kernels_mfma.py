@@ -213,6 +213,19 @@ def test_attention_decode_mfma(ops, nh, nkv, hd, n_slices):
         assert torch.allclose(got, ref, atol=2e-2), (lens, float((got - ref).abs().max()))
 
 
+@pytest.mark.parametrize("nh,nkv,hd", [(32, 8, 128), (4, 2, 64), (6, 1, 80)])
+def test_attention_mfma_long_sequences(ops, nh, nkv, hd):
+    """The measured lengths and beyond: a 2,048-token prompt (32 pages, query tiles paired from both ends, a
+    running maximum that is followed only now and then), a prompt's continuation far into a sequence, unequal
+    prompts together, and single queries over thousands of keys in few and in many slices."""
+    for lens in ([(2048, 2048)], [(4100, 1000)], [(1500, 1500), (70, 70), (2304, 300)]):
+        got, ref = _attention_case(ops, ops.attention_prefill, BF16, nh, nkv, hd, lens, None, seed=len(lens) + hd)
+        assert torch.allclose(got, ref, atol=2e-2), (lens, float((got - ref).abs().max()))
+    for n_slices in (2, 12, 64):
+        got, ref = _attention_case(ops, decode_fn(ops, n_slices), BF16, nh, nkv, hd, [(5000, 1), (2049, 1), (3, 1)], None, seed=hd)
+        assert torch.allclose(got, ref, atol=2e-2), (n_slices, float((got - ref).abs().max()))
+
+
 @pytest.mark.parametrize("window", [1, 5, 64, 100, 1000])
 def test_attention_mfma_window(ops, window):
     got, ref = _attention_case(ops, ops.attention_prefill, BF16, 4, 2, 32, [(200, 200), (150, 1), (70, 3), (90, 30)], window, seed=window)
