@@ -38,7 +38,7 @@ def real():
     return raw, cfg, spec, tensors, prompts, refs
 
 
-def engine_of(real, dtype):
+def engine_of(real, dtype, pages=16):
     from palm_infra_amd.engine import Engine
     from palm_infra_amd.weights.loader import Weights, kept_dtype
     raw, cfg, spec, tensors, _, _ = real
@@ -47,7 +47,7 @@ def engine_of(real, dtype):
     for ref in spec.tensor_refs():
         dt = kept_dtype(ref, ["BF16"] * len(ref.names), mode)
         held[ref.names] = torch.cat([tensors[n] for n in ref.names]).to("cuda:0", dt)
-    return Engine(cfg, spec, Weights(held), mode, max_tokens=64 * 16)
+    return Engine(cfg, spec, Weights(held), mode, max_tokens=64 * pages)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -75,4 +75,32 @@ def test_whole_prompts_then_tokens_one_by_one_and_a_batch(real, dtype):
         row += n
     for s in slots:
         eng.close(s)
+    eng.cache.check()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_steps_of_many_sequences(real, dtype):
+    """40 sequences, then 24 of them, each one token further: in bfloat16 these are the kernels for 17 to 64
+    rows at the measured widths (the gated product over 24,576 weight rows, products cut along K into planes
+    that the norms and the q/k/v pass add up), recorded into a graph on their second step."""
+    from palm_infra_amd.engine import StepEntry
+    raw = real[0]
+    eng = engine_of(real, dtype, pages=48)
+    oracle = {k: v.double() for k, v in real[3].items()}
+    g = torch.Generator().manual_seed(6)
+    seqs = [torch.randint(0, raw["vocab_size"], (2 + b % 4 + 3,), generator=g).tolist() for b in range(40)]
+    refs = [P.logits(raw, oracle, ids) for ids in seqs]
+    slots = [eng.open() for _ in seqs]
+    eng.step([StepEntry(s, ids[:-3], []) for s, ids in zip(slots, seqs)])
+    live = list(range(40))
+    for t in (3, 2, 1):                                  # 40 sequences twice (the second step is a replay), then 24
+        if t == 1:
+            for b in live[24:]:
+                eng.close(slots[b])
+            live = live[:24]
+        got = eng.step([StepEntry(slots[b], [seqs[b][-t]], [0]) for b in live])
+        ref = torch.stack([refs[b][len(seqs[b]) - t] for b in live])
+        tiny.assert_logits_close(got, ref, dtype, f"{len(live)} sequences, {t} tokens before the end")
+    for b in live:
+        eng.close(slots[b])
     eng.cache.check()
