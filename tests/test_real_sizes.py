@@ -106,3 +106,24 @@ def test_decode_steps_of_many_sequences(real, dtype):
     for b in live:
         eng.close(slots[b])
     eng.cache.check()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_long_prompt_and_the_tokens_after_it(real, dtype):
+    """2,100 tokens in one step (34 pages; in bfloat16 the prompt kernels of the measured run: library products
+    of thousands of rows, the q/k/v pass that holds heads in registers, matrix-core attention with query tiles
+    paired from both ends), then three tokens one by one over 33 and 34 pages in slices."""
+    from palm_infra_amd.engine import StepEntry
+    raw = real[0]
+    if raw["hidden_size"] != 4096:
+        pytest.skip("one size is enough for the long prompt")
+    eng = engine_of(real, dtype, pages=40)
+    oracle = {k: v.double() for k, v in real[3].items()}
+    ids = torch.randint(0, raw["vocab_size"], (2103,), generator=torch.Generator().manual_seed(8)).tolist()
+    places = [0, 63, 64, 1000, 2047, 2048, 2099]
+    ref = P.logits(raw, oracle, ids)
+    s = eng.open()
+    got = [eng.step([StepEntry(s, ids[:2100], places)])]
+    got += [eng.step([StepEntry(s, [t], [0])]) for t in ids[2100:]]
+    eng.close(s)
+    tiny.assert_logits_close(torch.cat(got), ref[places + [2100, 2101, 2102]], dtype, "2,100-token prompt and three more tokens")
