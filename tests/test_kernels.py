@@ -123,6 +123,24 @@ def test_swiglu(ops, dtype):
     assert not torch.allclose(got.double(), swapped, atol=0.1)
 
 
+def test_swiglu_of_bfloat16_rows_far_from_zero(ops):
+    """The prompt kernel for bfloat16 uses the hardware's 2^x and reciprocal: gates from -100 (where 2^x overflows
+    and the weight must come out as zero, not as a NaN) to +100, rounded to the nearest bfloat16."""
+    gate = torch.tensor([-100.0, -90.0, -40.0, -20.0, -5.0, -1.0, -0.0, 0.0, 0.5, 1.0, 3.0, 10.0, 30.0, 88.0, 90.0, 100.0])
+    gu = torch.cat([gate.repeat(3, 4), rand(3, 64, seed=9, scale=5.0, dtype=F32)], dim=1).to(BF16)         # [3, 2 * 64]
+    got = ops.swiglu(gu.to(DEV)).cpu()
+    g, u = gu[:, :64].double(), gu[:, 64:].double()
+    want = (g / (1 + torch.exp(-g)) * u).to(BF16)
+    assert torch.isfinite(got.float()).all()
+    # at most one step of bfloat16 away from the rounded exact value (a product that lies next to a rounding border);
+    # where 2^x overflows (a gate below -88) the exact weight is below 1e-36 and the kernel's is zero
+    steps = (got.view(torch.int16).int() - want.view(torch.int16).int()).abs()
+    tiny_ones = (want.float().abs() < 1e-30) & (got.float().abs() < 1e-30)
+    steps = torch.where(tiny_ones, torch.zeros_like(steps), steps)
+    assert int(steps.max()) <= 1 and float((steps > 0).float().mean()) < 0.05, (int(steps.max()), float((steps > 0).float().mean()))
+    assert int(tiny_ones.sum()) >= 6
+
+
 def test_cast_rounds_to_nearest_even(ops):
     x = torch.tensor([1.0, 1.00390625, 1.01171875, -3.1415927, 1e-40, 65504.0, float("inf")])
     assert torch.equal(ops.cast(x.to(DEV), BF16).cpu(), x.to(BF16))
