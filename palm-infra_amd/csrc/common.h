@@ -25,8 +25,14 @@ __host__ __device__ inline float to_float(bf16_t v) {
     return c.f;
 }
 
-// round to nearest, ties to even; NaN stays NaN
+// round to nearest, ties to even; NaN stays NaN.  On the device this is the hardware's conversion (one
+// instruction for two values); the arithmetic below serves host code and says what the conversion does.
 __host__ __device__ inline bf16_t f32_to_bf16(float f) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    bf16_t native;
+    native.bits = __builtin_bit_cast(uint16_t, (__bf16)f);
+    return native;
+#endif
     union { uint32_t u; float f; } c;
     c.f = f;
     bf16_t r;
