@@ -68,6 +68,25 @@ def test_rmsnorm_adds_the_pending_branch_in_32_bit(ops, out_dtype, delta_dtype):
     assert torch.allclose(sel.double(), P.rms_norm(x.double() + d.double(), w, 1e-5)[[6, 0, 3]], atol=2e-5)
 
 
+@pytest.mark.parametrize("width", [2048, 4096, 5120, 8200, 5000])
+@pytest.mark.parametrize("dtypes", [(BF16, BF16), (F32, F32), (BF16, F32), (None, BF16)])
+def test_rmsnorm_of_many_rows(ops, width, dtypes):
+    """Prompts: hundreds of rows of the widths that models have, with and without a pending branch, whole and
+    through a row selection."""
+    delta_dtype, out_dtype = dtypes
+    n = 300
+    x, w = rand(n, width, seed=width), rand(width, seed=4) + 1.0
+    d = rand(n, width, seed=3, dtype=delta_dtype) if delta_dtype is not None else None
+    xd = x.to(DEV)
+    got = ops.rmsnorm(xd, w.to(DEV), 1e-6, out_dtype, delta=None if d is None else d.to(DEV), update_x=d is not None).cpu()
+    total = x if d is None else x + d.float()
+    assert torch.equal(xd.cpu(), total)                               # the stream holds the exact 32-bit sum (or is untouched)
+    assert torch.allclose(got.double(), P.rms_norm(total.double(), w, 1e-6), atol=1e-4 if out_dtype == F32 else 2e-2, rtol=0 if out_dtype == F32 else 1e-2)
+    rows = torch.arange(n - 1, -1, -1, dtype=torch.int32).to(DEV)       # a selection of as many rows, backwards
+    sel = ops.rmsnorm(x.to(DEV), w.to(DEV), 1e-6, F32, delta=None if d is None else d.to(DEV), rows=rows).cpu()
+    assert torch.allclose(sel.double(), P.rms_norm(total.double(), w, 1e-6).flip(0), atol=1e-4)
+
+
 @pytest.mark.parametrize("planes", [2, 3, 4])
 @pytest.mark.parametrize("width", [96, 4096, 5000])
 def test_rmsnorm_adds_planes_of_partial_sums_in_their_order(ops, planes, width):
