@@ -241,28 +241,33 @@ def _generate_and_report(ap, args, engine, sampling, tokenizer, prompts, stop_id
 
 
 def repl(engine, sampling, tokenizer, args, stop_ids=None) -> int:
-    """Prompts from standard input, one a line (text with a tokenizer, else token ids); ``/quit`` ends,
-    ``/reset`` is accepted for the reference's users: every line starts a fresh sequence here."""
-    print("one prompt a line; /quit to end", file=sys.stderr)
+    """Turns from standard input, one a line (text with a tokenizer, else token ids).  The conversation stays in
+    the cache: a turn feeds only its own tokens on top of what earlier turns left (examples/main.cpp:394-466);
+    ``/reset`` starts over, ``/quit`` ends (examples/main.cpp:524-548)."""
+    print("one turn a line; /reset to start over, /quit to end", file=sys.stderr)
+    talk = engine.conversation(sampling, stop_token_ids=stop_ids, ignore_eos=args.ignore_eos)
     for line in sys.stdin:
         line = line.strip()
-        if not line or line == "/reset":
+        if not line:
+            continue
+        if line == "/reset":
+            talk.reset()
             continue
         if line in ("/quit", "/exit"):
             break
         try:
             ids = tokenizer.encode(line).ids if tokenizer else [int(t) for t in line.replace(",", " ").split()]
         except ValueError:
-            print("without a tokenizer a prompt is a list of token ids", file=sys.stderr)
+            print("without a tokenizer a turn is a list of token ids", file=sys.stderr)
             continue
         try:
-            results, _ = engine.generate([ids], sampling, args.max_new_tokens, stop_token_ids=stop_ids,
-                                         ignore_eos=args.ignore_eos)
+            result = talk.say(ids, args.max_new_tokens)
         except (ValueError, CacheFull) as e:
             print(f"{type(e).__name__}: {e}", file=sys.stderr)
             continue
-        out = results[0].token_ids
+        out = result.token_ids
         print(tokenizer.decode(out) if tokenizer else " ".join(map(str, out)), flush=True)
+    talk.reset()
     return 0
 
 

@@ -292,3 +292,11 @@ class Engine:
             stop = self.spec.stop_token_ids if stop_token_ids is None else stop_token_ids
         return generate(self, sampler, prompts, max_new_tokens=max_new_tokens, stop_token_ids=stop, max_batch=max_batch,
                         on_token=on_token, sync=torch.cuda.synchronize)
+
+    def conversation(self, sampling=None, stop_token_ids=None, ignore_eos: bool = False):
+        """A sequence that stays in the cache from turn to turn: ``say(new tokens)`` feeds only what is new and
+        generates; ``reset()`` starts over.  See ``engine.generate.Conversation``."""
+        from ..sampling import DeviceSampler, SamplingParams
+        from .generate import Conversation
+        stop = () if ignore_eos else (self.spec.stop_token_ids if stop_token_ids is None else stop_token_ids)
+        return Conversation(self, DeviceSampler(sampling or SamplingParams()), stop)

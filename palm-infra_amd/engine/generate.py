@@ -171,3 +171,66 @@ def generate(engine, sampler, prompts, max_new_tokens: int = 2048, stop_token_id
             for slot in slots.values():      # only after a fault: every sequence that ended has left already
                 engine.close(slot)
     return results, compute_metrics(results, total_prefill, total_decode)
+
+
+class Conversation:
+    """One sequence kept alive from turn to turn: a turn feeds only its new tokens on top of what the cache holds
+    and generates until a stop token, ``max_new_tokens`` or the cache's end, as the reference's chat loop does with
+    its ``cached_token_ids`` (examples/main.cpp:394-466).  ``reset()`` gives the slot back (the loop's ``/reset``).
+
+    ``engine`` and ``sampler`` as for ``generate``.  The tokens a turn generates are part of the sequence; the
+    last one of a turn (a stop token, or the token at which the turn's length ran out) was chosen but not yet fed
+    to the model, and goes in front of the next turn's tokens."""
+
+    def __init__(self, engine, sampler, stop_token_ids=()):
+        self.engine, self.sampler = engine, sampler
+        self.stop = set(int(t) for t in stop_token_ids)
+        self.slot = None
+        self.state = SequenceSampling(stream=0)
+        self.pending: list[int] = []          # chosen but not yet fed: they go in front of the next turn's tokens
+
+    @property
+    def length(self) -> int:
+        """Tokens the cache holds for this conversation."""
+        return 0 if self.slot is None else self.engine.length(self.slot)
+
+    def reset(self) -> None:
+        if self.slot is not None:
+            self.engine.close(self.slot)
+        self.slot = None
+        self.pending = []
+        self.state.reset()
+
+    def say(self, tokens, max_new_tokens: int = 2048, on_token=None) -> GenerationResult:
+        """Feed ``tokens`` (at least one, unless a token of the last turn is still pending) and generate."""
+        if max_new_tokens < 1:
+            raise ValueError("max_new_tokens must be >= 1")
+        feed = self.pending + [int(t) for t in tokens]
+        if not feed:
+            raise ValueError("a turn needs at least one token")
+        max_seq = self.engine.cache.max_seq_tokens
+        if self.length + len(feed) > max_seq:
+            raise RequestTooLong(f"the conversation holds {self.length} tokens; {len(feed)} more exceed the longest "
+                                 f"sequence the cache takes ({max_seq})")
+        if self.slot is None:
+            self.slot = self.engine.open()
+        result = GenerationResult(prompt_tokens=len(feed))
+        logits = self.engine.step([StepEntry(self.slot, feed, [len(feed) - 1])])
+        self.pending = []
+        self.state.accept(feed)
+        while True:
+            tok = int(self.sampler.sample(logits, [self.state]).tolist()[0])
+            result.token_ids.append(tok)
+            if on_token:
+                on_token(0, tok)
+            if tok in self.stop:
+                result.finish_reason = "stop"
+            elif len(result.token_ids) >= max_new_tokens:
+                result.finish_reason = "length"
+            elif self.length + 1 > max_seq:
+                result.finish_reason = "context"
+            if result.finish_reason:
+                self.pending = [tok]          # the model has not seen it yet
+                return result
+            logits = self.engine.step([StepEntry(self.slot, [tok], [0])])
+            self.state.accept([tok])

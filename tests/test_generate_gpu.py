@@ -180,3 +180,31 @@ def test_command_line_profile_and_trace(tmp_path):
     empty = subprocess.run([str(ROOT / "bin" / "palm_bench"), "--random", "tiny-b", "--trace", ""], capture_output=True,
                            text=True, timeout=120)
     assert empty.returncode == 1 and "--trace path must not be empty" in empty.stderr
+
+
+def test_a_conversation_continues_from_the_cache(model_dirs, engine_a):
+    """Turn by turn on one slot gives what the whole token sequence gives at once (greedy, float32), and the
+    command line's loop of turns does the same."""
+    from palm_infra_amd.sampling import GREEDY
+    cfg, w = P.read_model(model_dirs["A"]["float32"])
+    turns = tiny.prompts("A", [6, 3, 4], seed=33)
+    talk = engine_a.conversation(GREEDY, ignore_eos=True)
+    history, lines = [], []
+    for turn in turns:
+        r = talk.say(turn, max_new_tokens=5)
+        history += turn
+        want = P.greedy(cfg, w, history, 5)                     # the oracle reads the whole conversation again
+        assert r.token_ids == want and r.finish_reason == "length"
+        history += want
+        lines.append(want)
+    assert talk.length == len(history) - 1                      # the last chosen token is not fed yet
+    talk.reset()
+    assert engine_a.cache.slots.held_count == 0
+    engine_a.cache.check()
+    text = "".join(" ".join(map(str, t)) + "\n" for t in turns) + "/reset\n" + " ".join(map(str, turns[0])) + "\n/quit\n"
+    r = subprocess.run([str(ROOT / "bin" / "palm_chat"), "--package", str(model_dirs["A"]["float32"]), "--dtype", "float32",
+                        "--max-new-tokens", "5", "--temperature", "0", "--n-ctx", "256", "--ignore-eos"],
+                       input=text, capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stderr[-2000:]
+    got = [[int(t) for t in line.split()] for line in r.stdout.strip().splitlines()]
+    assert got == lines + [lines[0]]                            # after /reset the first turn gives its first answer again

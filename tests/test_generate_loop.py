@@ -134,3 +134,37 @@ def test_metrics_follow_the_reference_definitions():
     assert m.ttft_ms == 8.0 and m.tpot_ms == 2.0 and m.prefill_tps == 2000.0 and m.decode_tps == 500.0 and m.total_ms == 12.0
     m0 = compute_metrics([GenerationResult(prompt_tokens=3, token_ids=[1])], 1.0, 0.0)
     assert m0.decode_tokens == 0 and m0.tpot_ms == 0.0 and m0.decode_tps == 0.0
+
+
+def test_a_conversation_feeds_only_what_is_new_and_keeps_its_slot():
+    from palm_infra_amd.engine.generate import Conversation
+    # the model counts upwards from the last token it saw; the stop token is 9
+    eng = ScriptedEngine(lambda seen: min(seen[-1] + 1, 9), max_seq_tokens=64)
+    eng.length = lambda slot: len(eng.seen[slot])
+    sampler = ArgmaxSampler()
+    talk = Conversation(eng, sampler, stop_token_ids=(9,))
+    first = talk.say([1, 2, 5], max_new_tokens=10)
+    assert first.token_ids == [6, 7, 8, 9] and first.finish_reason == "stop" and first.prompt_tokens == 3
+    slot = talk.slot
+    assert eng.seen[slot] == [1, 2, 5, 6, 7, 8] and talk.pending == [9]          # the stop token is not fed yet
+    second = talk.say([3], max_new_tokens=2)
+    assert second.token_ids == [4, 5] and second.finish_reason == "length" and second.prompt_tokens == 2
+    assert talk.slot == slot and eng.seen[slot] == [1, 2, 5, 6, 7, 8, 9, 3, 4] and talk.pending == [5]
+    # a turn's first step brings only the new tokens (and the pending one), never the conversation again
+    assert eng.steps[0] == [(slot, 3)] and eng.steps[4] == [(slot, 2)] and all(st == [(slot, 1)] for st in eng.steps[1:4] + eng.steps[5:])
+    # penalties see the whole conversation
+    assert sampler.histories[-1] == [[1, 2, 5, 6, 7, 8, 9, 3, 4]]
+    # a turn may consist of the pending token alone
+    third = talk.say([], max_new_tokens=1)
+    assert third.token_ids == [6] and eng.seen[slot][-1] == 5
+    talk.reset()
+    assert talk.slot is None and eng.closed == [slot] and talk.length == 0 and talk.pending == []
+    with pytest.raises(ValueError, match="at least one token"):
+        talk.say([])
+    # the cache's end: a turn that does not fit is refused, a turn that reaches it ends for "context"
+    with pytest.raises(RequestTooLong):
+        talk.say([1] * 65)
+    assert talk.slot is None
+    full = talk.say([1] * 62, max_new_tokens=50)
+    assert full.finish_reason == "context" and talk.length == 64 and len(full.token_ids) == 3
+    talk.reset()
