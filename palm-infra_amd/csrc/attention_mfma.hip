@@ -21,6 +21,7 @@
 // prefill: one block of four waves per (sequence, kv head, 16 query positions); wave w owns the columns
 //          of query head w of the group (more heads: more passes).
 #include "mfma.h"
+#include "attention_api.h"
 
 #ifndef PALM_HEAD_DIM
 #error "compile with -DPALM_HEAD_DIM=<head size>"
@@ -272,11 +273,7 @@ __global__ __launch_bounds__(WAVE) void attention_merge_kernel(const float* __re
     }
 }
 
-PALM_API int palm_attention_decode_workspace_floats(int n_seqs, int nh, int n_slices) {
-    return n_seqs * nh * n_slices * WORK_STRIDE;
-}
-
-PALM_API int palm_attention_decode(hipStream_t stream, const void* q, const void* k_cache, const void* v_cache,
+static int launch_attention_decode(hipStream_t stream, const void* q, const void* k_cache, const void* v_cache,
                                    const int* block_table, int max_pages, const int* seq_slot, const int* seq_start,
                                    int n_seqs, int nh, int nkv, int hd, float scale, int window, int n_slices,
                                    float* work, void* out) {
@@ -298,6 +295,14 @@ PALM_API int palm_attention_decode(hipStream_t stream, const void* q, const void
         PALM_LAUNCHED();
     }
     return 0;
+}
+
+PALM_API int palm_attention_decode(hipStream_t stream, const void* q, const void* k_cache, const void* v_cache,
+                                   const int* block_table, int max_pages, const int* seq_slot, const int* seq_start,
+                                   int n_seqs, int nh, int nkv, int hd, float scale, int window, int n_slices,
+                                   float* work, void* out) {
+    return launch_attention_decode(stream, q, k_cache, v_cache, block_table, max_pages, seq_slot, seq_start, n_seqs, nh, nkv,
+                                   hd, scale, window, n_slices, work, out);
 }
 
 // ---- prefill --------------------------------------------------------------------------------------
@@ -322,11 +327,13 @@ constexpr float PF_LAZY_LOG2 = 8.0f;                       // how far (in powers
 constexpr int K_CHUNKS = (CHUNKS + 7) / 8 * 8;
 constexpr int K_STRIDE = K_CHUNKS * 8;
 __device__ inline int k_swizzle(int row) { return (row & 3) | (((row >> 3) & 1) << 2); }
-// Head sizes whose key rows are whole multiples of 128 bytes (64, 128) take their pages from memory straight into
-// LDS (global_load_lds: no registers in between, no write instruction); a wave's instruction fills 1 KB of LDS
-// in lane order, so rows cannot be padded there and V^T's chunks are permuted like K's instead (row d's chunk c
-// at c ^ v_swizzle(d): the 16 rows that lanes read together then start in 16 different groups of four banks).
-constexpr bool PF_DMA = CHUNKS % 8 == 0 && (PAGE_TOKENS * K_STRIDE + HD * PAGE_TOKENS) * 2 <= 60 * 1024;
+// Head sizes whose key rows are whole multiples of 128 bytes and of which a whole number fills 1 KB (64, 128)
+// take their pages from memory straight into LDS (global_load_lds: no registers in between, no write
+// instruction); a wave's instruction fills 1 KB of LDS in lane order, so rows cannot be padded there and V^T's
+// chunks are permuted like K's instead (row d's chunk c at c ^ v_swizzle(d): the 16 rows that lanes read together
+// then start in 16 different groups of four banks).  A row of 192 elements (24 chunks) would straddle two
+// instructions' kilobytes, which page_sources() does not describe: such sizes go through registers.
+constexpr bool PF_DMA = CHUNKS % 8 == 0 && WAVE % CHUNKS == 0 && (PAGE_TOKENS * K_STRIDE + HD * PAGE_TOKENS) * 2 <= 60 * 1024;
 constexpr int V_STRIDE = PF_DMA ? PAGE_TOKENS : PAGE_TOKENS + 8;
 __device__ inline int v_swizzle(int row) { return PF_DMA ? (row >> 1) & 7 : 0; }
 constexpr int PAGE_CHUNKS = PAGE_TOKENS * HD / 8;          // 16-byte chunks in a page of K (and of V^T)
@@ -371,7 +378,8 @@ struct PageSources { uint32_t k[PF_LOADS], v[PF_LOADS]; };       // byte offsets
 __device__ inline PageSources page_sources() {
     PageSources src;
     const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
-    constexpr int K_ROWS = WAVE / (CHUNKS > 0 ? CHUNKS : 1);     // key rows an instruction covers
+    static_assert(!PF_DMA || WAVE % CHUNKS == 0, "an instruction's 64 chunks must be whole key rows");
+    constexpr int K_ROWS = WAVE / CHUNKS;                        // key rows an instruction covers
 #pragma unroll
     for (int i = 0; i < PF_LOADS; ++i) {
         const int inst = i * PF_WAVES + wave;

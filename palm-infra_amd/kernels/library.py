@@ -37,7 +37,7 @@ CORE_SOURCES = ["elementwise.hip", "linear.hip", "rope_store.hip", "attention_si
                 "linear_mfma.hip", "linear_wide.hip", "linear_wide_store_32.hip", "linear_wide_store_64.hip",
                 "linear_wide_gated_32.hip", "linear_wide_gated_64.hip"]
 ATTENTION_SOURCES = ["attention_mfma.hip"]
-HEADERS = ["common.h", "mfma.h", "linear_wide.h"]
+HEADERS = ["common.h", "mfma.h", "linear_wide.h", "attention_api.h"]
 
 
 class KernelBuildError(RuntimeError):

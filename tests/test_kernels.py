@@ -435,9 +435,9 @@ def test_attention_exact_window(ops, dtype):
         assert torch.allclose(got, ref, atol=1e-5 if dtype == F32 else 2e-2), window
 
 
-def _spike_case(ops, fn, dtype, L, spike_at, window=None):
+def _spike_case(ops, fn, dtype, L, spike_at, window=None, hd=32):
     """One key among L is made to dominate the last query; the output must be that key's value."""
-    nh, nkv, hd = 2, 1, 32
+    nh, nkv = 2, 1
     k = rand(L, nkv, hd, seed=1, scale=0.1, dtype=dtype)
     v = rand(L, nkv, hd, seed=2, dtype=dtype)
     q = rand(1, nh, hd, seed=3, scale=0.1, dtype=dtype)

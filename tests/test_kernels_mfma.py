@@ -193,7 +193,10 @@ def decode_fn(ops, n_slices):
     return fn
 
 
-HEADS = [(8, 4, 16), (5, 5, 48), (6, 1, 80), (4, 2, 128), (32, 8, 128), (40, 2, 32), (3, 3, 256)]
+# 192 and 112: rows of 24 and 14 chunks, which do not divide an instruction's 64 (a page must then go through
+# registers into LDS); 144 and 240: two pages that need more LDS than the smaller sizes
+HEADS = [(8, 4, 16), (5, 5, 48), (6, 1, 80), (4, 2, 128), (32, 8, 128), (40, 2, 32), (3, 3, 256), (4, 2, 192), (6, 3, 112),
+         (2, 1, 144), (2, 2, 240)]
 
 
 @pytest.mark.parametrize("nh,nkv,hd", HEADS)
@@ -240,6 +243,9 @@ def test_attention_mfma_finds_a_far_key_and_respects_the_window_edge(ops):
         for L, at in ((700, 13), (700, 0), (700, 699), (513, 448), (64, 63), (65, 64), (129, 31)):
             got, v = _spike_case(ops, fn, BF16, L, at)
             assert torch.allclose(got, v[at, 0].float().expand(2, -1), atol=1e-2), (L, at)
+        for hd in (192, 112):
+            got, v = _spike_case(ops, fn, BF16, 200, 77, hd=hd)
+            assert torch.allclose(got, v[77, 0].float().expand(2, -1), atol=1e-2), hd
         L, w = 300, 70
         got, v = _spike_case(ops, fn, BF16, L, L - w, window=w)
         assert torch.allclose(got, v[L - w, 0].float().expand(2, -1), atol=1e-2)
