@@ -14,6 +14,23 @@ PALM_API int palm_attention_decode(hipStream_t stream, const void* q, const void
                                    int n_seqs, int nh, int nkv, int hd, float scale, int window, int n_slices,
                                    float* work, void* out);
 
+// The same computation for callers that cannot allocate: code under HIP graph capture, tight serving loops,
+// harnesses that forbid hipMalloc.  It has no counterpart in the reference (whose decode attention is a single
+// kernel without a workspace, engine/cuda_attention.cu).  It takes no workspace: the slices' partial results go
+// through a buffer that the library itself holds, a file-scope array in device memory of
+// palm_attention_decode_static_limit() floats (8 MiB), which every GPU the library runs on keeps until the
+// process ends.  The call allocates nothing, frees nothing and calls no allocating routine; it refuses
+// n_seqs * nh * n_slices * (hd + 4) beyond the limit with an error and launches nothing then.  All calls on one
+// GPU share that GPU's buffer, which keeps the last call's contents: nothing in it has to start at zero (every
+// slice, also an empty one, writes its whole record before the merge reads it), but two calls that overlap in
+// time on one GPU (different streams, or a graph replayed beside an eager call) race on it.  Calls on one stream,
+// one after the other, are safe.  The result is the same bits as palm_attention_decode's with the same slices.
+PALM_API int palm_attention_decode_static(hipStream_t stream, const void* q, const void* k_cache, const void* v_cache,
+                                          const int* block_table, int max_pages, const int* seq_slot,
+                                          const int* seq_start, int n_seqs, int nh, int nkv, int hd, float scale,
+                                          int window, int n_slices, void* out);
+PALM_API long long palm_attention_decode_static_limit();
+
 PALM_API int palm_attention_prefill(hipStream_t stream, const void* q, const void* k_cache, const void* v_cache,
                                     const int* block_table, int max_pages, const int* seq_slot, const int* seq_start,
                                     const int* seq_new, const int* cu_new, int n_seqs, int max_new, int nh, int nkv,

@@ -20,6 +20,8 @@
 //          merges the slices.  The kernel is bound by reading K and V once.
 // prefill: one block of four waves per (sequence, kv head, 16 query positions); wave w owns the columns
 //          of query head w of the group (more heads: more passes).
+#include <mutex>
+
 #include "mfma.h"
 #include "attention_api.h"
 
@@ -301,6 +303,59 @@ PALM_API int palm_attention_decode(hipStream_t stream, const void* q, const void
                                    const int* block_table, int max_pages, const int* seq_slot, const int* seq_start,
                                    int n_seqs, int nh, int nkv, int hd, float scale, int window, int n_slices,
                                    float* work, void* out) {
+    return launch_attention_decode(stream, q, k_cache, v_cache, block_table, max_pages, seq_slot, seq_start, n_seqs, nh, nkv,
+                                   hd, scale, window, n_slices, work, out);
+}
+
+// ---- decode without a workspace argument ------------------------------------------------------------
+// The slices' partial results go through this array instead of a buffer of the caller's.  Each GPU has a copy of
+// its own at an address of its own; in host code the array's name is only a handle for hipGetSymbolAddress, never
+// a pointer to hand to a kernel.  The address is asked for once per device, with that device current, and kept.
+constexpr long long STATIC_WORK_FLOATS = 2ll * 1024 * 1024;            // 8 MiB
+static __device__ __align__(256) float scratch[STATIC_WORK_FLOATS];
+constexpr int STATIC_MAX_DEVICES = 64;
+static float* g_scratch_of_device[STATIC_MAX_DEVICES];                  // null until the device's first call
+static std::mutex g_scratch_lock;
+
+PALM_API long long palm_attention_decode_static_limit() { return STATIC_WORK_FLOATS; }
+
+// The current device's copy of the array (null and an error text on failure).
+static float* scratch_of_current_device() {
+    int device = -1;
+    hipError_t e = hipGetDevice(&device);
+    if (e != hipSuccess) { palm_fail("attention_decode_static: hipGetDevice failed: %s", hipGetErrorString(e)); return nullptr; }
+    if (device < 0 || device >= STATIC_MAX_DEVICES) {
+        palm_fail("attention_decode_static: device %d is beyond the %d this library keeps a buffer for", device, STATIC_MAX_DEVICES);
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> hold(g_scratch_lock);
+    if (!g_scratch_of_device[device]) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr) {
+            palm_fail("attention_decode_static: hipGetSymbolAddress failed on device %d: %s", device, hipGetErrorString(e));
+            return nullptr;
+        }
+        g_scratch_of_device[device] = static_cast<float*>(ptr);
+    }
+    return g_scratch_of_device[device];
+}
+
+PALM_API int palm_attention_decode_static(hipStream_t stream, const void* q, const void* k_cache, const void* v_cache,
+                                          const int* block_table, int max_pages, const int* seq_slot,
+                                          const int* seq_start, int n_seqs, int nh, int nkv, int hd, float scale,
+                                          int window, int n_slices, void* out) {
+    PALM_CHECK(n_seqs >= 0 && nh > 0 && n_slices >= 1, "attention_decode_static: seqs=%d heads=%d slices=%d", n_seqs, nh, n_slices);
+    const long long need = n_slices > 1 ? (long long)n_seqs * nh * n_slices * WORK_STRIDE : 0;
+    PALM_CHECK(need <= STATIC_WORK_FLOATS,
+               "attention_decode_static: %d sequences x %d heads x %d slices x %d floats = %lld floats exceed the library's "
+               "buffer of %lld; use fewer slices, or palm_attention_decode with a workspace of the caller's",
+               n_seqs, nh, n_slices, WORK_STRIDE, need, STATIC_WORK_FLOATS);
+    float* work = nullptr;
+    if (n_slices > 1) {
+        work = scratch_of_current_device();
+        if (!work) return -1;
+    }
     return launch_attention_decode(stream, q, k_cache, v_cache, block_table, max_pages, seq_slot, seq_start, n_seqs, nh, nkv,
                                    hd, scale, window, n_slices, work, out);
 }
