@@ -276,20 +276,3 @@ PALM_API int palm_swiglu(hipStream_t stream, const void* gate_up, int dtype, voi
     PALM_LAUNCHED();
     return 0;
 }
-
-// ---- casts ----------------------------------------------------------------------------------------
-template <typename TS, typename TD>
-__global__ void cast_kernel(const TS* __restrict__ src, TD* __restrict__ dst, size_t n) {
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
-        dst[i] = from_float<TD>(to_float(src[i]));
-}
-
-PALM_API int palm_cast(hipStream_t stream, const void* src, int src_dtype, void* dst, int dst_dtype, long long n) {
-    PALM_CHECK(n >= 0, "cast: n=%lld", n);
-    if (n == 0) return 0;
-    const int blocks = (int)((n + 255) / 256 < 65536 ? (n + 255) / 256 : 65536);
-    PALM_DTYPE_SWITCH(src_dtype, TS, PALM_DTYPE_SWITCH(dst_dtype, TD,
-        cast_kernel<TS, TD><<<blocks, 256, 0, stream>>>((const TS*)src, (TD*)dst, (size_t)n)));
-    PALM_LAUNCHED();
-    return 0;
-}

@@ -52,7 +52,11 @@ def replay(engine, lines, out_dir, report=print) -> None:
 
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(prog="trace_run", description="Replay token ids through a model and write logits.")
-    ap.add_argument("--model", required=True, help="folder with config.json and model.safetensors")
+    src = ap.add_mutually_exclusive_group(required=True)
+    src.add_argument("--model", help="folder with config.json and model.safetensors")
+    src.add_argument("--random", metavar="CONFIG", help="instead of --model: a config.json, or a named size (tiny-a, "
+                     "qwen3-8b, ..), filled on the device with the random-weights mode's numbers for --seed")
+    ap.add_argument("--seed", type=int, default=0, help="seed of --random (default 0)")
     ap.add_argument("--dtype", required=True, choices=["bfloat16", "float32"])
     ap.add_argument("--out", required=True, help="folder for <step>.f32 files")
     ap.add_argument("--max-tokens", type=int, required=True,
@@ -61,7 +65,11 @@ def main(argv=None) -> int:
     from ..cache import CacheFull
     from .engine import Engine
     try:
-        engine = Engine.from_dir(args.model, dtype=args.dtype, max_tokens=args.max_tokens)
+        if args.random:
+            from ..config import config_source
+            engine = Engine.from_config(config_source(args.random), seed=args.seed, dtype=args.dtype, max_tokens=args.max_tokens)
+        else:
+            engine = Engine.from_dir(args.model, dtype=args.dtype, max_tokens=args.max_tokens)
     except (ValueError, FileNotFoundError, RuntimeError) as e:
         print(f"trace_run: {type(e).__name__}: {e}", file=sys.stderr)
         return 1

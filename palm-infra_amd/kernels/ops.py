@@ -2,11 +2,12 @@
 
 Every function checks on the host what its kernel assumes (device, element types, contiguity, shapes
 that fit each other) before it launches anything, and launches on torch's current stream.  Tensors
-are only memory here: no torch operator computes on the product path.
+are memory here; the one computation that torch does on the product path is the library matrix product of
+``linear_library`` (bfloat16 products of more rows than the kernels here stream weights past).
 """
 from __future__ import annotations
 
-from ctypes import c_float, c_int, c_longlong, c_void_p
+from ctypes import c_float, c_int, c_longlong, c_ulonglong, c_void_p
 
 import torch
 
@@ -22,7 +23,8 @@ _SIGNATURES = {
     "palm_rmsnorm": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p, c_float, c_void_p, c_int, c_int,
                      c_void_p, c_int, c_int, c_longlong],
     "palm_swiglu": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int],
-    "palm_cast": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_longlong],
+    "palm_convert": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_longlong],
+    "palm_random_fill": [c_void_p, c_void_p, c_int, c_longlong, c_ulonglong, c_float, c_float],
     "palm_linear": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int],
     "palm_qk_norm_rope_store": [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                                 c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
@@ -154,13 +156,26 @@ def swiglu(gate_up: torch.Tensor) -> torch.Tensor:
     return out
 
 
-def cast(src: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
-    _dev("cast", src)
-    if src.dtype == dtype:
-        return src
-    out = torch.empty(src.shape, dtype=dtype, device=src.device)
-    library.call(core(), "palm_cast", _stream(), _p(src), _code(src, "cast"), _p(out), _code(out, "cast"), src.numel())
-    return out
+_STORED_CODES = {F32: 0, BF16: 1, torch.float16: 2, torch.float64: 3}
+
+
+def convert_into(src: torch.Tensor, dst: torch.Tensor) -> None:
+    """dst = src in dst's element type (float32 or bfloat16); src is as a checkpoint stores it (float32, bfloat16,
+    float16 or float64).  One rounding to nearest where dst is narrower.  dst may be a run of rows of a larger
+    tensor: what a checkpoint's tensors go through when they are joined into one parameter."""
+    _dev("convert", src, dst)
+    _need(src.dtype in _STORED_CODES, f"convert: a tensor stored as {src.dtype} is not float32, bfloat16, float16 or float64")
+    _need(src.numel() == dst.numel(), f"convert: {tuple(src.shape)} into {tuple(dst.shape)}")
+    library.call(core(), "palm_convert", _stream(), _p(src), _STORED_CODES[src.dtype], _p(dst), _code(dst, "convert dst"),
+                 src.numel())
+
+
+def random_fill(out: torch.Tensor, key: int, mean: float, std: float) -> None:
+    """out[i] = normal(key, i) * std + mean, the counter-based numbers of weights/random_numbers.py (same bits)."""
+    _dev("random_fill", out)
+    _need(0 <= int(key) < 1 << 64, "random_fill: the key is 64 bits")
+    library.call(core(), "palm_random_fill", _stream(), _p(out), _code(out, "random_fill out"), out.numel(), int(key),
+                 float(mean), float(std))
 
 
 # ---- linear ---------------------------------------------------------------------------------------

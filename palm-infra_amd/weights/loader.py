@@ -15,6 +15,8 @@ from __future__ import annotations
 import torch
 
 from ..config.spec import ModelSpec, TensorRef
+from ..kernels import ops
+from .random_numbers import tensor_key
 from .safetensors_io import ModelFiles
 
 _FLOAT_NAMES = ("F32", "F16", "BF16", "F64")
@@ -91,7 +93,15 @@ class Weights:
         return total
 
 
-def load_weights(spec: ModelSpec, files: ModelFiles, mode: torch.dtype, device) -> Weights:
+def _convert_on_device(stored: torch.Tensor, part: torch.Tensor) -> None:
+    """The file's bytes go up as they are stored; the conversion into the kept type and into the parameter's
+    rows is the device's (the reference converts and joins when it packs a model, models/qwen3.py:125-160)."""
+    ops.convert_into(stored.to(part.device), part)
+
+
+def load_weights(spec: ModelSpec, files: ModelFiles, mode: torch.dtype, device, place=_convert_on_device) -> Weights:
+    """``place(stored tensor of the file, rows of the parameter)`` puts a checkpoint tensor where it belongs; the
+    default converts on the device.  (Tests of the binding alone, which run without a GPU, hand in a stand-in.)"""
     names = files.names()
     check_names(spec, {n: files.shape(n) for n in names}, {n: files.dtype_name(n) for n in names},
                 where=str(files.files[0].path.parent))
@@ -101,26 +111,37 @@ def load_weights(spec: ModelSpec, files: ModelFiles, mode: torch.dtype, device) 
         dst = torch.empty(ref.shape, dtype=dt, device=device)
         row = 0
         for name, shape in zip(ref.names, ref.shapes):
-            dst[row:row + shape[0]].copy_(files.tensor(name))
-            row += shape[0]
+            part = dst[row:row + shape[0]] if shape else dst
+            if ref.role == "integer":
+                part.copy_(files.tensor(name).to(torch.int32))
+            else:
+                place(files.tensor(name), part)
+            row += shape[0] if shape else 0
         out[ref.names] = dst
     return Weights(out)
 
 
 def random_weights(spec: ModelSpec, seed: int, mode: torch.dtype, device) -> Weights:
-    """Random parameters made on the device without a file (for measurements at sizes whose folder
-    would be tens of gigabytes).  Each tensor has a generator of its own, seeded by the seed and the
-    tensor's place in the model, so a parameter does not depend on the ones before it."""
+    """Random parameters made on the device without a file (for measurements at sizes whose folder would be
+    tens of gigabytes).  They are, bit for bit, what ``load_weights`` gives for the folder that
+    ``write_random_model(config, seed, folder, "bfloat16")`` writes: both take element i of checkpoint tensor
+    ``name`` from ``random_numbers``' function of (seed, name, i), rounded to bfloat16 as the folder stores it,
+    and kept as the mode keeps it (vectors, and everything in the float32 mode, widened to float32)."""
     out = {}
-    for i, ref in enumerate(spec.tensor_refs()):
+    for ref in spec.tensor_refs():
         dt = kept_dtype(ref, ["BF16"], mode)
-        g = torch.Generator(device=device)
-        g.manual_seed((int(seed) * 1000003 + i) & 0x7FFFFFFF)
-        if ref.role == "integer":
-            out[ref.names] = torch.zeros(ref.shape, dtype=dt, device=device)
-            continue
-        _, mean, std = ref.init
-        t = torch.empty(ref.shape, dtype=dt, device=device)
-        t.normal_(mean, std, generator=g)
-        out[ref.names] = t
+        dst = torch.zeros(ref.shape, dtype=dt, device=device)
+        row = 0
+        for name, shape in zip(ref.names, ref.shapes):
+            if ref.role != "integer":
+                _, mean, std = ref.init
+                part = dst[row:row + shape[0]] if shape else dst
+                if dt == torch.bfloat16:
+                    ops.random_fill(part, tensor_key(seed, name), mean, std)
+                else:
+                    stored = torch.empty(part.shape, dtype=torch.bfloat16, device=device)
+                    ops.random_fill(stored, tensor_key(seed, name), mean, std)
+                    ops.convert_into(stored, part)
+            row += shape[0] if shape else 0
+        out[ref.names] = dst
     return Weights(out)

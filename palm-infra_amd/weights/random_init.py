@@ -3,26 +3,22 @@ configuration and a seed.
 
 The reference has this only as a test fixture (tests/run_tiny_qwen3_cpu_e2e.py:52-95).  Here matrices
 and the embedding are N(0, 0.02) and norm weights 1 + N(0, 0.02), as each parameter's description
-says.  A tensor's values depend on the seed and on the tensor's name only, so a model with more layers
-starts with the same layers.
+says.  A tensor's values depend on the seed, on the tensor's name and on the element's index only
+(``random_numbers``), so a model with more layers starts with the same layers, and the folder written here
+holds the same numbers as ``loader.random_weights`` makes on the device.
 """
 from __future__ import annotations
 
-import hashlib
 import json
 from pathlib import Path
 
 import torch
 
 from ..config.registry import config_from_dict, config_source
+from .random_numbers import normal, tensor_key
 from .safetensors_io import write_safetensors
 
 _STORE = {"bfloat16": torch.bfloat16, "float32": torch.float32, "float16": torch.float16}
-
-
-def _tensor_seed(seed: int, name: str) -> int:
-    digest = hashlib.sha256(f"{int(seed)}:{name}".encode()).digest()
-    return int.from_bytes(digest[:8], "little") & 0x7FFFFFFFFFFFFFFF
 
 
 def random_tensors(spec, seed: int, dtype: str = "bfloat16") -> dict[str, torch.Tensor]:
@@ -34,10 +30,11 @@ def random_tensors(spec, seed: int, dtype: str = "bfloat16") -> dict[str, torch.
             if ref.role == "integer":
                 out[name] = torch.zeros(shape, dtype=torch.int32)
                 continue
-            g = torch.Generator()
-            g.manual_seed(_tensor_seed(seed, name))
             _, mean, std = ref.init
-            t = torch.empty(shape, dtype=torch.float32).normal_(mean, std, generator=g)
+            count = 1
+            for extent in shape:
+                count *= int(extent)
+            t = torch.from_numpy(normal(tensor_key(seed, name), count, mean, std)).reshape(shape)
             out[name] = t.to(_STORE[dtype])
     return out
 

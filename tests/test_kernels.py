@@ -160,10 +160,39 @@ def test_swiglu_of_bfloat16_rows_far_from_zero(ops):
     assert int(tiny_ones.sum()) >= 6
 
 
-def test_cast_rounds_to_nearest_even(ops):
-    x = torch.tensor([1.0, 1.00390625, 1.01171875, -3.1415927, 1e-40, 65504.0, float("inf")])
-    assert torch.equal(ops.cast(x.to(DEV), BF16).cpu(), x.to(BF16))
-    assert torch.equal(ops.cast(x.to(BF16).to(DEV), F32).cpu(), x.to(BF16).float())
+def test_conversion_at_load_rounds_to_nearest_even_from_every_stored_type(ops):
+    x = torch.tensor([1.0, 1.00390625, 1.01171875, -3.1415927, 1e-40, 65504.0, float("inf"), 0.3, -7.7e-3])
+    for stored in (F32, BF16, torch.float16, torch.float64):
+        src = x.to(stored)
+        for kept in (F32, BF16):
+            # into the middle rows of a larger tensor, as the loader joins q, k and v
+            dst = torch.full((3, x.numel()), 9.0, dtype=kept, device=DEV)
+            ops.convert_into(src.to(DEV), dst[1])
+            assert torch.equal(dst[1].cpu(), src.to(kept)), (stored, kept)
+            assert bool((dst[0] == 9.0).all()) and bool((dst[2] == 9.0).all())
+    with pytest.raises(Exception, match="stored as"):
+        ops.convert_into(torch.zeros(4, dtype=torch.int32, device=DEV), torch.zeros(4, dtype=F32, device=DEV))
+
+
+def test_random_fill_gives_the_host_function_s_bits(ops):
+    """The device kernel and weights/random_numbers.py are the same function of (key, index): float32 and
+    bfloat16, a count that is no multiple of anything, several keys, mean and scale as the model's tensors use."""
+    from palm_infra_amd.weights import random_numbers as R
+    for key, n, mean, std in ((R.tensor_key(0, "model.embed_tokens.weight"), 1_000_003, 0.0, 0.02),
+                              (R.tensor_key(7, "model.norm.weight"), 4099, 1.0, 0.02), ((1 << 64) - 1, 70_001, -3.0, 1.0),
+                              (0, 65, 0.0, 1.0)):
+        want = torch.from_numpy(R.normal(key, n, mean, std))
+        for dtype in (F32, BF16):
+            got = torch.empty(n, dtype=dtype, device=DEV)
+            ops.random_fill(got, key, mean, std)
+            assert torch.equal(got.cpu(), want.to(dtype)), (key, n, dtype, int((got.cpu() != want.to(dtype)).sum()))
+    # a window far into a long stream (what a large tensor's later rows are)
+    key = R.tensor_key(3, "model.layers.0.mlp.down_proj.weight")
+    n, first, count = 50_331_648, 50_000_000, 100_000
+    got = torch.empty(n, dtype=BF16, device=DEV)
+    ops.random_fill(got, key, 0.0, 0.02)
+    want = torch.from_numpy(R.standard_normal(key, first, count)) * torch.tensor(0.02) + torch.tensor(0.0)
+    assert torch.equal(got[first:first + count].cpu(), want.to(BF16))
 
 
 # ---- linear -------------------------------------------------------------------------------------

@@ -359,12 +359,15 @@ def test_another_norm_a_routed_feed_forward_and_another_position_encoding(model_
         h = c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + 1e-5) * extra[("toy.norm",)].double()
         if dtype == "bfloat16":
             h = h.to(torch.bfloat16).double()                   # the choice of expert is made from the rounded rows
-        choice = (h.float() @ extra[("toy.router",)].float().T).argmax(-1)
+        router_logits = h.float() @ extra[("toy.router",)].float().T
+        choice = router_logits.argmax(-1)
+        top2 = router_logits.topk(2, dim=-1).values
+        clear = (top2[:, 0] - top2[:, 1]) > 1.0                  # router logits are of order 8; bfloat16 moves them by tenths
         A = extra[("toy.a",)].double().reshape(E, I, H)
         B = extra[("toy.b",)].double().reshape(E, H, I)
         hid = torch.relu(torch.einsum("th,tih->ti", h, A[choice]))
         x = x + torch.einsum("ti,thi->th", hid, B[choice])
-        return P.linear(P.rms_norm(x, w["model.norm.weight"], S["eps"]), P.head_weight(w)), choice
+        return P.linear(P.rms_norm(x, w["model.norm.weight"], S["eps"]), P.head_weight(w)), choice, clear
 
     reqs = tiny.prompts("A", [45, 12, 70], seed=23)
     slots = [eng.open() for _ in reqs]
@@ -380,8 +383,15 @@ def test_another_norm_a_routed_feed_forward_and_another_position_encoding(model_
         for r_, i in enumerate(live):
             got[i].append(out[r_:r_ + 1]); fed[i] += 1
     for i in range(3):
-        ref, choice = plain(reqs[i])
+        ref, choice, clear = plain(reqs[i])
         assert len(set(choice.tolist())) > 1                     # the router does choose
-        tiny.assert_logits_close(torch.cat(got[i]), ref, dtype, f"toy norm, routing and rotation, request {i}")
+        rows = torch.cat(got[i])
+        if dtype == "bfloat16":
+            # A choice between two experts whose router logits nearly tie is not a rounding matter: the rounded
+            # run may take the other expert, and that row (the last layer's, so that row alone) is then another
+            # function.  Such rows are left out of the bfloat16 comparison; float32 compares every row.
+            assert int(clear.sum()) >= 0.7 * len(clear)
+            rows, ref = rows[clear.to(rows.device)], ref[clear]
+        tiny.assert_logits_close(rows, ref, dtype, f"toy norm, routing and rotation, request {i}")
         eng.close(slots[i])
     eng.cache.check()

@@ -12,6 +12,11 @@ from palm_infra_amd.weights import (ModelFiles, SafetensorsError, SafetensorsFil
                                     random_tensors, write_random_model, write_safetensors)
 
 
+def host_copy(stored, part):
+    """Stands in for the device's conversion kernel where only the binding is tested (no GPU here)."""
+    part.copy_(stored)
+
+
 def test_round_trip_is_bit_exact(tmp_path):
     g = torch.Generator().manual_seed(0)
     tensors = {"a": torch.randn(3, 5, generator=g), "b": torch.randn(7, generator=g).to(torch.bfloat16),
@@ -68,7 +73,7 @@ def test_one_error_lists_missing_unexpected_and_misshapen(tmp_path):
     cfg = config_from_dir(tmp_path)
     files = ModelFiles(tmp_path)
     with pytest.raises(WeightError) as e:
-        load_weights(cfg.spec(files.names()), files, torch.float32, "cpu")
+        load_weights(cfg.spec(files.names()), files, torch.float32, "cpu", place=host_copy)
     err = e.value
     assert sorted(err.missing) == ["model.layers.1.self_attn.k_proj.weight", "model.norm.weight"]
     assert sorted(err.unexpected) == ["model.layers.7.mlp.up_proj.weight", "rotary.inv_freq"]
@@ -87,7 +92,7 @@ def test_a_stored_head_is_used_whatever_the_config_says(tmp_path):
     write_safetensors(tmp_path / "model.safetensors", tensors)
     files = ModelFiles(tmp_path)
     spec = config_from_dir(tmp_path).spec(files.names())
-    w = load_weights(spec, files, torch.float32, "cpu")
+    w = load_weights(spec, files, torch.float32, "cpu", place=host_copy)
     assert torch.equal(w.get(spec.head.tensors["weight"]), tensors["lm_head.weight"])
     # and the other way round: the key says untied, the checkpoint has no head of its own
     d = tmp_path / "b"
@@ -97,7 +102,7 @@ def test_a_stored_head_is_used_whatever_the_config_says(tmp_path):
     write_safetensors(d / "model.safetensors", tensors)
     files = ModelFiles(d)
     spec = config_from_dir(d).spec(files.names())
-    w = load_weights(spec, files, torch.float32, "cpu")
+    w = load_weights(spec, files, torch.float32, "cpu", place=host_copy)
     assert w.get(spec.head.tensors["weight"]).data_ptr() == w.get(spec.embedding.tensors["table"]).data_ptr()
 
 
@@ -106,18 +111,18 @@ def test_what_is_kept_in_which_precision(tmp_path):
     d = tiny.write_model("B", tmp_path / "bf", "bfloat16")
     files = ModelFiles(d)
     spec = cfg.spec(files.names())
-    w = load_weights(spec, files, torch.bfloat16, "cpu")
+    w = load_weights(spec, files, torch.bfloat16, "cpu", place=host_copy)
     mixer = spec.layers[0].parts["mixer"]
     assert w.get(mixer.tensors["qkv"]).dtype == torch.bfloat16
     assert w.get(mixer.tensors["qkv"]).shape == (8 * 32 + 2 * 32, 96)
     assert w.get(mixer.parts["q_norm"].tensors["weight"]).dtype == torch.float32      # vectors are widened
     assert w.get(spec.embedding.tensors["table"]).dtype == torch.bfloat16
-    w32 = load_weights(spec, files, torch.float32, "cpu")
+    w32 = load_weights(spec, files, torch.float32, "cpu", place=host_copy)
     assert w32.get(mixer.tensors["qkv"]).dtype == torch.float32
     # a tensor stored in 32-bit stays so in the bfloat16 mode
     d32 = tiny.write_model("B", tmp_path / "f32", "float32")
     f32 = ModelFiles(d32)
-    wmix = load_weights(spec, f32, torch.bfloat16, "cpu")
+    wmix = load_weights(spec, f32, torch.bfloat16, "cpu", place=host_copy)
     assert wmix.get(mixer.tensors["qkv"]).dtype == torch.float32
     # the joined matrix is q rows, k rows, v rows
     q = f32.tensor("model.layers.0.self_attn.q_proj.weight")
@@ -130,7 +135,7 @@ def test_tied_head_is_the_embedding_itself(tmp_path):
     d = tiny.write_model("A", tmp_path / "a", "float32")
     files = ModelFiles(d)
     spec = config_from_dir(d).spec(files.names())
-    w = load_weights(spec, files, torch.float32, "cpu")
+    w = load_weights(spec, files, torch.float32, "cpu", place=host_copy)
     assert w.get(spec.head.tensors["weight"]).data_ptr() == w.get(spec.embedding.tensors["table"]).data_ptr()
 
 
@@ -162,10 +167,29 @@ def test_random_weights_mode_writes_a_loadable_folder(tmp_path):
     assert a.dtype_name(n) == "BF16"
     assert torch.equal(a.tensor(n).float(), b.tensor(n).float())            # the seed decides
     assert not torch.equal(a.tensor(n).float(), c.tensor(n).float())
-    load_weights(cfg.spec(a.names()), a, torch.bfloat16, "cpu")
+    load_weights(cfg.spec(a.names()), a, torch.bfloat16, "cpu", place=host_copy)
     t = random_tensors(cfg.spec(), 5, "float32")
     assert abs(float(t[n].std()) - 0.02) < 2e-3 and abs(float(t["model.norm.weight"].mean()) - 1.0) < 2e-2
     # a tensor depends on the seed and its name only: a model with fewer layers starts the same
     small = config_from_dict(dict(tiny.CONFIGS["B"], num_hidden_layers=1))
     assert torch.equal(random_tensors(small.spec(), 5, "float32")["model.layers.0.mlp.up_proj.weight"],
                        t["model.layers.0.mlp.up_proj.weight"])
+
+
+def test_random_numbers_are_a_function_of_seed_name_and_index():
+    from palm_infra_amd.weights import random_numbers as R
+    key = R.tensor_key(5, "model.layers.1.mlp.up_proj.weight")
+    assert key == R.tensor_key(5, "model.layers.1.mlp.up_proj.weight") and 0 <= key < 1 << 64
+    assert len({R.tensor_key(s, n) for s in (0, 1, 5) for n in ("a", "b", "model.layers.1.mlp.up_proj.weight")}) == 9
+    z = R.standard_normal(key, 0, 400_000)
+    # cutting the stream anywhere gives the same elements
+    assert (R.standard_normal(key, 1234, 1000) == z[1234:2234]).all()
+    assert (R.normal(key, 5000, 0.0, 1.0, chunk=777) == z[:5000]).all()
+    # standard normal: moments, tails, no correlation between neighbours or with another key's stream
+    import numpy as np
+    assert abs(float(z.mean())) < 6e-3 and abs(float(z.std()) - 1) < 5e-3
+    assert abs(float((z ** 4).mean()) - 3) < 0.1 and abs(float((np.abs(z) > 2).mean()) - 0.0455) < 2e-3
+    assert abs(float(np.corrcoef(z[:-1], z[1:])[0, 1])) < 6e-3
+    other = R.standard_normal(R.tensor_key(5, "model.layers.2.mlp.up_proj.weight"), 0, 400_000)
+    assert abs(float(np.corrcoef(z, other)[0, 1])) < 6e-3
+    assert np.isfinite(z).all() and float(np.abs(z).max()) < 6.0
