@@ -173,6 +173,89 @@ def test_scale_is_head_dim_not_hidden_over_heads():
     assert torch.allclose(got, P.linear(ref, w["model.layers.0.self_attn.o_proj.weight"]), atol=1e-10)
 
 
+def _attention_inputs(name="B", n=9, seed=0):
+    cfg, w = _model(name)
+    S = P.sizes(cfg)
+    ids = tiny.prompts(name, [n], seed=seed)[0]
+    x = P.embedding(w["model.embed_tokens.weight"], ids)
+    h = P.rms_norm(x, w["model.layers.0.input_layernorm.weight"], S["eps"])
+    return cfg, w, S, h
+
+
+def test_q_and_k_are_normed_before_they_are_rotated():
+    """models/qwen3.py:315-334: RMSNorm of q and k per head, then the rotation.  With a norm weight that differs
+    from element to element the two orders differ (the rotation mixes element i with i + half, which carry
+    different weights); with a constant weight they would not, which is why the weight is made uneven here."""
+    cfg, w, S, h = _attention_inputs("B")
+    a = "model.layers.0.self_attn."
+    hd, nh, nkv, n = S["hd"], S["nh"], S["nkv"], h.shape[0]
+    w[a + "q_norm.weight"] = torch.linspace(0.2, 3.0, hd, dtype=F64)
+    w[a + "k_norm.weight"] = torch.linspace(2.5, 0.3, hd, dtype=F64)
+    got = P.attention_block(h, w, a, S, list(range(n)))
+    q = P.linear(h, w[a + "q_proj.weight"]).reshape(n, nh, hd)
+    k = P.linear(h, w[a + "k_proj.weight"]).reshape(n, nkv, hd)
+    v = P.linear(h, w[a + "v_proj.weight"]).reshape(n, nkv, hd)
+    cos, sin = P.rope_table(list(range(n)), hd, S["theta"])
+
+    def finish(q, k):
+        return P.linear(P.causal_attention(q, k, v, hd ** -0.5).reshape(n, nh * hd), w[a + "o_proj.weight"])
+    norm_then_rotate = finish(P.rope_half_split(P.rms_norm(q, w[a + "q_norm.weight"], S["eps"]), cos, sin),
+                              P.rope_half_split(P.rms_norm(k, w[a + "k_norm.weight"], S["eps"]), cos, sin))
+    rotate_then_norm = finish(P.rms_norm(P.rope_half_split(q, cos, sin), w[a + "q_norm.weight"], S["eps"]),
+                              P.rms_norm(P.rope_half_split(k, cos, sin), w[a + "k_norm.weight"], S["eps"]))
+    assert torch.allclose(got, norm_then_rotate, atol=1e-12)
+    assert float((got - rotate_then_norm).abs().max()) > 1e-2 * float(got.abs().max())
+
+
+def test_one_q_norm_weight_serves_all_heads():
+    """The q norm's weight has head_dim elements and every head uses it (models/qwen3.py:315-324): so renumbering
+    the query heads of a kv group (rows of q_proj, columns of o_proj) changes nothing.  A weight of its own for
+    each head, or a norm over all heads together, would not commute with the renumbering."""
+    cfg, w, S, h = _attention_inputs("B")
+    a = "model.layers.0.self_attn."
+    hd, nh, n = S["hd"], S["nh"], h.shape[0]
+    w[a + "q_norm.weight"] = torch.linspace(0.2, 3.0, hd, dtype=F64)
+    before = P.attention_block(h, w, a, S, list(range(n)))
+    perm = torch.tensor([3, 0, 7, 1, 6, 2, 5, 4])                    # B has one kv head: all eight heads are one group
+    rows = (perm[:, None] * hd + torch.arange(hd)[None, :]).reshape(-1)
+    w2 = dict(w)
+    w2[a + "q_proj.weight"] = w[a + "q_proj.weight"][rows]
+    w2[a + "o_proj.weight"] = w[a + "o_proj.weight"][:, rows]
+    assert torch.allclose(P.attention_block(h, w2, a, S, list(range(n))), before, atol=1e-12)
+    # and the norm is over one head's elements, not over all heads: scaling one head's rows of q_proj changes nothing
+    w3 = dict(w)
+    w3[a + "q_proj.weight"] = w[a + "q_proj.weight"].clone()
+    w3[a + "q_proj.weight"][2 * hd:3 * hd] *= 7.0
+    # (up to eps, which weighs 49 times less beside the larger mean square)
+    assert torch.allclose(P.attention_block(h, w3, a, S, list(range(n))), before, atol=1e-4 * float(before.abs().max()))
+
+
+def test_the_q_and_k_norms_use_the_model_s_eps_and_v_is_not_normed():
+    """models/qwen3.py:315-324 hands rms_norm_eps to both head norms; v goes to the cache as it is."""
+    cfg, w, S, h = _attention_inputs("B")
+    a = "model.layers.0.self_attn."
+    hd, nh, nkv, n = S["hd"], S["nh"], S["nkv"], h.shape[0]
+    for key in ("q_proj.weight", "k_proj.weight"):
+        w[a + key] = w[a + key] * 1e-3                               # mean squares of the order of eps (1e-5): eps counts
+    got = P.attention_block(h, w, a, S, list(range(n)))
+    q = P.linear(h, w[a + "q_proj.weight"]).reshape(n, nh, hd)
+    k = P.linear(h, w[a + "k_proj.weight"]).reshape(n, nkv, hd)
+    v = P.linear(h, w[a + "v_proj.weight"]).reshape(n, nkv, hd)
+    cos, sin = P.rope_table(list(range(n)), hd, S["theta"])
+
+    def with_eps(eps):
+        qn = (q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + eps)) * w[a + "q_norm.weight"]
+        kn = (k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + eps)) * w[a + "k_norm.weight"]
+        o = P.causal_attention(P.rope_half_split(qn, cos, sin), P.rope_half_split(kn, cos, sin), v, hd ** -0.5)
+        return P.linear(o.reshape(n, nh * hd), w[a + "o_proj.weight"])
+    assert torch.allclose(got, with_eps(cfg["rms_norm_eps"]), atol=1e-12)
+    assert float((got - with_eps(1e-6)).abs().max()) > 1e-3 * float(got.abs().max())         # another eps shows
+    # v is used as it is: three times v gives three times the output (a normed v would give the same output)
+    w2 = dict(w)
+    w2[a + "v_proj.weight"] = w[a + "v_proj.weight"] * 3.0
+    assert torch.allclose(P.attention_block(h, w2, a, S, list(range(n))), 3.0 * got, atol=1e-10)
+
+
 def test_tied_and_untied_heads():
     cfg, w = _model("A")
     ids = [1, 2, 3]
