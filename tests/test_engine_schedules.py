@@ -234,3 +234,70 @@ def test_a_step_with_more_tokens_than_run_at_once_goes_through_in_pieces(model_d
     for s in slots:
         eng.close(s)
     eng.cache.check()
+
+
+@pytest.mark.parametrize("name,dtype", [(n, d) for n in ("A", "B") for d in ("float32", "bfloat16")])
+def test_a_mixed_step_of_running_sequences_a_fresh_prompt_and_a_continuation(model_dirs, name, dtype):
+    """One step that brings, side by side: two running sequences with one token each, a fresh prompt, and a
+    further piece of a prompt whose first piece an earlier step brought; then a second mixed step in which a
+    new sequence starts in the slot that a finished one gave back."""
+    from palm_infra_amd.engine import StepEntry
+    eng = engine_for(model_dirs, name, dtype)
+    r0, r1, r2, r3, r4 = tiny.prompts(name, [40, 23, 50, 70, 9], seed=33)
+    ref = [reference(model_dirs, name, dtype, r) for r in (r0, r1, r2, r3, r4)]
+    s0, s1, s2, s3 = (eng.open() for _ in range(4))
+    eng.step([StepEntry(s0, r0[:30], []), StepEntry(s1, r1[:10], []), StepEntry(s3, r3[:33], [])])
+    out = eng.step([StepEntry(s0, [r0[30]], [0]), StepEntry(s2, r2, list(range(50))), StepEntry(s1, [r1[10]], [0]),
+                    StepEntry(s3, r3[33:53], list(range(20)))])
+    assert out.shape[0] == 1 + 50 + 1 + 20
+    pool = tiny.LogitsPool(dtype, f"{name} {dtype} mixed steps")
+    pool.add(out[0:1], ref[0][30:31], "running sequence 0")
+    pool.add(out[1:51], ref[2], "fresh prompt among running sequences")
+    pool.add(out[51:52], ref[1][10:11], "running sequence 1")
+    pool.add(out[52:72], ref[3][33:53], "continuation piece")
+    eng.close(s2)
+    s4 = eng.open()
+    assert s4 == s2                                                 # the slot (and its pages) are used again
+    out = eng.step([StepEntry(s3, r3[53:], list(range(17))), StepEntry(s0, [r0[31]], [0]), StepEntry(s4, r4, [0, 8]),
+                    StepEntry(s1, [r1[11]], [0])])
+    pool.add(out[0:17], ref[3][53:], "last piece")
+    pool.add(out[17:18], ref[0][31:32], "running sequence 0, next token")
+    pool.add(out[18:20], ref[4][[0, 8]], "a new sequence in a slot given back")
+    pool.add(out[20:21], ref[1][11:12], "running sequence 1, next token")
+    pool.check()
+    assert [eng.length(s) for s in (s0, s1, s3, s4)] == [32, 12, 70, 9]
+    for s in (s0, s1, s3, s4):
+        eng.close(s)
+    eng.cache.check()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("n_seqs", [70, 130])
+def test_decode_steps_of_more_sequences_than_a_recorded_step_takes(model_dirs, dtype, n_seqs):
+    """70 and 130 sequences one token each: beyond the batch sizes that are recorded into graphs, so these are
+    plain launches with the products of more than 64 rows and an attention grid of more than 64 sequences.
+    Unequal lengths; some of the sequences end between the steps."""
+    from palm_infra_amd.engine import Engine, StepEntry
+    name = "B"
+    eng = Engine.from_dir(model_dirs[name][dtype], dtype=dtype, max_tokens=64 * 2 * n_seqs)
+    assert n_seqs > eng.GRAPH_MAX_BATCH
+    reqs = tiny.prompts(name, [4 + (11 * i) % 90 for i in range(n_seqs)], seed=34)
+    cfg, w = P.read_model(model_dirs[name][dtype])
+    refs = [P.logits(cfg, w, r) for r in reqs]
+    slots = [eng.open() for _ in reqs]
+    eng.step([StepEntry(s, r[:-3], []) for s, r in zip(slots, reqs)])
+    live = list(range(n_seqs))
+    pool = tiny.LogitsPool(dtype, f"{n_seqs} sequences a step")
+    for t in (3, 2, 1):
+        if t == 1:                                                  # 130 -> 87, 70 -> 65: still more than a recorded step takes
+            every = 3 if n_seqs == 130 else 14
+            gone, live = live[::every], [i for k, i in enumerate(live) if k % every]
+            for i in gone:
+                eng.close(slots[i])
+        got = eng.step([StepEntry(slots[i], [reqs[i][-t]], [0]) for i in live])
+        pool.add(got, torch.stack([refs[i][len(reqs[i]) - t] for i in live]), f"{len(live)} sequences, {t} before the end")
+    pool.check()
+    assert not eng._decode_graphs
+    for i in live:
+        eng.close(slots[i])
+    eng.cache.check()

@@ -29,18 +29,26 @@ def real_8b():
 
 def one_layer_of(size):
     from palm_infra_amd.config import config_from_dict, preset_dict
-    from palm_infra_amd.weights import random_tensors
+    from palm_infra_amd.weights import random_weights
     raw = dict(preset_dict(size), num_hidden_layers=1, vocab_size=3001, max_position_embeddings=4096)
     cfg = config_from_dict(raw)
     spec = cfg.spec()
     # values that bfloat16 holds exactly, so that both modes and the oracle start from the same numbers.  At this
     # width the usual spread already gives logits of order one; the q norm is four times larger, so that scores
     # are of order four and a wrong or missing key moves the logits by their own order
+    # (made on the device, whose numbers are the random-weights mode's: hundreds of millions of them take the host
+    # function half a minute)
+    made = random_weights(spec, 11, torch.bfloat16, "cuda:0")
     tensors = {}
-    for name, t in random_tensors(spec, 11, "float32").items():
-        if name.endswith("q_norm.weight"):
-            t = t * 4.0
-        tensors[name] = t.to(torch.bfloat16)
+    for ref in spec.tensor_refs():
+        row, joined = 0, made.get(ref).cpu()
+        for name, shape in zip(ref.names, ref.shapes):
+            t = joined[row:row + shape[0]].float()
+            row += shape[0]
+            if name.endswith("q_norm.weight"):
+                t = t * 4.0
+            tensors[name] = t.to(torch.bfloat16)
+    del made
     oracle = {k: v.double() for k, v in tensors.items()}
     g = torch.Generator().manual_seed(5)
     prompts = [torch.randint(0, raw["vocab_size"], (n,), generator=g).tolist() for n in LENGTHS]
@@ -135,3 +143,94 @@ def test_a_long_prompt_and_the_tokens_after_it(real_8b, dtype):
     got += [eng.step([StepEntry(s, [t], [0])]) for t in ids[2100:]]
     eng.close(s)
     tiny.assert_logits_close(torch.cat(got), ref[places + [2100, 2101, 2102]], dtype, "2,100-token prompt and three more tokens")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_mixed_step_at_large_sizes(real_8b, dtype):
+    """Two running sequences with one token each, a fresh prompt and a continuation piece in one step."""
+    from palm_infra_amd.engine import StepEntry
+    _, _, _, _, prompts, refs = real_8b
+    eng = engine_of(real_8b, dtype, pages=24)
+    r0, r1, r2, r3 = prompts                                   # 70, 5, 33, 300 tokens
+    s0, s1, s2, s3 = (eng.open() for _ in range(4))
+    eng.step([StepEntry(s0, r0[:60], []), StepEntry(s1, r1[:3], []), StepEntry(s3, r3[:130], [])])
+    out = eng.step([StepEntry(s0, [r0[60]], [0]), StepEntry(s2, r2, list(range(33))), StepEntry(s1, [r1[3]], [0]),
+                    StepEntry(s3, r3[130:250], list(range(120)))])
+    pool = tiny.LogitsPool(dtype, "mixed step at large sizes")
+    pool.add(out[0:1], refs[0][60:61], "running sequence")
+    pool.add(out[1:34], refs[2], "fresh prompt")
+    pool.add(out[34:35], refs[1][3:4], "short running sequence")
+    pool.add(out[35:155], refs[3][130:250], "continuation piece")
+    out = eng.step([StepEntry(s3, r3[250:], [0, 49]), StepEntry(s0, [r0[61]], [0]), StepEntry(s1, [r1[4]], [0])])
+    pool.add(out[0:2], refs[3][[250, 299]], "last piece")
+    pool.add(out[2:3], refs[0][61:62])
+    pool.add(out[3:4], refs[1][4:5])
+    pool.check()
+    for s in (s0, s1, s2, s3):
+        eng.close(s)
+    eng.cache.check()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_steps_of_70_and_130_sequences_at_large_sizes(real_8b, dtype):
+    """Beyond the batch sizes that are recorded: plain launches, library products of 70 and 130 rows, decode
+    attention over more than 64 sequences."""
+    from palm_infra_amd.engine import StepEntry
+    raw = real_8b[0]
+    eng = engine_of(real_8b, dtype, pages=140)
+    oracle = {k: v.double() for k, v in real_8b[3].items()}
+    g = torch.Generator().manual_seed(16)
+    seqs = [torch.randint(0, raw["vocab_size"], (3 + b % 5,), generator=g).tolist() for b in range(130)]
+    refs = [P.logits(raw, oracle, ids) for ids in seqs]
+    slots = [eng.open() for _ in seqs]
+    eng.step([StepEntry(s, ids[:-2], []) for s, ids in zip(slots, seqs)])
+    live = list(range(130))
+    pool = tiny.LogitsPool(dtype, "decode steps of 130 and 70 sequences")
+    for t in (2, 1):
+        if t == 1:
+            for b in live[70:]:
+                eng.close(slots[b])
+            live = live[:70]
+        got = eng.step([StepEntry(slots[b], [seqs[b][-t]], [0]) for b in live])
+        pool.add(got, torch.stack([refs[b][len(seqs[b]) - t] for b in live]), f"{len(live)} sequences")
+    pool.check()
+    assert not eng._decode_graphs
+    for b in live:
+        eng.close(slots[b])
+    eng.cache.check()
+
+
+@pytest.fixture(scope="module")
+def long_sequence(real_8b):
+    """9,000 tokens and the plain logits at the places the test asks for (the float64 attention of 32 heads over
+    9,000 x 9,000 scores takes most of a minute: made once for both precisions)."""
+    raw = real_8b[0]
+    oracle = {k: v.double() for k, v in real_8b[3].items()}
+    ids = torch.randint(0, raw["vocab_size"], (9000,), generator=torch.Generator().manual_seed(17)).tolist()
+    places = [0, 63, 64, 4095, 4096, 8189] + list(range(8190, 8200)) + [8999]
+    S = P.sizes(raw)
+    n = len(ids)
+    x = P.embedding(oracle["model.embed_tokens.weight"], ids)
+    x = P.decoder_layer(x, oracle, 0, S, list(range(n)))
+    ref = P.linear(P.rms_norm(x[places], oracle["model.norm.weight"], S["eps"]), P.head_weight(oracle))
+    return ids, places, ref
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_sequence_that_grows_across_8192_tokens(real_8b, long_sequence, dtype):
+    """8,190 tokens in one step (logits at a handful of places), then ten tokens one by one across the edge at
+    8,192 where the recorded step's length bucket and the cut of the key range into slices change, then the
+    rest of the 9,000 in one piece."""
+    from palm_infra_amd.engine import StepEntry
+    ids, places, ref = long_sequence
+    eng = engine_of(real_8b, dtype, pages=144)
+    s = eng.open()
+    first = [p for p in places if p < 8190]
+    got = [eng.step([StepEntry(s, ids[:8190], first)])]
+    for t in range(8190, 8200):
+        got.append(eng.step([StepEntry(s, [ids[t]], [0])]))
+    got.append(eng.step([StepEntry(s, ids[8200:], [799])]))
+    assert eng.length(s) == 9000
+    tiny.assert_logits_close(torch.cat(got), ref, dtype, "9,000 tokens")
+    eng.close(s)
+    eng.cache.check()
