@@ -26,7 +26,7 @@ if ROOT not in sys.path:
 PEAK_HBM_GBS = 8000.0
 PEAK_FLOPS = {"bf16": 2.5e15, "fp16": 2.5e15, "fp8": 5.0e15, "fp32": 157.3e12}
 
-# BASELINE.json configs[2]: Qwen3-8B sizes, kept as data beside the configuration code
+# the measured configuration: Qwen3-8B sizes, kept as data beside the configuration code
 from palm_infra_amd.config import preset_dict  # noqa: E402
 
 QWEN3_8B = preset_dict("qwen3-8b")

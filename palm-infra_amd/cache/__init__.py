@@ -1,6 +1,7 @@
 """Slots, pages, key/value groups and per-sequence state."""
 from .pool import PAGE_TOKENS, CacheFull, CacheMisuse, FreeList, PageTable, pages_for
-from .cache import KVGroup, KVNeed, LayerCache, ModelCache, StateGroup, StateNeed
+from .cache import (KVGroup, KVNeed, LayerCache, ModelCache, PagedGroup, RowsGroup, RowsNeed, RowsView, StateGroup,
+                    StateNeed)
 
 __all__ = ["PAGE_TOKENS", "CacheFull", "CacheMisuse", "FreeList", "PageTable", "pages_for", "KVGroup", "KVNeed",
-           "LayerCache", "ModelCache", "StateGroup", "StateNeed"]
+           "LayerCache", "ModelCache", "PagedGroup", "RowsGroup", "RowsNeed", "RowsView", "StateGroup", "StateNeed"]

@@ -17,7 +17,7 @@ import torch
 from ..cache import ModelCache
 from ..config import config_from_dict, config_from_dir
 from ..kernels import profile
-from ..parts import make_context
+from ..parts import context_ints, make_context
 from ..weights import ModelFiles, load_weights, random_weights
 from .model import DecoderModel
 
@@ -62,9 +62,10 @@ class Engine:
         self.cache = ModelCache(needs, shares, max_tokens, max_seqs, spec.max_positions, dtype, self.device)
         self.vocab_size = spec.vocab_size
         self.graphs_enabled = bool(graphs)
-        self._decode_graphs: dict = {}
+        self._decode_graphs: dict = {}            # (batch bucket, length bucket) -> recorded step, least recently used first
+        self._graph_pool_handle = None
         # a windowed group gives pages back only between steps, so long prompts go through it in pieces
-        windows = [g.need.window for g in self.cache.kv_groups if g.need.window]
+        windows = [g.need.window for g in self.cache.paged_groups if g.need.window]
         self.step_tokens_per_seq = max(1024, 2 * max(windows)) if windows else None
         # the most tokens that run through the layers at once: longer steps go through in pieces, so that a step's
         # activations (the widest: tokens x twice the feed-forward width) stay within a few gigabytes
@@ -187,8 +188,9 @@ class Engine:
         return (self.graphs_enabled and self.model.capturable and len(entries) <= self.GRAPH_MAX_BATCH
                 and all(len(e.tokens) == 1 for e in entries) and profile.active() is None)
 
+    GRAPH_LIMIT = 24        # recorded steps kept at once; the least recently used one goes when another is recorded
+
     def _run_decode_graph(self, entries) -> torch.Tensor:
-        from ..parts import StepContext
         cache = self.cache
         growth = [(e.slot, 1) for e in entries]
         cache.reserve(growth)
@@ -197,32 +199,27 @@ class Engine:
         Bb = self._batch_bucket(B)
         key = (Bb, self._length_bucket(max(starts) + 1))
         pad = Bb - B
-        slots = [e.slot for e in entries] + [cache.pad_slot] * pad
-        meta = ([int(e.tokens[0]) for e in entries] + [0] * pad + starts + [0] * pad + slots     # ids, positions, slots
-                + starts + [0] * pad + [1] * Bb + list(range(Bb + 1)))                           # starts, counts, offsets
-        state = self._decode_graphs.get(key)
+        state = self._decode_graphs.pop(key, None)
         if state is None:
-            buf = torch.zeros((len(meta),), dtype=torch.int32, device=self.device)
-            v = [buf[i * Bb:(i + 1) * Bb] for i in range(5)]
-            ctx = StepContext(n_tokens=Bb, n_seqs=Bb, max_new=1, max_total=key[1], dtype=self.dtype, token_ids=v[0],
-                              positions=v[1], tok_slot=v[2], seq_slot=v[2], seq_start=v[3], seq_new=v[4],
-                              cu_new=buf[5 * Bb:], is_decode=True)
-            state = self._decode_graphs[key] = {"buf": buf, "ctx": ctx, "rows": None, "graph": None, "logits": None,
-                                                "calls": 0}
-        state["buf"].copy_(torch.tensor(meta, dtype=torch.int32))
-        ctx = state["ctx"]
-        ctx.host = {"slots": slots, "starts": starts + [0] * pad, "counts": [1] * Bb, "cu": list(range(Bb + 1))}
+            while len(self._decode_graphs) >= self.GRAPH_LIMIT:          # a graph holds its activations and logits: bound them
+                self._decode_graphs.pop(next(iter(self._decode_graphs)))
+            state = {"buf": torch.zeros((context_ints(Bb, Bb),), dtype=torch.int32, device=self.device), "graph": None,
+                     "logits": None, "calls": 0}
+        self._decode_graphs[key] = state                                 # (re)inserted last: the most recently used
+        # the step's arrays, laid out as for any step, at the addresses the recording reads; rows that pad the batch
+        # belong to a slot of their own whose page is never read
+        ctx = make_context([e.slot for e in entries] + [cache.pad_slot] * pad, starts + [0] * pad,
+                           [[int(e.tokens[0])] for e in entries] + [[0]] * pad, self.dtype, self.device,
+                           max_total=key[1], into=state["buf"])
         if state["graph"] is None and state["calls"] == 0:
             # the first step of a shape runs as it is (and loads or builds whatever it needs)
-            ctx.memo = {}
-            logits = self.model.forward(ctx, cache, state["rows"])
+            logits = self.model.forward(ctx, cache, None)
         else:
             if state["graph"] is None:
-                ctx.memo = {}
                 torch.cuda.synchronize()
                 graph = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(graph):
-                    state["logits"] = self.model.forward(ctx, cache, state["rows"])
+                with torch.cuda.graph(graph, pool=self._graph_pool()):
+                    state["logits"] = self.model.forward(ctx, cache, None)
                 state["graph"] = graph
             state["graph"].replay()
             logits = state["logits"].clone()        # the graph's own buffer is overwritten by the next replay
@@ -232,6 +229,13 @@ class Engine:
         if len(wanted) == B:
             return logits[:B]
         return logits[torch.tensor(wanted, dtype=torch.long, device=self.device)] if wanted else logits[:0]
+
+    def _graph_pool(self):
+        """One memory pool for all recorded steps: replays never overlap (one stream, one at a time), so their
+        activations may share memory, and a dropped recording's memory serves the next."""
+        if self._graph_pool_handle is None:
+            self._graph_pool_handle = torch.cuda.graph_pool_handle()
+        return self._graph_pool_handle
 
     def _run(self, entries) -> torch.Tensor:
         recorder = profile.active()

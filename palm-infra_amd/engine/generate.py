@@ -110,14 +110,18 @@ def generate(engine, sampler, prompts, max_new_tokens: int = 2048, stop_token_id
     stop = set(int(t) for t in stop_token_ids)
     max_seq = engine.cache.max_seq_tokens
     results = [GenerationResult(prompt_tokens=len(p)) for p in prompts]
+    # a batch holds no more sequences than the cache has slots for
+    max_batch = min(max_batch, getattr(engine.cache, "max_seqs", max_batch))
     batches = plan_batches([len(p) for p in prompts], max_new_tokens, max_batch, engine.cache.max_tokens, max_seq)
     sync = sync or (lambda: None)
     total_prefill = total_decode = 0.0
 
     for batch in batches:
-        slots = {i: engine.open() for i in batch}
+        slots = {}
         states = {i: SequenceSampling(stream=i) for i in batch}
         try:
+            for i in batch:                  # one by one inside the try: if a slot cannot be had, those taken go back
+                slots[i] = engine.open()
             # ---- all prompts in one step; it yields each request's first token ----
             sync()
             t0 = timer()

@@ -99,8 +99,17 @@ class StepContext:
     host: dict = field(default_factory=dict)   # the same facts as Python lists, for parts that plan on the host
 
 
-def make_context(slots, starts, new_tokens, dtype, device, max_total=None) -> StepContext:
-    """A context from host lists: ``new_tokens[b]`` is the list of token ids of sequence b."""
+def context_ints(n_tokens: int, n_seqs: int) -> int:
+    """How many int32 a step's index arrays take together."""
+    return 3 * n_tokens + 4 * n_seqs + 1
+
+
+def make_context(slots, starts, new_tokens, dtype, device, max_total=None, into: torch.Tensor | None = None) -> StepContext:
+    """A context from host lists: ``new_tokens[b]`` is the list of token ids of sequence b.  This is the one place
+    where a step's arrays are laid out: a part that needs one more of them finds it here.
+
+    ``into``: an int32 device buffer of ``context_ints(n, B)`` elements to lay the arrays in instead of a new
+    one: a recorded step keeps its arrays at fixed addresses and gets new contents before every replay."""
     counts = [len(t) for t in new_tokens]
     ids = [t for seq in new_tokens for t in seq]
     pos = [starts[b] + j for b in range(len(slots)) for j in range(counts[b])]
@@ -110,7 +119,14 @@ def make_context(slots, starts, new_tokens, dtype, device, max_total=None) -> St
         cu.append(cu[-1] + c)
     n, B = len(ids), len(slots)
     # one transfer for all index arrays
-    flat = torch.tensor(ids + pos + tslot + list(slots) + list(starts) + counts + cu, dtype=torch.int32).to(device)
+    host = torch.tensor(ids + pos + tslot + list(slots) + list(starts) + counts + cu, dtype=torch.int32)
+    if into is None:
+        flat = host.to(device)
+    else:
+        if into.shape != host.shape or into.dtype != torch.int32:
+            raise ValueError(f"a step of {n} tokens in {B} sequences needs {host.numel()} int32, the buffer has {tuple(into.shape)}")
+        flat = into
+        flat.copy_(host)
     o = 0
     parts = []
     for size in (n, n, n, B, B, B, B + 1):

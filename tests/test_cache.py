@@ -174,3 +174,71 @@ def test_random_traffic_keeps_the_books():
         c.close(s)
     c.check()
     assert all(g.table.pages.free_count == g.n_pages for g in c.kv_groups) and c.slots.free_count == 9
+
+
+def test_rows_of_a_part_s_own_shape_grow_in_pages_beside_keys_and_values():
+    from palm_infra_amd.cache import RowsGroup, RowsNeed
+    needs = [[KVNeed(2, 16)], [RowsNeed("latent", (24,), dtype="float32")], [RowsNeed("latent", (24,), dtype="float32"), StateNeed("s", (3,))],
+             [RowsNeed("codes", (2, 5), dtype="int32", window=70)]]
+    c = _cache(needs)
+    rows = [g for g in c.groups if isinstance(g, RowsGroup)]
+    assert len(rows) == 2 and len(c.kv_groups) == 1 and len(c.paged_groups) == 3 and len(c.state_groups) == 1
+    latent, codes = rows
+    assert latent.data.shape == (2, 13, PAGE_TOKENS, 24) and latent.data.dtype == torch.float32       # two entries share the group
+    assert codes.data.shape == (1, 13, PAGE_TOKENS, 2, 5) and codes.data.dtype == torch.int32
+    lc = c.layer_caches
+    assert lc[1].rows["latent"].data.data_ptr() != lc[2].rows["latent"].data.data_ptr() and lc[1].kv is None
+    assert lc[1].rows["latent"].table_dev is latent.table_dev and "s" in lc[2].states
+    s = c.open()
+    c.reserve([(s, 200)]); c.commit([(s, 200)])
+    assert latent.table.slot_pages[s] == [0, 1, 2, 3] and codes.table.slot_pages[s] == [-1, -1, 2, 3]     # the window gave two back
+    assert latent.table_dev[s, :4].tolist() == [0, 1, 2, 3]
+    c.check()
+    c.close(s)
+    assert all(g.table.pages.free_count == g.n_pages for g in c.paged_groups)
+    with pytest.raises(ValueError, match="twice for rows named"):
+        _cache([[RowsNeed("x", (4,)), RowsNeed("x", (4,), dtype="float32")]])
+
+
+def test_a_need_of_a_kind_the_cache_has_never_heard_of():
+    """The cache asks a need how it is stored and asks the group how it shows itself to its part: a kind of
+    storage defined here, outside the package, is grouped, opened and handed to its entries like the others."""
+    from dataclasses import dataclass
+
+    class CounterGroup:
+        table = None
+
+        def __init__(self, need, n_entries, n_slots):
+            self.need, self.n_entries = need, n_entries
+            self.data = torch.zeros((n_entries, n_slots + 1), dtype=torch.int64)
+            self.opened = []
+
+        def sync(self):
+            pass
+
+        def on_open(self, slot):
+            self.opened.append(slot)
+            self.data[:, slot] = self.need.start
+
+        def nbytes(self):
+            return self.data.numel() * 8
+
+        def attach(self, layer_cache, entry):
+            layer_cache.states = layer_cache.states or {}
+            layer_cache.states["counter"] = self.data[entry]
+
+    @dataclass(frozen=True)
+    class CounterNeed:
+        start: int
+
+        def make_group(self, n_entries, n_pages, n_slots, max_pages_per_slot, dtype, device):
+            return CounterGroup(self, n_entries, n_slots)
+
+    c = _cache([[KVNeed(2, 16), CounterNeed(7)], [CounterNeed(7)], [CounterNeed(9)]])
+    mine = [g for g in c.groups if isinstance(g, CounterGroup)]
+    assert [g.n_entries for g in mine] == [2, 1]
+    s = c.open()
+    assert mine[0].opened == [s] and int(c.layer_caches[1].states["counter"][s]) == 7 and int(c.layer_caches[2].states["counter"][s]) == 9
+    assert c.nbytes() >= sum(g.nbytes() for g in mine)
+    c.reserve([(s, 100)]); c.commit([(s, 100)])
+    c.check()

@@ -118,3 +118,44 @@ def test_replays_of_steps_with_17_to_64_sequences(model_dirs, name):
         g.close(sg[i]); e.close(se[i])
     g.cache.check(); e.cache.check()
     assert sum(st["graph"] is not None for st in g._decode_graphs.values()) >= 4
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_sequences_that_grow_across_length_buckets_and_few_recordings_are_kept(model_dirs, dtype):
+    """Recorded steps are keyed by the longest sequence rounded up to a power of two (256, 512, 1,024): three
+    sequences grow from under 256 to over 512 tokens, every step checked against plain launches and pooled
+    against the plain implementation; and an engine keeps no more recordings than its limit, dropping the one
+    used longest ago."""
+    import plain_qwen3 as P
+    from palm_infra_amd.engine import Engine, StepEntry
+    name = "C"
+    g = Engine.from_dir(model_dirs[name][dtype], dtype=dtype, max_tokens=64 * 40, graphs=True)
+    e = Engine.from_dir(model_dirs[name][dtype], dtype=dtype, max_tokens=64 * 40, graphs=False)
+    g.GRAPH_LIMIT = 2
+    reqs = tiny.prompts(name, [530, 300, 270], seed=35)
+    starts = [245, 100, 5]
+    cfg, w = P.read_model(model_dirs[name][dtype])
+    refs = [P.logits(cfg, w, r) for r in reqs]
+    sg, se = [g.open() for _ in reqs], [e.open() for _ in reqs]
+    for eng, slots in ((g, sg), (e, se)):
+        eng.step([StepEntry(s, r[:c], []) for s, r, c in zip(slots, reqs, starts)])
+    pool = tiny.LogitsPool(dtype, "growing across length buckets")
+    fed = list(starts)
+    seen = set()
+    for t in range(285):
+        live = [i for i in range(3) if fed[i] < len(reqs[i])]
+        a = g.step([StepEntry(sg[i], [reqs[i][fed[i]]], [0]) for i in live])
+        b = e.step([StepEntry(se[i], [reqs[i][fed[i]]], [0]) for i in live])
+        seen |= set(g._decode_graphs)
+        assert len(g._decode_graphs) <= 2
+        if dtype == "float32":
+            assert torch.equal(a, b), t
+        if t % 9 == 0 or 8 <= t <= 14 or 262 <= t <= 270:            # around the edges at 256 and 512, and now and then
+            pool.add(a, torch.stack([refs[i][fed[i]] for i in live]), f"step {t}")
+        for i in live:
+            fed[i] += 1
+    pool.check()
+    assert {k[1] for k in seen} == {256, 512, 1024} and len(seen) >= 4      # more shapes than are kept at once
+    for i in range(3):
+        g.close(sg[i]); e.close(se[i])
+    g.cache.check()

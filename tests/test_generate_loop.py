@@ -168,3 +168,26 @@ def test_a_conversation_feeds_only_what_is_new_and_keeps_its_slot():
     full = talk.say([1] * 62, max_new_tokens=50)
     assert full.finish_reason == "context" and talk.length == 64 and len(full.token_ids) == 3
     talk.reset()
+
+
+def test_a_batch_holds_no_more_sequences_than_the_cache_has_slots_and_a_refused_slot_leaks_none():
+    eng = ScriptedEngine(lambda seen: 1, n_slots=3)
+    eng.cache.max_seqs = 3
+    results, _ = generate(eng, ArgmaxSampler(), [[1], [2], [3], [4], [5]], max_new_tokens=2, max_batch=8)
+    assert [len(r.token_ids) for r in results] == [2] * 5
+    assert len(eng.steps[0]) == 3 and max(len(s) for s in eng.steps) == 3          # batches of three, then two
+    assert not eng.seen and len(eng.free) == 3
+
+    # an engine that runs out of slots part-way (its cache does not say how many it has): those taken go back
+    class NoSlots(RuntimeError):
+        pass
+
+    class Short(ScriptedEngine):
+        def open(self):
+            if not self.free:
+                raise NoSlots("no free slot")
+            return super().open()
+    eng = Short(lambda seen: 1, n_slots=2)
+    with pytest.raises(NoSlots):
+        generate(eng, ArgmaxSampler(), [[1], [2], [3]], max_new_tokens=2, max_batch=8)
+    assert not eng.seen and sorted(eng.free) == [0, 1] and not eng.steps

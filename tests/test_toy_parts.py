@@ -395,3 +395,112 @@ def test_another_norm_a_routed_feed_forward_and_another_position_encoding(model_
         tiny.assert_logits_close(rows, ref, dtype, f"toy norm, routing and rotation, request {i}")
         eng.close(slots[i])
     eng.cache.check()
+
+
+# ---- a mixer whose growing store is not keys and values ----------------------------------------------
+
+def register_latent_mixer():
+    from palm_infra_amd.cache import PAGE_TOKENS, RowsNeed
+    from palm_infra_amd.parts import register_part
+
+    @register_part("mixer", "toy_latent")
+    class LatentMixer:
+        """Keeps one latent row c_t = h_t W_in^T (24 wide, float32) for every position and attends over them:
+        out_t = sum_{j <= t} softmax_j(c_t . c_j / sqrt(width)) c_j W_out^T.  Its store grows with the sequence
+        but has neither heads nor separate values: it asks the cache for rows of its own shape."""
+
+        def __init__(self, spec, builder):
+            self.w_in, self.w_out = builder.tensor(spec, "w_in"), builder.tensor(spec, "w_out")
+            self.width, self.dtype = int(spec.params["width"]), builder.dtype
+
+        @staticmethod
+        def cache_needs(spec):
+            return [RowsNeed("latent", (int(spec.params["width"]),), dtype="float32")]
+
+        def forward(self, h, ctx):
+            view = ctx.layer_cache.rows["latent"]                      # data [pages + 1, 64, width], table_dev [slots + 1, pages]
+            c = h.float() @ self.w_in.float().T
+            out = torch.empty_like(c)
+            for b, (slot, start, n) in enumerate(zip(ctx.host["slots"], ctx.host["starts"], ctx.host["counts"])):
+                r0 = ctx.host["cu"][b]
+                pos = torch.arange(start, start + n, device=c.device)
+                pages = view.table_dev[slot].long()
+                view.data[pages[pos // PAGE_TOKENS], pos % PAGE_TOKENS] = c[r0:r0 + n]
+                every = torch.arange(0, start + n, device=c.device)
+                held = view.data[pages[every // PAGE_TOKENS], every % PAGE_TOKENS]          # [start + n, width], from the cache
+                s = (c[r0:r0 + n] @ held.T) * self.width ** -0.5
+                s = s.masked_fill(every[None, :] > pos[:, None], float("-inf"))
+                out[r0:r0 + n] = torch.softmax(s, dim=-1) @ held
+            return (out @ self.w_out.float().T).to(self.dtype)
+    return LatentMixer
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_mixer_that_keeps_one_latent_row_for_each_position(model_dirs, dtype):
+    """The cache gives a part growing storage of the part's own row shape (here 24 floats a position) with pages,
+    a page table and slots handled as for keys and values: registered, built and stepped from here."""
+    from palm_infra_amd.cache import RowsGroup
+    from palm_infra_amd.config import PartSpec, config_from_dir, tensor
+    from palm_infra_amd.engine import Engine, StepEntry
+    from palm_infra_amd.weights import ModelFiles, load_weights
+    register_latent_mixer()
+    d = model_dirs["A"][dtype]
+    tdt = torch.float32 if dtype == "float32" else torch.bfloat16
+    config, files = config_from_dir(d), ModelFiles(d)
+    base = config.spec(files.names())
+    H, width = base.hidden_size, 24
+    layer = base.layers[1]
+    toy = PartSpec("mixer", "toy_latent", {"width": width},
+                   {"w_in": tensor("toy.w_in", (width, H)), "w_out": tensor("toy.w_out", (H, width))})
+    spec = dataclasses.replace(base, layers=(base.layers[0], dataclasses.replace(layer, parts=dict(layer.parts, mixer=toy))))
+    g = torch.Generator().manual_seed(4)
+    w_in = (torch.randn(width, H, generator=g) * 0.5).to(tdt)
+    w_out = (torch.randn(H, width, generator=g) * 0.3).to(tdt)
+    weights = ExtraWeights(load_weights(base, files, tdt, DEV), {("toy.w_in",): w_in.to(DEV), ("toy.w_out",): w_out.to(DEV)})
+    eng = Engine(config, spec, weights, tdt, max_tokens=64 * 6)
+    rows_groups = [g_ for g_ in eng.cache.groups if isinstance(g_, RowsGroup)]
+    assert len(rows_groups) == 1 and rows_groups[0].data.shape == (1, 7, 64, width) and rows_groups[0].data.dtype == torch.float32
+    assert len(eng.cache.kv_groups) == 1 and len(eng.cache.paged_groups) == 2
+    assert not eng.model.capturable
+
+    cfg, w = P.read_model(d)
+    S = P.sizes(cfg)
+
+    def plain(ids):
+        n = len(ids)
+        x = P.embedding(w["model.embed_tokens.weight"], ids)
+        x = P.decoder_layer(x, w, 0, S, list(range(n)))
+        p = "model.layers.1."
+        h = P.rms_norm(x, w[p + "input_layernorm.weight"], S["eps"])
+        if dtype == "bfloat16":
+            h = h.to(torch.bfloat16).double()
+        c = h @ w_in.double().T
+        s = (c @ c.T) * width ** -0.5
+        s = s.masked_fill(torch.ones(n, n, dtype=torch.bool).triu(1), float("-inf"))
+        x = x + (torch.softmax(s, dim=-1) @ c) @ w_out.double().T
+        h = P.rms_norm(x, w[p + "post_attention_layernorm.weight"], S["eps"])
+        x = x + P.swiglu_mlp(h, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+        return P.linear(P.rms_norm(x, w["model.norm.weight"], S["eps"]), P.head_weight(w))
+
+    reqs = tiny.prompts("A", [100, 9, 70], seed=24)                  # two of them cross a page's edge
+    refs = [plain(r) for r in reqs]
+    for round_no in range(2):                                        # the second round finds the first one's rows in its pages
+        slots = [eng.open() for _ in reqs]
+        cuts = [60, 9, 1]
+        out = eng.step([StepEntry(s, r[:c], list(range(c))) for s, r, c in zip(slots, reqs, cuts)])
+        got, o = {i: [] for i in range(3)}, 0
+        for i, c in enumerate(cuts):
+            got[i].append(out[o:o + c]); o += c
+        fed = list(cuts)
+        while any(fed[i] < len(reqs[i]) for i in range(3)):
+            live = [i for i in range(3) if fed[i] < len(reqs[i])]
+            out = eng.step([StepEntry(slots[i], [reqs[i][fed[i]]], [0]) for i in live])
+            for r_, i in enumerate(live):
+                got[i].append(out[r_:r_ + 1]); fed[i] += 1
+        held = rows_groups[0].table.pages.held_count
+        assert held == 2 + 1 + 2                                     # pages of 100, 9 and 70 positions
+        for i in range(3):
+            tiny.assert_logits_close(torch.cat(got[i]), refs[i], dtype, f"latent mixer round {round_no} request {i}")
+            eng.close(slots[i])
+        assert rows_groups[0].table.pages.held_count == 0
+    eng.cache.check()
