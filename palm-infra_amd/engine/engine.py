@@ -190,6 +190,35 @@ class Engine:
 
     GRAPH_LIMIT = 24        # recorded steps kept at once; the least recently used one goes when another is recorded
 
+    def _recorded(self, key, n_tokens: int, n_seqs: int, n_rows: int | None) -> dict:
+        """The state of the recorded step ``key`` (made if new; the most recently used is kept last)."""
+        state = self._decode_graphs.pop(key, None)
+        if state is None:
+            while len(self._decode_graphs) >= self.GRAPH_LIMIT:          # a graph holds its activations and logits: bound them
+                self._decode_graphs.pop(next(iter(self._decode_graphs)))
+            state = {"buf": torch.zeros((context_ints(n_tokens, n_seqs),), dtype=torch.int32, device=self.device),
+                     "rows": None if n_rows is None else torch.zeros((n_rows,), dtype=torch.int32, device=self.device),
+                     "graph": None, "logits": None, "calls": 0}
+        self._decode_graphs[key] = state
+        return state
+
+    def _replay(self, state, ctx) -> torch.Tensor:
+        """Run the step whose arrays ``ctx`` has just laid into the state's buffer: as it is the first time (which
+        loads or builds whatever it needs), recorded the second time, replayed from then on."""
+        if state["graph"] is None and state["calls"] == 0:
+            logits = self.model.forward(ctx, self.cache, state["rows"])
+        else:
+            if state["graph"] is None:
+                torch.cuda.synchronize()
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph, pool=self._graph_pool()):
+                    state["logits"] = self.model.forward(ctx, self.cache, state["rows"])
+                state["graph"] = graph
+            state["graph"].replay()
+            logits = state["logits"].clone()        # the graph's own buffer is overwritten by the next replay
+        state["calls"] += 1
+        return logits
+
     def _run_decode_graph(self, entries) -> torch.Tensor:
         cache = self.cache
         growth = [(e.slot, 1) for e in entries]
@@ -199,36 +228,44 @@ class Engine:
         Bb = self._batch_bucket(B)
         key = (Bb, self._length_bucket(max(starts) + 1))
         pad = Bb - B
-        state = self._decode_graphs.pop(key, None)
-        if state is None:
-            while len(self._decode_graphs) >= self.GRAPH_LIMIT:          # a graph holds its activations and logits: bound them
-                self._decode_graphs.pop(next(iter(self._decode_graphs)))
-            state = {"buf": torch.zeros((context_ints(Bb, Bb),), dtype=torch.int32, device=self.device), "graph": None,
-                     "logits": None, "calls": 0}
-        self._decode_graphs[key] = state                                 # (re)inserted last: the most recently used
+        state = self._recorded(key, Bb, Bb, None)
         # the step's arrays, laid out as for any step, at the addresses the recording reads; rows that pad the batch
         # belong to a slot of their own whose page is never read
         ctx = make_context([e.slot for e in entries] + [cache.pad_slot] * pad, starts + [0] * pad,
                            [[int(e.tokens[0])] for e in entries] + [[0]] * pad, self.dtype, self.device,
                            max_total=key[1], into=state["buf"])
-        if state["graph"] is None and state["calls"] == 0:
-            # the first step of a shape runs as it is (and loads or builds whatever it needs)
-            logits = self.model.forward(ctx, cache, None)
-        else:
-            if state["graph"] is None:
-                torch.cuda.synchronize()
-                graph = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(graph, pool=self._graph_pool()):
-                    state["logits"] = self.model.forward(ctx, cache, None)
-                state["graph"] = graph
-            state["graph"].replay()
-            logits = state["logits"].clone()        # the graph's own buffer is overwritten by the next replay
-        state["calls"] += 1
+        logits = self._replay(state, ctx)
         cache.commit(growth)
         wanted = [b for b, e in enumerate(entries) if e.want]
         if len(wanted) == B:
             return logits[:B]
         return logits[torch.tensor(wanted, dtype=torch.long, device=self.device)] if wanted else logits[:0]
+
+    # A short prompt (or a short further piece) of one sequence is some hundred launches of kernels that take a few
+    # microseconds each: launched one by one the host takes longer than the device.  Such steps are recorded too, by
+    # the number of tokens rounded up to the next multiple of 8; the tokens that pad the step are a sequence of their
+    # own in the slot whose page is never read.
+    PROMPT_GRAPH_MAX_TOKENS = 63
+
+    def _prompt_graph_serves(self, entries) -> bool:
+        return (self.graphs_enabled and self.model.capturable and len(entries) == 1
+                and 2 <= len(entries[0].tokens) <= self.PROMPT_GRAPH_MAX_TOKENS and len(entries[0].want) == 1
+                and profile.active() is None)
+
+    def _run_prompt_graph(self, entries) -> torch.Tensor:
+        cache, e = self.cache, entries[0]
+        n = len(e.tokens)
+        bucket = (n // 8 + 1) * 8                   # at least one token pads the step
+        growth = [(e.slot, n)]
+        cache.reserve(growth)
+        start = cache.lengths[e.slot]
+        state = self._recorded(("prompt", bucket), bucket, 2, 1)
+        ctx = make_context([e.slot, cache.pad_slot], [start, 0], [list(map(int, e.tokens)), [0] * (bucket - n)], self.dtype,
+                           self.device, into=state["buf"], max_new=bucket)
+        state["rows"].copy_(torch.tensor([int(e.want[0])], dtype=torch.int32))
+        logits = self._replay(state, ctx)
+        cache.commit(growth)
+        return logits
 
     def _graph_pool(self):
         """One memory pool for all recorded steps: replays never overlap (one stream, one at a time), so their
@@ -247,6 +284,8 @@ class Engine:
                 return self._run_plain(entries)
         if self._graph_serves(entries):
             return self._run_decode_graph(entries)
+        if self._prompt_graph_serves(entries):
+            return self._run_prompt_graph(entries)
         return self._run_plain(entries)
 
     def _run_plain(self, entries) -> torch.Tensor:

@@ -104,12 +104,15 @@ def context_ints(n_tokens: int, n_seqs: int) -> int:
     return 3 * n_tokens + 4 * n_seqs + 1
 
 
-def make_context(slots, starts, new_tokens, dtype, device, max_total=None, into: torch.Tensor | None = None) -> StepContext:
+def make_context(slots, starts, new_tokens, dtype, device, max_total=None, into: torch.Tensor | None = None,
+                 max_new: int | None = None) -> StepContext:
     """A context from host lists: ``new_tokens[b]`` is the list of token ids of sequence b.  This is the one place
     where a step's arrays are laid out: a part that needs one more of them finds it here.
 
     ``into``: an int32 device buffer of ``context_ints(n, B)`` elements to lay the arrays in instead of a new
-    one: a recorded step keeps its arrays at fixed addresses and gets new contents before every replay."""
+    one: a recorded step keeps its arrays at fixed addresses and gets new contents before every replay.
+    ``max_new``, ``max_total``: bounds to size launches by instead of the step's own longest run and sequence (a
+    recorded step is sized for the largest step it will be replayed for)."""
     counts = [len(t) for t in new_tokens]
     ids = [t for seq in new_tokens for t in seq]
     pos = [starts[b] + j for b in range(len(slots)) for j in range(counts[b])]
@@ -133,7 +136,7 @@ def make_context(slots, starts, new_tokens, dtype, device, max_total=None, into:
         parts.append(flat[o:o + size])
         o += size
     return StepContext(
-        n_tokens=n, n_seqs=B, max_new=max(counts) if counts else 0,
+        n_tokens=n, n_seqs=B, max_new=max_new if max_new is not None else (max(counts) if counts else 0),
         max_total=max_total if max_total is not None else max((s + c for s, c in zip(starts, counts)), default=0),
         dtype=dtype, token_ids=parts[0], positions=parts[1], tok_slot=parts[2], seq_slot=parts[3], seq_start=parts[4],
         seq_new=parts[5], cu_new=parts[6], is_decode=all(c == 1 for c in counts),

@@ -48,7 +48,7 @@ def test_replays_equal_plain_launches(model_dirs, name, dtype):
         g.cache.check(); e.cache.check()
     if dtype != "float32":
         pool.check()                                            # a few rows a step: all of them together, too
-    keys = sorted(g._decode_graphs)
+    keys = sorted(k for k in g._decode_graphs if k[0] != "prompt")        # (the extra prompt between replays is recorded too)
     assert len(keys) >= 4 and all(st["graph"] is not None for k, st in g._decode_graphs.items() if st["calls"] > 1)
     assert not e._decode_graphs
 
@@ -158,4 +158,48 @@ def test_sequences_that_grow_across_length_buckets_and_few_recordings_are_kept(m
     assert {k[1] for k in seen} == {256, 512, 1024} and len(seen) >= 4      # more shapes than are kept at once
     for i in range(3):
         g.close(sg[i]); e.close(se[i])
+    g.cache.check()
+
+
+@pytest.mark.parametrize("name,dtype", [("A", "float32"), ("B", "bfloat16"), ("C", "bfloat16"), ("B", "float32")])
+def test_short_prompts_of_one_sequence_are_recorded_too(model_dirs, name, dtype):
+    """A prompt (or a further piece) of 2 to 63 tokens of one sequence with one place wanted runs as a recorded
+    step, padded to a multiple of 8 tokens by a sequence of its own: every length three times (as it is,
+    recorded, replayed), at the start of a sequence and on top of what it already holds, against plain launches
+    and against the plain implementation."""
+    import plain_qwen3 as P
+    from palm_infra_amd.engine import Engine, StepEntry
+    g = Engine.from_dir(model_dirs[name][dtype], dtype=dtype, max_tokens=64 * 12, graphs=True)
+    e = Engine.from_dir(model_dirs[name][dtype], dtype=dtype, max_tokens=64 * 12, graphs=False)
+    cfg, w = P.read_model(model_dirs[name][dtype])
+    pool = tiny.LogitsPool(dtype, f"{name} {dtype}: short prompts as recorded steps")
+    lengths = [2, 7, 8, 9, 15, 16, 17, 31, 40, 63]
+    for round_no in range(3):
+        for n in lengths:
+            ids = tiny.prompts(name, [n + 1 + 5], seed=50 + n + 100 * round_no)[0]
+            ref = P.logits(cfg, w, ids)
+            sg, se = g.open(), e.open()
+            a = g.step([StepEntry(sg, ids[:n], [n - 1])])
+            b = e.step([StepEntry(se, ids[:n], [n - 1])])
+            a1 = g.step([StepEntry(sg, ids[n:n + 1], [0])])               # a decode step on what the recorded prompt left
+            b1 = e.step([StepEntry(se, ids[n:n + 1], [0])])
+            a2 = g.step([StepEntry(sg, ids[n + 1:], [2])])                # a further piece of five tokens, recorded as well
+            b2 = e.step([StepEntry(se, ids[n + 1:], [2])])
+            if dtype == "float32":
+                assert torch.equal(a, b) and torch.equal(a1, b1) and torch.equal(a2, b2), (round_no, n)
+            pool.add(torch.cat([a, a1, a2]), ref[[n - 1, n, n + 3]], f"round {round_no}, {n} tokens")
+            assert g.length(sg) == n + 6
+            g.close(sg); e.close(se)
+    pool.check()
+    recorded = {k: st for k, st in g._decode_graphs.items() if k[0] == "prompt"}
+    assert set(recorded) == {("prompt", b) for b in (8, 16, 24, 32, 48, 64)}
+    assert all(st["graph"] is not None and st["calls"] >= 3 for st in recorded.values())
+    assert not e._decode_graphs
+    # what is not served: two sequences, more than one place wanted, 64 tokens or more
+    s1, s2 = g.open(), g.open()
+    before = {k: st["calls"] for k, st in g._decode_graphs.items()}
+    g.step([StepEntry(s1, [1, 2, 3], [2]), StepEntry(s2, [4, 5], [1])])
+    g.step([StepEntry(s1, [1, 2, 3], [0, 2])])
+    g.step([StepEntry(s2, list(range(1, 65)), [63])])
+    assert {k: st["calls"] for k, st in g._decode_graphs.items()} == before
     g.cache.check()
