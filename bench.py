@@ -115,6 +115,66 @@ def time_prefill(engine, tokens: int, vocab: int, repeats: int = 3) -> float:
     return best
 
 
+def kernel_table(engine, cfg, slots, batch: int, context: int) -> dict:
+    """The decode step's dominant kernels one by one: each launched once for every layer (so that no weight is read
+    twice from a cache) inside a recorded graph, timed with events around its replays; the bytes each has to
+    read, the time of one launch, and the fraction of the HBM peak that makes."""
+    import torch
+    from palm_infra_amd.kernels import ops
+    from palm_infra_amd.parts import ResidualSink
+    model, cache = engine.model, engine.cache
+    layers = model.layers
+    L = len(layers)
+    H, I = cfg["hidden_size"], cfg["intermediate_size"]
+    nh, nkv, hd = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+    dev, bf16 = engine.device, torch.bfloat16
+    g = torch.Generator(device=dev).manual_seed(1)
+    h = torch.randn(batch, H, device=dev, dtype=bf16, generator=g)
+    attn = torch.randn(batch, nh * hd, device=dev, dtype=bf16, generator=g)
+    act = torch.randn(batch, I, device=dev, dtype=bf16, generator=g)
+    resid = torch.zeros(batch, H, device=dev, dtype=torch.float32)
+    kv = cache.kv_groups[0]
+    seq_slot = torch.tensor(slots, dtype=torch.int32, device=dev)
+    seq_start = torch.tensor([cache.lengths[s] - 1 for s in slots], dtype=torch.int32, device=dev)
+    n_slices = ops.decode_slices(batch, nh, nkv, engine._length_bucket(context + 1))
+
+    def each_layer(fn):
+        return lambda: [fn(i) for i in range(L)]
+    work = {
+        "qkv_proj": (each_layer(lambda i: layers[i].mixer.qkv(h, planes_ok=True)), (nh + 2 * nkv) * hd * H * 2, L),
+        "attention": (each_layer(lambda i: ops.attention_decode(attn, kv.k[i], kv.v[i], kv.table_dev, seq_slot, seq_start, nh, nkv, hd,
+                                                                hd ** -0.5, None, n_slices)),
+                      2 * nkv * hd * 2 * context * batch, L),
+        "o_proj": (each_layer(lambda i: layers[i].mixer.out(attn, sink=ResidualSink(resid, layers[i].feed_forward_norm))),
+                   nh * hd * H * 2, L),
+        "gate_up_proj": (each_layer(lambda i: layers[i].feed_forward.gate_up.gated(h)), 2 * I * H * 2, L),
+        "down_proj": (each_layer(lambda i: layers[i].feed_forward.down(act, sink=ResidualSink(resid, layers[i].mixer_norm))),
+                      I * H * 2, L),
+        "lm_head": (lambda: [model.head.forward(h)], cfg["vocab_size"] * H * 2, 1),
+    }
+    table = {}
+    for name, (fn, nbytes, launches) in work.items():
+        fn()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            fn()
+        graph.replay()
+        torch.cuda.synchronize()
+        best = float("inf")
+        for _ in range(5):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            graph.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            best = min(best, e0.elapsed_time(e1) * 1000.0 / launches)
+        gbs = nbytes / best / 1e3
+        table[name] = {"bytes": int(nbytes), "us": round(best, 2), "gbs": round(gbs, 1), "frac": round(gbs / PEAK_HBM_GBS, 4)}
+        del graph
+    return table
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -145,14 +205,18 @@ def main(argv=None) -> int:
     prefill_ms = time_prefill(engine, PREFILL_TOKENS, vocab)
     pf = prefill_flops(cfg, PREFILL_TOKENS)
 
-    def decode_at(batch: int, steps: int, warmup: int) -> float:
+    kernels = {}
+
+    def decode_at(batch: int, steps: int, warmup: int, table: bool = False) -> float:
         slots = fill_contexts(engine, batch, CONTEXT, vocab)
         ms = time_decode(engine, sampler, slots, steps, warmup, vocab)
+        if table:
+            kernels.update(kernel_table(engine, cfg, slots, batch, CONTEXT + warmup + steps))
         for s in slots:
             engine.close(s)
         return ms
 
-    ms_step = decode_at(args.batch, args.steps, args.warmup)
+    ms_step = decode_at(args.batch, args.steps, args.warmup, table=True)
     value = args.batch * 1000.0 / ms_step
     points = {}
     if not args.no_points:
@@ -177,7 +241,9 @@ def main(argv=None) -> int:
         "prefill": {"value": round(PREFILL_TOKENS * 1000.0 / prefill_ms, 1), "tokens": PREFILL_TOKENS,
                     "ms": round(prefill_ms, 3), "frac": round(pf / (prefill_ms * 1e-3) / PEAK_FLOPS["bf16"], 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                     "frac": round(achieved / PEAK_HBM_GBS, 4)},
+                     "frac": round(achieved / PEAK_HBM_GBS, 4),
+                     # the step's dominant kernels alone (a launch for each layer in a recorded graph, event-timed)
+                     "kernels": kernels, **{f"frac_{k}": v["frac"] for k, v in kernels.items()}},
         "points": points,
     }
     print(json.dumps(record), flush=True)

@@ -22,7 +22,7 @@ PALM_API int palm_attention_decode(hipStream_t stream, const void* q, const void
 // process ends.  The call allocates nothing, frees nothing and calls no allocating routine; it refuses
 // n_seqs * nh * n_slices * (hd + 4) beyond the limit with an error and launches nothing then.  All calls on one
 // GPU share that GPU's buffer, which keeps the last call's contents: nothing in it has to start at zero (every
-// slice, also an empty one, writes its whole record before the merge reads it), but two calls that overlap in
+// slice that holds keys writes its whole record before the merge reads it, and the merge reads no other), but two calls that overlap in
 // time on one GPU (different streams, or a graph replayed beside an eager call) race on it.  Calls on one stream,
 // one after the other, are safe.  The result is the same bits as palm_attention_decode's with the same slices.
 PALM_API int palm_attention_decode_static(hipStream_t stream, const void* q, const void* k_cache, const void* v_cache,

@@ -225,8 +225,9 @@ __global__ __launch_bounds__(WAVE) DECODE_WAVES_PER_SIMD void attention_decode_k
         }
         return;
     }
+    if (p0 >= p1) return;                               // an empty slice: the merge does not read its record
     float* w = work + (((size_t)b * nh + head) * n_slices + slice) * WORK_STRIDE;
-    if (g == 0) { w[0] = c.m; w[1] = l; }               // an empty slice leaves m = -inf, l = 0
+    if (g == 0) { w[0] = c.m; w[1] = l; }
 #pragma unroll
     for (int dt = 0; dt < DTILES; ++dt)                    // the lane's four elements of a tile lie side by side: one store
         *reinterpret_cast<float4*>(w + WORK_O + dt * 16 + 4 * g) = make_float4(c.o[dt][0], c.o[dt][1], c.o[dt][2], c.o[dt][3]);
@@ -234,26 +235,34 @@ __global__ __launch_bounds__(WAVE) DECODE_WAVES_PER_SIMD void attention_decode_k
 
 // One wave per (sequence, head): merge the slices in a fixed order.  Lane s first reads slice s's maximum
 // and sum (all at once), the wave agrees on the overall maximum and on each slice's weight, then lane d sums
-// output element d over the slices, eight reads in flight at a time.
-__global__ __launch_bounds__(WAVE) void attention_merge_kernel(const float* __restrict__ work, int n_slices,
+// output element d over the slices, eight reads in flight at a time.  Only the slices that hold pages of this
+// sequence are read: a launch is cut for the longest sequence a recorded step may serve, and a shorter one leaves
+// its last slices empty (one sequence of 2,048 tokens in a step recorded for 4,096: 33 of 64).
+__global__ __launch_bounds__(WAVE) void attention_merge_kernel(const float* __restrict__ work, int n_slices, int nh,
+                                                               const int* __restrict__ seq_start, int window,
                                                                bf16_t* __restrict__ out) {
     const float* w = work + (size_t)blockIdx.x * n_slices * WORK_STRIDE;
     const int lane = threadIdx.x;
+    const int pos = seq_start[blockIdx.x / nh];
+    const int first = window > 0 ? max(0, pos - window + 1) : 0;
+    const int n_pages = pos / PAGE_TOKENS - first / PAGE_TOKENS + 1;
+    const int per = (n_pages + n_slices - 1) / n_slices;
+    const int live = (n_pages + per - 1) / per;                 // as attention_decode_kernel cuts the range: <= n_slices
     float m = -INFINITY;
-    for (int s = lane; s < n_slices; s += WAVE) m = fmaxf(m, w[(size_t)s * WORK_STRIDE]);
+    for (int s = lane; s < live; s += WAVE) m = fmaxf(m, w[(size_t)s * WORK_STRIDE]);
     m = wave_max(m);
     float l = 0.f;
-    for (int s = lane; s < n_slices; s += WAVE) l += w[(size_t)s * WORK_STRIDE + 1] * exp2f(w[(size_t)s * WORK_STRIDE] - m);
+    for (int s = lane; s < live; s += WAVE) l += w[(size_t)s * WORK_STRIDE + 1] * exp2f(w[(size_t)s * WORK_STRIDE] - m);
     l = wave_sum(l);
     constexpr int PER = (HD + WAVE - 1) / WAVE;
     float o[PER];
 #pragma unroll
     for (int i = 0; i < PER; ++i) o[i] = 0.f;
-    for (int s0 = 0; s0 < n_slices; s0 += 8) {
+    for (int s0 = 0; s0 < live; s0 += 8) {
         float ms[8], v[8][PER];
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
-            const int s = min(s0 + u, n_slices - 1);
+            const int s = min(s0 + u, live - 1);
             ms[u] = w[(size_t)s * WORK_STRIDE];
 #pragma unroll
             for (int i = 0; i < PER; ++i) {
@@ -263,7 +272,7 @@ __global__ __launch_bounds__(WAVE) void attention_merge_kernel(const float* __re
         }
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
-            const float wt = s0 + u < n_slices ? exp2f(ms[u] - m) : 0.f;
+            const float wt = s0 + u < live ? exp2f(ms[u] - m) : 0.f;
 #pragma unroll
             for (int i = 0; i < PER; ++i) o[i] += v[u][i] * wt;
         }
@@ -293,7 +302,7 @@ static int launch_attention_decode(hipStream_t stream, const void* q, const void
                                                       window, n_slices, work, (bf16_t*)out);
     PALM_LAUNCHED();
     if (n_slices > 1) {
-        attention_merge_kernel<<<n_seqs * nh, WAVE, 0, stream>>>(work, n_slices, (bf16_t*)out);
+        attention_merge_kernel<<<n_seqs * nh, WAVE, 0, stream>>>(work, n_slices, nh, seq_start, window, (bf16_t*)out);
         PALM_LAUNCHED();
     }
     return 0;

@@ -39,9 +39,10 @@ _SIGNATURES = {
     "palm_linear_wide": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int],
     "palm_linear_wide_parts": [c_int, c_int, c_int, c_int],
     "palm_linear_wide_blocks": [c_int, c_int, c_int, c_int, c_int],
-    "palm_linear_tile": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_float,
-                         c_void_p, c_void_p, c_void_p],
+    "palm_linear_tile": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int,
+                         c_float, c_void_p, c_void_p, c_void_p],
     "palm_linear_tile_pieces": [c_int],
+    "palm_linear_tile_parts": [c_int, c_int, c_int],
     "palm_argmax": [c_void_p, c_void_p, c_int, c_int, c_void_p],
     "palm_apply_penalties": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_float, c_float, c_float],
     "palm_sample": [c_void_p, c_void_p, c_int, c_int, c_void_p, c_float, c_int, c_float, c_float, c_void_p, c_void_p],
@@ -485,10 +486,12 @@ def _tile_row_ss(what: str, a: torch.Tensor, row_ss) -> int:
     return row_ss.shape[1]
 
 
-def linear_tile(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, gated: bool = False, row_ss=None,
-                row_eps: float = 0.0) -> torch.Tensor:
+def linear_tile(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, gated: bool = False, planes_ok: bool = False,
+                row_ss=None, row_eps: float = 0.0) -> torch.Tensor:
     """bfloat16 a [M, K] . w [N, K]^T for many rows, tiled over the matrix cores; result bfloat16 or float32.
     ``gated``: w is [gate rows | up rows] and the result is silu(a gate^T) * (a up^T), [M, N/2].
+    ``planes_ok``: the caller takes float32 planes [P, M, N] of partial sums (see linear_thin); the kernel then
+    cuts K into ranges where the tiles alone would leave most of the chip without work.
     ``row_ss`` with ``row_eps``: the rows of a lack their norm's factor (see linear_thin)."""
     _dev("linear_tile", a, w)
     _need(a.dim() == 2 and w.dim() == 2 and tile_serves(a, w), f"linear_tile: a {tuple(a.shape)} {a.dtype}, w {tuple(w.shape)} "
@@ -497,9 +500,13 @@ def linear_tile(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, gated:
     N = w.shape[0]
     _need(not gated or N % 2 == 0, f"linear_tile: a gated product needs an even number of weight rows, got {N}")
     pieces = _tile_row_ss("linear_tile", a, row_ss)
-    out = torch.empty((M, N // 2 if gated else N), dtype=out_dtype, device=a.device)
+    parts = core().palm_linear_tile_parts(M, N, K) if planes_ok and not gated and row_ss is None else 1
+    if parts > 1:
+        out = torch.empty((parts, M, N), dtype=F32, device=a.device)
+    else:
+        out = torch.empty((M, N // 2 if gated else N), dtype=out_dtype, device=a.device)
     library.call(core(), "palm_linear_tile", _stream(), _p(a), _p(w), _p(out), _code(out, "linear_tile out"), M, N, K,
-                 1 if gated else 0, _p(row_ss), pieces, float(row_eps), None, None, None)
+                 1 if gated else 0, parts, _p(row_ss), pieces, float(row_eps), None, None, None)
     return out
 
 
@@ -517,7 +524,7 @@ def linear_tile_into_residual(a: torch.Tensor, w: torch.Tensor, x: torch.Tensor,
     pieces = _tile_row_ss("linear_tile_into_residual", a, row_ss)
     values = torch.empty((M, N), dtype=BF16, device=a.device)
     ss = torch.empty((M, core().palm_linear_tile_pieces(N)), dtype=F32, device=a.device)
-    library.call(core(), "palm_linear_tile", _stream(), _p(a), _p(w), _p(values), _code(values, "values"), M, N, K, 2,
+    library.call(core(), "palm_linear_tile", _stream(), _p(a), _p(w), _p(values), _code(values, "values"), M, N, K, 2, 1,
                  _p(row_ss), pieces, float(row_eps), _p(x), _p(norm_w), _p(ss))
     return values, ss
 

@@ -60,9 +60,11 @@ def test_linear_for_17_to_64_rows_as_planes_of_partial_sums(ops, M, N, K, cut):
     a, w = rand(M, K, seed=M, dtype=BF16), rand(N, K, seed=N + K, dtype=BF16)
     got = ops.linear_thin(a.to(DEV), w.to(DEV), F32, planes_ok=True).cpu()
     want = P.linear(a, w)
-    if cut:
-        assert got.dim() == 3 and 2 <= got.shape[0] <= 4 and got.shape[1:] == (M, N) and got.dtype == F32
-        assert all(float(got[p].abs().max()) > 0 for p in range(got.shape[0]))       # no range of K is empty
+    parts = ops.core().palm_linear_tile_parts(M, N, K)
+    assert parts > 1 if cut else parts >= 1
+    if parts > 1:
+        assert got.shape == (parts, M, N) and parts <= 4 and got.dtype == F32
+        assert all(float(got[p].abs().max()) > 0 for p in range(parts))              # no range of K is empty
         got = got.double().sum(0)
     else:
         assert got.shape == (M, N)
@@ -195,6 +197,27 @@ def test_linear_tile_against_the_plain_product(ops, M, N, K):
     assert torch.equal(got16, got32.to(BF16))                          # one rounding at the end
     # and through the dispatcher: a float32 result for more than 64 rows takes this kernel
     assert torch.equal(ops.linear_thin(a.to(DEV), w.to(DEV), F32).cpu(), got32)
+
+
+@pytest.mark.parametrize("M", [70, 256, 300])
+@pytest.mark.parametrize("N,K,cut", [(4096, 12288, True), (4096, 4096, True), (1000, 3072, True), (24576, 4096, False),
+                                     (4096, 1024, False)])
+def test_linear_tile_as_planes_of_partial_sums(ops, M, N, K, cut):
+    """Few tiles and a long K: K is cut into ranges, each block writes its range's sums to a float32 plane, and the
+    planes add up to the product; a product with tiles enough comes whole."""
+    a, w = rand(M, K, seed=M), rand(N, K, seed=N + K, scale=0.5)
+    got = ops.linear_tile(a.to(DEV), w.to(DEV), F32, planes_ok=True).cpu()
+    want = P.linear(a, w)
+    parts = ops.core().palm_linear_tile_parts(M, N, K)
+    assert parts > 1 if cut else parts >= 1
+    if parts > 1:
+        assert got.shape == (parts, M, N) and parts <= 4 and got.dtype == F32
+        assert all(float(got[p].abs().max()) > 0 for p in range(parts))              # no range of K is empty
+        got = got.double().sum(0)
+    else:
+        assert got.shape == (M, N)
+    assert torch.allclose(got.double(), want, atol=2e-4 * (K ** 0.5), rtol=1e-5)
+    assert ops.linear_tile(a.to(DEV), w.to(DEV), BF16, planes_ok=False).shape == (M, N)
 
 
 def test_linear_tile_orientation_and_every_k_once(ops):
