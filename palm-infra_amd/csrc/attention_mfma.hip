@@ -371,7 +371,7 @@ PALM_API int palm_attention_decode_static(hipStream_t stream, const void* q, con
 
 // ---- prefill --------------------------------------------------------------------------------------
 // A block of four waves serves one kv head, up to eight query heads of its group (more heads: more blocks)
-// and a tile of QB query positions, QB = 16 * max(1, 8 / heads): at most eight "units" of 16 columns
+// and a tile of QB query positions, QB = 16 * max(1, 8 / heads): at most eight "units" (two a wave) of 16 columns
 // (head, 16 positions), two for each wave.  A page of K and of V^T is read from memory once for the block,
 // into LDS; every wave takes its MFMA operands from there, each operand serving both of its units.  The next
 // page is on its way into registers while the current one is being used.
@@ -381,7 +381,12 @@ PALM_API int palm_attention_decode_static(hipStream_t stream, const void* q, con
 // tokens (sub-tile f with sub-tile N - 1 - f): every block then has about the same number of (unit, page)
 // products.  The early sub-tile's keys are among the late one's, so the block walks the late one's pages and
 // the early one's units just stop taking part (`active`) once the pages lie beyond them.
-constexpr int PF_WAVES = 4;
+// (Eight waves a block, 16 units, halve what a block's queries read of K and V from L2; measured at 2,048 tokens:
+// 77 us against 64, the barrier of eight waves and one block a compute unit costing more than the reads save.)
+#ifndef PALM_PF_WAVES
+#define PALM_PF_WAVES 4
+#endif
+constexpr int PF_WAVES = PALM_PF_WAVES;
 constexpr int PF_THREADS = PF_WAVES * WAVE;
 constexpr int PF_UNITS = 2;                                // units of 16 columns held by a wave
 constexpr float PF_LAZY_LOG2 = 8.0f;                       // how far (in powers of two) a maximum may rise before the outputs are rescaled
@@ -796,8 +801,9 @@ PALM_API int palm_attention_prefill(hipStream_t stream, const void* q, const voi
     PALM_CHECK(window >= 0 && max_pages > 0, "attention_prefill: window=%d max_pages=%d", window, max_pages);
     if (n_seqs == 0 || max_new == 0) return 0;
     const int G = nh / nkv;
-    const int hg = G < 8 ? G : 8;                              // query heads of the group served by one block
-    const int qb = 16 * (8 / hg > 0 ? 8 / hg : 1);             // query positions in a tile: at most 8 units a block
+    constexpr int UNITS = PF_UNITS * PF_WAVES;                 // (head, 16 queries) units a block holds
+    const int hg = G < UNITS ? G : UNITS;                      // query heads of the group served by one block
+    const int qb = 16 * (UNITS / hg > 0 ? UNITS / hg : 1);     // query positions in a tile
     const int n_hg = (G + hg - 1) / hg;
     PALM_CHECK(nkv * n_hg <= 65535 && n_seqs <= 65535, "attention_prefill: grid too large");
     const int n16 = (max_new + 15) / 16, subs = qb / 16;

@@ -60,11 +60,9 @@ def test_linear_for_17_to_64_rows_as_planes_of_partial_sums(ops, M, N, K, cut):
     a, w = rand(M, K, seed=M, dtype=BF16), rand(N, K, seed=N + K, dtype=BF16)
     got = ops.linear_thin(a.to(DEV), w.to(DEV), F32, planes_ok=True).cpu()
     want = P.linear(a, w)
-    parts = ops.core().palm_linear_tile_parts(M, N, K)
-    assert parts > 1 if cut else parts >= 1
-    if parts > 1:
-        assert got.shape == (parts, M, N) and parts <= 4 and got.dtype == F32
-        assert all(float(got[p].abs().max()) > 0 for p in range(parts))              # no range of K is empty
+    if cut:
+        assert got.dim() == 3 and 2 <= got.shape[0] <= 4 and got.shape[1:] == (M, N) and got.dtype == F32
+        assert all(float(got[p].abs().max()) > 0 for p in range(got.shape[0]))       # no range of K is empty
         got = got.double().sum(0)
     else:
         assert got.shape == (M, N)
