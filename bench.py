@@ -175,6 +175,64 @@ def kernel_table(engine, cfg, slots, batch: int, context: int) -> dict:
     return table
 
 
+def prefill_kernel_table(engine, cfg, tokens: int) -> dict:
+    """The prompt step's dominant kernels one by one at `tokens` rows, as kernel_table does it: the four products
+    of a layer (the library's), the prompt attention, the norm with the residual add and the gated activation;
+    flops (or bytes) each has to do, the time of one launch and the fraction of the peak that makes."""
+    import torch
+    from palm_infra_amd.engine import StepEntry
+    from palm_infra_amd.kernels import ops
+    model, cache = engine.model, engine.cache
+    layers = model.layers
+    L = len(layers)
+    H, I = cfg["hidden_size"], cfg["intermediate_size"]
+    nh, nkv, hd = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+    dev, bf16 = engine.device, torch.bfloat16
+    g = torch.Generator(device=dev).manual_seed(2)
+    h = torch.randn(tokens, H, device=dev, dtype=bf16, generator=g)
+    attn = torch.randn(tokens, nh * hd, device=dev, dtype=bf16, generator=g)
+    act = torch.randn(tokens, I, device=dev, dtype=bf16, generator=g)
+    gate_up = torch.randn(tokens, 2 * I, device=dev, dtype=bf16, generator=g)
+    resid = torch.zeros(tokens, H, device=dev, dtype=torch.float32)
+    slot = engine.open()
+    engine.step([StepEntry(slot, random_ids(tokens, cfg["vocab_size"], 900), [])])       # keys and values to attend over
+    kv = cache.kv_groups[0]
+    i32 = lambda xs: torch.tensor(xs, dtype=torch.int32, device=dev)
+    seq_slot, seq_start, seq_new, cu = i32([slot]), i32([0]), i32([tokens]), i32([0, tokens])
+    mfma, hbm = PEAK_FLOPS["bf16"], PEAK_HBM_GBS * 1e9
+
+    def each_layer(fn):
+        return lambda: [fn(i) for i in range(L)]
+    work = {
+        "qkv_proj": (each_layer(lambda i: layers[i].mixer.qkv(h)), 2.0 * tokens * (nh + 2 * nkv) * hd * H, mfma),
+        "attention": (each_layer(lambda i: ops.attention_prefill(attn, kv.k[i], kv.v[i], kv.table_dev, seq_slot, seq_start, seq_new, cu,
+                                                                 tokens, nh, nkv, hd, hd ** -0.5, None)),
+                      4.0 * nh * hd * tokens * (tokens + 1) / 2.0, mfma),
+        "o_proj": (each_layer(lambda i: layers[i].mixer.out(attn)), 2.0 * tokens * nh * hd * H, mfma),
+        "gate_up_proj": (each_layer(lambda i: layers[i].feed_forward.gate_up(h)), 2.0 * tokens * 2 * I * H, mfma),
+        "down_proj": (each_layer(lambda i: layers[i].feed_forward.down(act)), 2.0 * tokens * I * H, mfma),
+        # memory-bound passes: bytes instead of flops, against the HBM peak
+        "norm_with_add": (each_layer(lambda i: layers[i].feed_forward_norm(resid, delta=h, update=True)), tokens * H * (4 + 2 + 4 + 2.0), hbm),
+        "gated_activation": (each_layer(lambda i: ops.swiglu(gate_up)), tokens * I * (4 + 2.0), hbm),
+    }
+    table = {}
+    for name, (fn, amount, peak) in work.items():
+        fn()
+        torch.cuda.synchronize()
+        best = float("inf")
+        for _ in range(3):                     # launched one by one, as a prompt step launches them
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            fn()
+            e1.record()
+            torch.cuda.synchronize()
+            best = min(best, e0.elapsed_time(e1) * 1000.0 / L)
+        table[name] = {"us": round(best, 1), "frac": round(amount / (best * 1e-6) / peak, 4),
+                       "of": "mfma" if peak == mfma else "hbm"}
+    engine.close(slot)
+    return table
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -204,6 +262,7 @@ def main(argv=None) -> int:
 
     prefill_ms = time_prefill(engine, PREFILL_TOKENS, vocab)
     pf = prefill_flops(cfg, PREFILL_TOKENS)
+    prefill_kernels = prefill_kernel_table(engine, cfg, PREFILL_TOKENS)
 
     kernels = {}
 
@@ -239,7 +298,10 @@ def main(argv=None) -> int:
                    "rms_norm_eps": cfg["rms_norm_eps"], "tied_head": False, "cache_context": 4096,
                    "prefill_tokens": PREFILL_TOKENS, "decode_steps": args.steps, "load_s": round(load_s, 1)},
         "prefill": {"value": round(PREFILL_TOKENS * 1000.0 / prefill_ms, 1), "tokens": PREFILL_TOKENS,
-                    "ms": round(prefill_ms, 3), "frac": round(pf / (prefill_ms * 1e-3) / PEAK_FLOPS["bf16"], 4)},
+                    "ms": round(prefill_ms, 3), "frac": round(pf / (prefill_ms * 1e-3) / PEAK_FLOPS["bf16"], 4),
+                    # the step's dominant kernels alone (a launch for each layer, event-timed): us a layer, and the
+                    # fraction of the matrix cores' (or, for the two memory-bound passes, of HBM's) peak
+                    "kernels": prefill_kernels},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": round(achieved / PEAK_HBM_GBS, 4),
                      # the step's dominant kernels alone (a launch for each layer in a recorded graph, event-timed)
