@@ -141,21 +141,28 @@ __device__ inline void weigh_values(const PageOperands& ops, const bf16x8 (&pv)[
 
 // All pages p0 <= p < p1 of one sequence and kv head.  The reads of the next page are issued as soon as the
 // registers of the current one are free: K after the scores, V after the weighted sum, so that a page's
-// latency hides behind the previous page's arithmetic.  first/pos: the column's own key range.
+// latency hides behind the previous page's arithmetic.  first/last: the column's own key range.
+// start.prepare(qv, c) is called once, after the first page's keys have been asked for: a caller whose query is
+// not finished yet finishes it there, while the keys are on their way (Ready: nothing to do).
+struct Ready {
+    __device__ void prepare(bf16x8 (&)[KSTEPS], Columns&) {}
+};
+template <typename Start>
 __device__ inline void attend_pages(const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
                                     const int* __restrict__ pages, int nkv, int kvh, int p0, int p1,
-                                    const bf16x8 (&qv)[KSTEPS], int first, int pos, float scale_log2, Columns& c,
-                                    int r, int g) {
+                                    bf16x8 (&qv)[KSTEPS], int first, int last, float scale_log2, Columns& c,
+                                    int r, int g, Start& start) {
     if (p0 >= p1) return;
     PageOperands ops;
     size_t base = ((size_t)pages[p0] * nkv + kvh) * PAGE_TOKENS * HD;
     load_keys(k_cache + base, r, g, ops);
+    start.prepare(qv, c);
     load_values(v_cache + base, r, g, ops);
     for (int p = p0; p < p1; ++p) {
         const bool more = p + 1 < p1;
         const size_t next = more ? ((size_t)pages[p + 1] * nkv + kvh) * PAGE_TOKENS * HD : base;
         bf16x8 pv[2];
-        const float alpha = score_page(ops, qv, first - p * PAGE_TOKENS, pos - p * PAGE_TOKENS, scale_log2, c, g, pv);
+        const float alpha = score_page(ops, qv, first - p * PAGE_TOKENS, last - p * PAGE_TOKENS, scale_log2, c, g, pv);
         if (more) load_keys(k_cache + next, r, g, ops);
         weigh_values(ops, pv, alpha, c);
         if (more) load_values(v_cache + next, r, g, ops);
@@ -177,6 +184,35 @@ __device__ inline void load_query(const bf16_t* qrow, bool valid, int g, bf16x8 
 // grid (slices, nkv * query groups, sequences), one wave each.  Workspace per (sequence, head, slice):
 // m, l, two floats unused, then HD floats of the unnormalised output (which so start on 16 bytes).
 constexpr int WORK_O = 4, WORK_STRIDE = HD + WORK_O;
+
+// What a slice's wave leaves: with one slice the output itself, else its record in the workspace (maximum, sum, two
+// floats unused, HD floats of the unnormalised output) for the merge; an empty slice leaves nothing.
+__device__ inline void finish_slice(Columns& c, bool valid, int b, int head, int nh, int slice, int n_slices, bool empty,
+                                    int g, float* __restrict__ work, bf16_t* __restrict__ out) {
+    float l = c.l;
+    l += __shfl_xor(l, 16, WAVE);
+    l += __shfl_xor(l, 32, WAVE);
+    if (!valid) return;
+    if (n_slices == 1) {
+        const float inv = 1.0f / l;
+        bf16_t* o = out + ((size_t)b * nh + head) * HD;
+#pragma unroll
+        for (int dt = 0; dt < DTILES; ++dt) {
+            uint2 four;
+            four.x = (uint32_t)f32_to_bf16(c.o[dt][0] * inv).bits | ((uint32_t)f32_to_bf16(c.o[dt][1] * inv).bits << 16);
+            four.y = (uint32_t)f32_to_bf16(c.o[dt][2] * inv).bits | ((uint32_t)f32_to_bf16(c.o[dt][3] * inv).bits << 16);
+            *reinterpret_cast<uint2*>(o + dt * 16 + 4 * g) = four;
+        }
+        return;
+    }
+    if (empty) return;                                  // the merge does not read its record
+    float* w = work + (((size_t)b * nh + head) * n_slices + slice) * WORK_STRIDE;
+    if (g == 0) { w[0] = c.m; w[1] = l; }
+#pragma unroll
+    for (int dt = 0; dt < DTILES; ++dt)                    // the lane's four elements of a tile lie side by side: one store
+        *reinterpret_cast<float4*>(w + WORK_O + dt * 16 + 4 * g) = make_float4(c.o[dt][0], c.o[dt][1], c.o[dt][2], c.o[dt][3]);
+}
+
 #if PALM_HEAD_DIM <= 128
 #define DECODE_WAVES_PER_SIMD __attribute__((amdgpu_waves_per_eu(2)))     // fits without spilling up to this head size
 #else
@@ -208,29 +244,9 @@ __global__ __launch_bounds__(WAVE) DECODE_WAVES_PER_SIMD void attention_decode_k
     for (int dt = 0; dt < DTILES; ++dt) c.o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     const int* pages = block_table + (size_t)seq_slot[b] * max_pages;
-    attend_pages(k_cache, v_cache, pages, nkv, kvh, p0, p1, qv, first, pos, scale_log2, c, r, g);
-    float l = c.l;
-    l += __shfl_xor(l, 16, WAVE);
-    l += __shfl_xor(l, 32, WAVE);
-    if (!valid) return;
-    if (n_slices == 1) {
-        const float inv = 1.0f / l;
-        bf16_t* o = out + ((size_t)b * nh + head) * HD;
-#pragma unroll
-        for (int dt = 0; dt < DTILES; ++dt) {
-            uint2 four;
-            four.x = (uint32_t)f32_to_bf16(c.o[dt][0] * inv).bits | ((uint32_t)f32_to_bf16(c.o[dt][1] * inv).bits << 16);
-            four.y = (uint32_t)f32_to_bf16(c.o[dt][2] * inv).bits | ((uint32_t)f32_to_bf16(c.o[dt][3] * inv).bits << 16);
-            *reinterpret_cast<uint2*>(o + dt * 16 + 4 * g) = four;
-        }
-        return;
-    }
-    if (p0 >= p1) return;                               // an empty slice: the merge does not read its record
-    float* w = work + (((size_t)b * nh + head) * n_slices + slice) * WORK_STRIDE;
-    if (g == 0) { w[0] = c.m; w[1] = l; }
-#pragma unroll
-    for (int dt = 0; dt < DTILES; ++dt)                    // the lane's four elements of a tile lie side by side: one store
-        *reinterpret_cast<float4*>(w + WORK_O + dt * 16 + 4 * g) = make_float4(c.o[dt][0], c.o[dt][1], c.o[dt][2], c.o[dt][3]);
+    Ready ready;
+    attend_pages(k_cache, v_cache, pages, nkv, kvh, p0, p1, qv, first, pos, scale_log2, c, r, g, ready);
+    finish_slice(c, valid, b, head, nh, slice, n_slices, p0 >= p1, g, work, out);
 }
 
 // One wave per (sequence, head): merge the slices in a fixed order.  Lane s first reads slice s's maximum
@@ -314,6 +330,346 @@ PALM_API int palm_attention_decode(hipStream_t stream, const void* q, const void
                                    float* work, void* out) {
     return launch_attention_decode(stream, q, k_cache, v_cache, block_table, max_pages, seq_slot, seq_start, n_seqs, nh, nkv,
                                    hd, scale, window, n_slices, work, out);
+}
+
+// ---- decode with the q/k/v pass folded in -----------------------------------------------------------
+// The same grid and the same slices, but the kernel starts from the joined projection's output (whole rows, or
+// float32 planes of partial sums to be added) instead of a finished query: every wave adds the planes of its query
+// heads, norms and rotates them (the arithmetic of qk_norm_rope_store_kernel, with a lane holding chunks g, g + 4, ..
+// of its head, so that a rotation pair (i, i + HD/2) lies in one lane).  The cache does not hold the new position's
+// key and value yet: the slice whose pages include that position makes them too, writes them to the cache for the
+// steps to come, and starts its softmax state from them (one key: weight 1, the output the value itself); the pages
+// are then walked up to the position before.  A step saves a launch and the finished query's way through memory.
+// Served: head sizes that are multiples of 64 (the pair in one lane), and a rotation that is half-split over the
+// whole head, or none.
+constexpr bool FUSED_SERVES_HEAD = HD % 64 == 0;
+constexpr int LANE_ELEMS = (HD + WAVE - 1) / WAVE;          // elements d = lane + 64 i of a head that a lane holds
+constexpr int LANE_PAIRS = (HD / 2 + WAVE - 1) / WAVE;      // rotation pairs (i, i + HD/2), i = lane + 64 ii
+
+// Eight consecutive elements as they come from memory; widened only where they are used, so that a read can be
+// asked for long before.
+template <typename TIN> struct Raw8;
+template <> struct Raw8<float> {
+    float4 a, b;
+    __device__ void read(const float* p) { a = *reinterpret_cast<const float4*>(p); b = *reinterpret_cast<const float4*>(p + 4); }
+    __device__ void widen(float (&x)[8]) const { x[0] = a.x; x[1] = a.y; x[2] = a.z; x[3] = a.w; x[4] = b.x; x[5] = b.y; x[6] = b.z; x[7] = b.w; }
+};
+template <> struct Raw8<bf16_t> {
+    uint4 u;
+    __device__ void read(const bf16_t* p) { u = *reinterpret_cast<const uint4*>(p); }
+    __device__ void widen(float (&x)[8]) const {
+        x[0] = __uint_as_float(u.x << 16); x[1] = __uint_as_float(u.x & 0xffff0000u);
+        x[2] = __uint_as_float(u.y << 16); x[3] = __uint_as_float(u.y & 0xffff0000u);
+        x[4] = __uint_as_float(u.z << 16); x[5] = __uint_as_float(u.z & 0xffff0000u);
+        x[6] = __uint_as_float(u.w << 16); x[7] = __uint_as_float(u.w & 0xffff0000u);
+    }
+};
+
+// The step's rows and what is to be done with them.  ask() only asks memory for what does not depend on the
+// sequence's length (the rows, the norm weights, the rotation), so that it can stand at the kernel's very start and
+// the answers arrive while the page table is being looked up; prepare() does the arithmetic.
+template <typename TIN, int PLANES>
+struct FromProjection {
+    static constexpr int HELD = PLANES > 0 ? PLANES : 1;          // planes whose reads are on their way together
+    const TIN* q_row;  const TIN* k_row;  const TIN* v_row;      // this lane's query head, the kv head's key and value
+    int planes;  size_t plane_stride;
+    const float* q_norm_w;  const float* k_norm_w;  float eps;
+    const float* cos_row;  const float* sin_row;
+    float scale_log2;
+    bool valid;          // the lane's column is a query head
+    bool owner;          // this wave's slice holds the new position's page, and the layer writes its cache
+    bf16_t* k_dst;  bf16_t* v_dst;                               // where the new key's row and the new value's column start
+    int r, g, lane;
+    float* k_vals;  float* v_vals;                               // HD floats each in LDS
+    // asked for at the start
+    Raw8<TIN> q_raw[HELD][KSTEPS];
+    Raw8<float> qw_raw[KSTEPS], cos_raw[KSTEPS / 2 > 0 ? KSTEPS / 2 : 1], sin_raw[KSTEPS / 2 > 0 ? KSTEPS / 2 : 1];
+    TIN k_raw[HELD][LANE_ELEMS], v_raw[HELD][LANE_ELEMS];
+    float kw_raw[LANE_ELEMS], k_cos[LANE_PAIRS], k_sin[LANE_PAIRS];
+
+    __device__ void ask() {
+#pragma unroll
+        for (int pl = 0; pl < HELD; ++pl)
+#pragma unroll
+            for (int j = 0; j < KSTEPS; ++j) q_raw[pl][j].read(q_row + pl * plane_stride + (j * 4 + g) * 8);
+        if (q_norm_w) {
+#pragma unroll
+            for (int j = 0; j < KSTEPS; ++j) qw_raw[j].read(q_norm_w + (j * 4 + g) * 8);
+        }
+        if (cos_row) {
+#pragma unroll
+            for (int j = 0; j < KSTEPS / 2; ++j) {
+                cos_raw[j].read(cos_row + (j * 4 + g) * 8);
+                sin_raw[j].read(sin_row + (j * 4 + g) * 8);
+            }
+        }
+        // the new key and value, spread over the wave; every slice asks (a few bytes), the owner uses them
+#pragma unroll
+        for (int i = 0; i < LANE_ELEMS; ++i) {
+            const int d = lane + WAVE * i;
+#pragma unroll
+            for (int pl = 0; pl < HELD; ++pl) {
+                k_raw[pl][i] = k_row[pl * plane_stride + d];
+                v_raw[pl][i] = v_row[pl * plane_stride + d];
+            }
+            kw_raw[i] = k_norm_w ? k_norm_w[d] : 1.f;
+        }
+#pragma unroll
+        for (int ii = 0; ii < LANE_PAIRS; ++ii) {
+            const int i = min(lane + WAVE * ii, HD / 2 - 1);
+            k_cos[ii] = cos_row ? cos_row[i] : 1.f;
+            k_sin[ii] = cos_row ? sin_row[i] : 0.f;
+        }
+    }
+
+    __device__ void prepare(bf16x8 (&qv)[KSTEPS], Columns& c) {
+        // the query: planes added in their order, RMS norm over the head (the four lanes of a column share a head),
+        // rotation of (i, i + HD/2), rounding
+        float x[KSTEPS][8];
+#pragma unroll
+        for (int j = 0; j < KSTEPS; ++j) {
+            q_raw[0][j].widen(x[j]);
+#pragma unroll
+            for (int pl = 1; pl < HELD; ++pl) {
+                float y[8];
+                q_raw[pl][j].widen(y);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) x[j][e] += y[e];
+            }
+        }
+        if (PLANES == 0) {
+            for (int pl = 1; pl < planes; ++pl) {
+#pragma unroll
+                for (int j = 0; j < KSTEPS; ++j) {
+                    Raw8<TIN> more;
+                    float y[8];
+                    more.read(q_row + pl * plane_stride + (j * 4 + g) * 8);
+                    more.widen(y);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) x[j][e] += y[e];
+                }
+            }
+        }
+        if (q_norm_w) {
+            float ss = 0.f;
+#pragma unroll
+            for (int j = 0; j < KSTEPS; ++j)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) ss += x[j][e] * x[j][e];
+            ss += __shfl_xor(ss, 16, WAVE);
+            ss += __shfl_xor(ss, 32, WAVE);
+            const float inv = 1.0f / sqrtf(ss / (float)HD + eps);
+#pragma unroll
+            for (int j = 0; j < KSTEPS; ++j) {
+                float w[8];
+                qw_raw[j].widen(w);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) x[j][e] = x[j][e] * inv * w[e];
+            }
+        }
+        if (cos_row) {
+#pragma unroll
+            for (int j = 0; j < KSTEPS / 2; ++j) {
+                float cs[8], sn[8];
+                cos_raw[j].widen(cs);
+                sin_raw[j].widen(sn);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float x0 = x[j][e], x1 = x[j + KSTEPS / 2][e];
+                    x[j][e] = x0 * cs[e] - x1 * sn[e];
+                    x[j + KSTEPS / 2][e] = x0 * sn[e] + x1 * cs[e];
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < KSTEPS; ++j)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) qv[j][e] = valid ? (__bf16)x[j][e] : (__bf16)0.f;
+        if (!owner) return;
+
+        // the new key and value, element d = lane + 64 i in this lane, as qk_norm_rope_store_kernel makes them
+        float kx[LANE_ELEMS], vx[LANE_ELEMS], ss = 0.f;
+#pragma unroll
+        for (int i = 0; i < LANE_ELEMS; ++i) {
+            kx[i] = to_float(k_raw[0][i]);
+            vx[i] = to_float(v_raw[0][i]);
+#pragma unroll
+            for (int pl = 1; pl < HELD; ++pl) {
+                kx[i] += to_float(k_raw[pl][i]);
+                vx[i] += to_float(v_raw[pl][i]);
+            }
+            if (PLANES == 0) {
+                for (int pl = 1; pl < planes; ++pl) {
+                    kx[i] += to_float(k_row[pl * plane_stride + lane + WAVE * i]);
+                    vx[i] += to_float(v_row[pl * plane_stride + lane + WAVE * i]);
+                }
+            }
+            ss += kx[i] * kx[i];
+        }
+        if (k_norm_w) {
+            ss = wave_sum(ss);
+            const float inv = 1.0f / sqrtf(ss / (float)HD + eps);
+#pragma unroll
+            for (int i = 0; i < LANE_ELEMS; ++i) kx[i] = kx[i] * inv * kw_raw[i];
+        }
+#pragma unroll
+        for (int i = 0; i < LANE_ELEMS; ++i) {
+            const int d = lane + WAVE * i;
+            const bf16_t v_rounded = f32_to_bf16(vx[i]);
+            k_vals[d] = kx[i];
+            v_vals[d] = to_float(v_rounded);
+            v_dst[(size_t)d * PAGE_TOKENS] = v_rounded;
+        }
+        __syncthreads();                                 // the block is this one wave
+        if (cos_row) {
+#pragma unroll
+            for (int ii = 0; ii < LANE_PAIRS; ++ii) {
+                const int i = lane + WAVE * ii;
+                if (i < HD / 2) {
+                    const float x0 = k_vals[i], x1 = k_vals[i + HD / 2];
+                    k_vals[i] = x0 * k_cos[ii] - x1 * k_sin[ii];
+                    k_vals[i + HD / 2] = x0 * k_sin[ii] + x1 * k_cos[ii];
+                }
+            }
+            __syncthreads();
+        }
+        // its score against the finished query, both as the cache and the matrix cores hold them
+        float s = 0.f;
+#pragma unroll
+        for (int j = 0; j < KSTEPS; ++j) {
+            Raw8<float> chunk;
+            float kf[8];
+            bf16x8 kb;
+            chunk.read(k_vals + (j * 4 + g) * 8);
+            chunk.widen(kf);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                kb[e] = (__bf16)kf[e];
+                s += (float)qv[j][e] * (float)kb[e];
+            }
+            if (r == 0) *reinterpret_cast<bf16x8*>(k_dst + (j * 4 + g) * 8) = kb;      // lanes (0, g): the whole row
+        }
+        s += __shfl_xor(s, 16, WAVE);
+        s += __shfl_xor(s, 32, WAVE);
+        // one key: its weight is exp2(s - s) = 1; the sum's share lies with group 0, the others hold none
+        c.m = s * scale_log2;
+        c.l = g == 0 ? 1.f : 0.f;
+#pragma unroll
+        for (int dt = 0; dt < DTILES; ++dt) {           // this lane's output elements 16 dt + 4 g .. + 3
+            const float4 four = *reinterpret_cast<const float4*>(v_vals + dt * 16 + 4 * g);
+            c.o[dt] = f32x4{four.x, four.y, four.z, four.w};
+        }
+    }
+};
+
+template <typename TIN, int PLANES>
+__global__ __launch_bounds__(WAVE) DECODE_WAVES_PER_SIMD void attention_decode_fused_kernel(
+    const TIN* __restrict__ qkv, int planes, size_t plane_stride, const float* __restrict__ q_norm_w,
+    const float* __restrict__ k_norm_w, float eps, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+    int write_cache, bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache,
+    const int* __restrict__ block_table, int max_pages, const int* __restrict__ seq_slot,
+    const int* __restrict__ seq_start, int nh, int nkv, float scale_log2, int window, int n_slices,
+    float* __restrict__ work, bf16_t* __restrict__ out) {
+    if constexpr (FUSED_SERVES_HEAD) {
+        __shared__ float new_key[HD], new_value[HD];
+        const int slice = blockIdx.x, b = blockIdx.z;
+        const int G = nh / nkv, groups = (G + 15) / 16;
+        const int kvh = blockIdx.y / groups, qg = blockIdx.y % groups;
+        const int lane = threadIdx.x, r = lane % 16, g = lane / 16;
+        const int head = kvh * G + qg * 16 + r;
+        const bool valid = qg * 16 + r < G;
+
+        FromProjection<TIN, PLANES> start;
+        const TIN* row = qkv + (size_t)b * (nh + 2 * nkv) * HD;
+        start.q_row = row + (size_t)(valid ? head : 0) * HD;
+        start.k_row = row + (size_t)(nh + kvh) * HD;
+        start.v_row = row + (size_t)(nh + nkv + kvh) * HD;
+        start.planes = planes;
+        start.plane_stride = plane_stride;
+        start.q_norm_w = q_norm_w;
+        start.k_norm_w = k_norm_w;
+        start.eps = eps;
+        start.cos_row = cos_t ? cos_t + (size_t)b * (HD / 2) : nullptr;
+        start.sin_row = sin_t ? sin_t + (size_t)b * (HD / 2) : nullptr;
+        start.scale_log2 = scale_log2;
+        start.valid = valid;
+        start.r = r;
+        start.g = g;
+        start.lane = lane;
+        start.k_vals = new_key;
+        start.v_vals = new_value;
+        start.ask();
+
+        const int pos = seq_start[b];
+        const int first = window > 0 ? max(0, pos - window + 1) : 0;
+        const int page_lo = first / PAGE_TOKENS, n_pages = pos / PAGE_TOKENS - page_lo + 1;
+        const int per = (n_pages + n_slices - 1) / n_slices;
+        const int p0 = page_lo + slice * per, p1 = min(p0 + per, page_lo + n_pages);
+        const int* pages = block_table + (size_t)seq_slot[b] * max_pages;
+        const int page = pos / PAGE_TOKENS;
+        start.owner = write_cache && page >= p0 && page < p1;
+        start.k_dst = start.v_dst = nullptr;
+        if (start.owner) {
+            const size_t at = ((size_t)pages[page] * nkv + kvh) * PAGE_TOKENS * HD;
+            start.k_dst = k_cache + at + (size_t)(pos % PAGE_TOKENS) * HD;
+            start.v_dst = v_cache + at + pos % PAGE_TOKENS;
+        }
+
+        bf16x8 qv[KSTEPS];
+        Columns c;
+        c.m = -INFINITY;
+        c.l = 0.f;
+#pragma unroll
+        for (int dt = 0; dt < DTILES; ++dt) c.o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+        // with a key and value of its own making the step sees the cache up to the position before
+        attend_pages(k_cache, v_cache, pages, nkv, kvh, p0, p1, qv, first, write_cache ? pos - 1 : pos, scale_log2, c, r, g, start);
+        finish_slice(c, valid, b, head, nh, slice, n_slices, p0 >= p1, g, work, out);
+    }
+}
+
+PALM_API int palm_attention_decode_fused_serves(int rotary_dim, int pairing) {
+    return FUSED_SERVES_HEAD && (rotary_dim == 0 || (rotary_dim == HD && pairing == 0));
+}
+
+// qkv: [n_seqs, (nh + 2 nkv) hd] bfloat16 (qkv_is_planes = 0), or [planes, n_seqs, (nh + 2 nkv) hd] float32.
+// cos_t, sin_t: [n_seqs, hd / 2] float32 rows of the sequences' positions, or both null for no rotation.
+// Without write_cache the cache already holds the new position's key and value (a layer that reads another's).
+PALM_API int palm_attention_decode_fused(hipStream_t stream, const void* qkv, int qkv_is_planes, int planes,
+                                         const float* q_norm_w, const float* k_norm_w, float eps, const float* cos_t,
+                                         const float* sin_t, int rotary_dim, int pairing, int write_cache, void* k_cache,
+                                         void* v_cache, const int* block_table, int max_pages, const int* seq_slot,
+                                         const int* seq_start, int n_seqs, int nh, int nkv, int hd, float scale,
+                                         int window, int n_slices, float* work, void* out) {
+    PALM_CHECK(hd == HD, "attention_decode_fused: this library was built for head size %d, not %d", HD, hd);
+    PALM_CHECK((cos_t == nullptr) == (sin_t == nullptr), "attention_decode_fused: cos and sin tables come together");
+    PALM_CHECK(palm_attention_decode_fused_serves(cos_t ? rotary_dim : 0, pairing),
+               "attention_decode_fused: head size %d with rotation over %d (pairing %d) is not served: the head size must be a "
+               "multiple of 64 and the rotation half-split over the whole head, or absent", HD, rotary_dim, pairing);
+    PALM_CHECK((q_norm_w == nullptr) == (k_norm_w == nullptr), "attention_decode_fused: q and k norm weights come together");
+    PALM_CHECK(n_seqs >= 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attention_decode_fused: seqs=%d heads=%d kv=%d", n_seqs, nh, nkv);
+    PALM_CHECK(n_slices >= 1 && n_slices <= 65535, "attention_decode_fused: %d slices", n_slices);
+    PALM_CHECK(n_slices == 1 || work, "attention_decode_fused: more than one slice needs a workspace");
+    PALM_CHECK(window >= 0 && max_pages > 0, "attention_decode_fused: window=%d max_pages=%d", window, max_pages);
+    PALM_CHECK(planes >= 1 && (qkv_is_planes || planes == 1), "attention_decode_fused: %d planes of whole rows", planes);
+    if (n_seqs == 0) return 0;
+    const int groups = (nh / nkv + 15) / 16;
+    PALM_CHECK(nkv * groups <= 65535 && n_seqs <= 65535, "attention_decode_fused: grid too large");
+    dim3 grid(n_slices, nkv * groups, n_seqs);
+    const size_t plane_stride = (size_t)n_seqs * (nh + 2 * nkv) * HD;
+#define PALM_FUSED(TIN, P) attention_decode_fused_kernel<TIN, P><<<grid, WAVE, 0, stream>>>( \
+        (const TIN*)qkv, planes, plane_stride, q_norm_w, k_norm_w, eps, cos_t, sin_t, write_cache, (bf16_t*)k_cache, \
+        (bf16_t*)v_cache, block_table, max_pages, seq_slot, seq_start, nh, nkv, scale * LOG2E, window, n_slices, work, (bf16_t*)out)
+    if (!qkv_is_planes) PALM_FUSED(bf16_t, 1);
+    else if (planes == 1) PALM_FUSED(float, 1);
+    else if (planes == 2) PALM_FUSED(float, 2);
+    else PALM_FUSED(float, 0);
+#undef PALM_FUSED
+    PALM_LAUNCHED();
+    if (n_slices > 1) {
+        attention_merge_kernel<<<n_seqs * nh, WAVE, 0, stream>>>(work, n_slices, nh, seq_start, window, (bf16_t*)out);
+        PALM_LAUNCHED();
+    }
+    return 0;
 }
 
 // ---- decode without a workspace argument ------------------------------------------------------------

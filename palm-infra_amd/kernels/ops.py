@@ -225,6 +225,7 @@ def qk_norm_rope_store(qkv: torch.Tensor, nh: int, nkv: int, hd: int, positions:
         planes = qkv.shape[0]
         _need(qkv.dtype == F32 and qkv.is_contiguous() and out_dtype is not None,
               "qk_norm_rope_store: planes are contiguous float32 and come with the type of the result")
+        _need(planes >= 2 or out_dtype == F32, "qk_norm_rope_store: a single plane comes as rows of the result's type")
         n = qkv.shape[1]
     else:
         _need(qkv.dim() == 2, f"qk_norm_rope_store: qkv {tuple(qkv.shape)}")
@@ -536,6 +537,10 @@ _ATTENTION_SIGNATURES = {
                               c_int, c_int, c_float, c_int, c_int, c_void_p, c_void_p],
     "palm_attention_prefill": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
                                c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
+    "palm_attention_decode_fused": [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_int,
+                                    c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int,
+                                    c_int, c_int, c_float, c_int, c_int, c_void_p, c_void_p],
+    "palm_attention_decode_fused_serves": [c_int, c_int],
 }
 _attention_libs: dict = {}
 MFMA_HEAD_DIMS = tuple(range(16, 257, 16))
@@ -590,6 +595,50 @@ def attention_decode(q, k_cache, v_cache, block_table, seq_slot, seq_start, nh: 
     return out
 
 
+def decode_fused_serves(qkv: torch.Tensor, hd: int, out_dtype, rotary_dim: int, pairing: int) -> bool:
+    """Whether attention_decode_fused takes this step's q/k/v rows: bfloat16 attention on the matrix cores, a head
+    size and a rotation for which a rotation pair lies in one lane."""
+    if out_dtype != BF16 or hd not in MFMA_HEAD_DIMS:
+        return False
+    if not (qkv.dim() == 3 and qkv.dtype == F32 or qkv.dim() == 2 and qkv.dtype == BF16):
+        return False
+    return bool(attention_lib(hd).palm_attention_decode_fused_serves(int(rotary_dim), int(pairing)))
+
+
+def attention_decode_fused(qkv, k_cache, v_cache, block_table, seq_slot, seq_start, nh: int, nkv: int, hd: int, scale: float,
+                           window: int | None, n_slices: int, *, q_norm_w=None, k_norm_w=None, eps: float = 0.0, cos=None,
+                           sin=None, rotary_dim: int = 0, pairing: int = 0, write_cache: bool = True) -> torch.Tensor:
+    """A decode step's attention from the joined projection's rows: qk_norm_rope_store and attention_decode in one
+    launch.  qkv is [B, (nh + 2 nkv) hd] bfloat16 or float32 planes [P, B, (nh + 2 nkv) hd]; sequence b's token is
+    row b, at position seq_start[b]; cos, sin are [B, hd / 2] rows of those positions.  Returns [B, nh hd] bfloat16."""
+    what = "attention_decode_fused"
+    _dev(what, qkv, k_cache, v_cache, block_table, seq_slot, seq_start, q_norm_w, k_norm_w, cos, sin)
+    _i32(what, block_table, seq_slot, seq_start)
+    as_planes = qkv.dim() == 3
+    _need(qkv.is_contiguous() and (as_planes and qkv.dtype == F32 or qkv.dim() == 2 and qkv.dtype == BF16),
+          f"{what}: qkv {tuple(qkv.shape)} {qkv.dtype} is neither bfloat16 rows nor float32 planes")
+    B = seq_slot.shape[0]
+    _need(qkv.shape[-2] == B and qkv.shape[-1] == (nh + 2 * nkv) * hd and seq_start.shape == (B,),
+          f"{what}: qkv {tuple(qkv.shape)} is not [.., {B}, ({nh} + 2*{nkv}) * {hd}]")
+    _need(nh % nkv == 0, f"{what}: {nh} heads are not a multiple of {nkv} kv heads")
+    _check_cache(what, k_cache, v_cache, block_table, nkv, hd)
+    _need(k_cache.dtype == BF16, f"{what}: the cache is {k_cache.dtype}, not bfloat16")
+    for w, nm in ((q_norm_w, "q"), (k_norm_w, "k")):
+        _need(w is None or (w.shape == (hd,) and w.dtype == F32), f"{what}: {nm} norm weight must be float32 [{hd}]")
+    _need((cos is None) == (sin is None), f"{what}: cos and sin come together")
+    for tab in (cos, sin):
+        _need(tab is None or (tab.dtype == F32 and tab.shape == (B, hd // 2) and tab.is_contiguous() and rotary_dim == hd),
+              f"{what}: a rotation table is float32 [{B}, {hd // 2}] over the whole head")
+    out = torch.empty((B, nh * hd), dtype=BF16, device=qkv.device)
+    work = torch.empty((B * nh * n_slices * (hd + 4),), dtype=F32, device=qkv.device) if n_slices > 1 else None
+    library.call(attention_lib(hd), "palm_attention_decode_fused", _stream(), _p(qkv), int(as_planes),
+                 qkv.shape[0] if as_planes else 1, _p(q_norm_w), _p(k_norm_w), float(eps), _p(cos), _p(sin),
+                 int(rotary_dim if cos is not None else 0), int(pairing), int(write_cache), _p(k_cache), _p(v_cache),
+                 _p(block_table), block_table.shape[1], _p(seq_slot), _p(seq_start), B, nh, nkv, hd, float(scale),
+                 int(window or 0), int(n_slices), _p(work), _p(out))
+    return out
+
+
 def attention_prefill(q, k_cache, v_cache, block_table, seq_slot, seq_start, seq_new, cu_new, max_new: int, nh: int,
                       nkv: int, hd: int, scale: float, window: int | None) -> torch.Tensor:
     """The step's queries (several for each sequence) over the cache, on the matrix cores."""
@@ -604,12 +653,17 @@ def attention_prefill(q, k_cache, v_cache, block_table, seq_slot, seq_start, seq
     return out
 
 
+def slices_of_step(ctx, nh: int, nkv: int, window: int | None) -> int:
+    """The slices of a decode step's key ranges: what a recorded step was cut for, else what fills the chip."""
+    keys = min(ctx.max_total, window) if window else ctx.max_total
+    return ctx.decode_slices or decode_slices(ctx.n_seqs, nh, nkv, keys)
+
+
 def attention(q, k_cache, v_cache, block_table, ctx, nh: int, nkv: int, hd: int, scale: float, window: int | None):
     """The step's queries over the cache; picks the kernel by element type, head size and step shape."""
     if mfma_attention_serves(q, hd):
         if ctx.is_decode:
-            keys = min(ctx.max_total, window) if window else ctx.max_total
-            n_slices = ctx.decode_slices or decode_slices(ctx.n_seqs, nh, nkv, keys)
+            n_slices = slices_of_step(ctx, nh, nkv, window)
             return attention_decode(q, k_cache, v_cache, block_table, ctx.seq_slot, ctx.seq_start, nh, nkv, hd, scale,
                                     window, n_slices)
         return attention_prefill(q, k_cache, v_cache, block_table, ctx.seq_slot, ctx.seq_start, ctx.seq_new, ctx.cu_new,

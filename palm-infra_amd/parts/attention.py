@@ -59,12 +59,23 @@ class Attention:
         qkv = self.qkv(h, planes_ok=True)
         tables = self.position.tables(ctx) if self.position is not None else None
         cos, sin = tables if tables is not None else (None, None)
+        rotary_dim = self.position.rotary_dim if tables is not None else 0
+        pairing = PAIRINGS[self.position.pairing] if tables is not None else 0
+        if ctx.is_decode and ops.decode_fused_serves(qkv, self.hd, self.dtype, rotary_dim, pairing):
+            # one token a sequence: its slot and position are the sequence's, and the q/k/v pass rides in the
+            # attention kernel
+            o = ops.attention_decode_fused(
+                qkv, lc.k, lc.v, lc.kv.table_dev, ctx.seq_slot, ctx.seq_start, self.nh, self.nkv, self.hd, self.scale,
+                self.window, ops.slices_of_step(ctx, self.nh, self.nkv, self.window),
+                q_norm_w=self.q_norm.weight if self.q_norm else None, k_norm_w=self.k_norm.weight if self.k_norm else None,
+                eps=self.q_norm.eps if self.q_norm else 0.0, cos=cos, sin=sin, rotary_dim=rotary_dim, pairing=pairing,
+                write_cache=lc.writes)
+            return self.out(o, sink=sink)
         q = ops.qk_norm_rope_store(
             qkv, self.nh, self.nkv, self.hd, ctx.positions,
             q_norm_w=self.q_norm.weight if self.q_norm else None, k_norm_w=self.k_norm.weight if self.k_norm else None,
             eps=self.q_norm.eps if self.q_norm else 0.0, cos=cos, sin=sin,
-            rotary_dim=self.position.rotary_dim if tables is not None else 0,
-            pairing=PAIRINGS[self.position.pairing] if tables is not None else 0,
+            rotary_dim=rotary_dim, pairing=pairing,
             k_cache=lc.k, v_cache=lc.v, block_table=lc.kv.table_dev, tok_slot=ctx.tok_slot, write_cache=lc.writes,
             out_dtype=self.dtype)
         o = ops.attention(q, lc.k, lc.v, lc.kv.table_dev, ctx, self.nh, self.nkv, self.hd, self.scale, self.window)

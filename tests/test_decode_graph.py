@@ -9,7 +9,7 @@ import tiny
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("name,dtype", [("A", "float32"), ("B", "bfloat16"), ("C", "bfloat16")])
+@pytest.mark.parametrize("name,dtype", [("A", "float32"), ("B", "bfloat16"), ("C", "bfloat16"), ("D", "bfloat16")])
 def test_replays_equal_plain_launches(model_dirs, name, dtype):
     from palm_infra_amd.engine import Engine, StepEntry
     g = Engine.from_dir(model_dirs[name][dtype], dtype=dtype, max_tokens=64 * 40, graphs=True)

@@ -10,8 +10,9 @@ import tiny
 
 pytestmark = pytest.mark.gpu
 
-CASES = [(name, dtype) for name in ("A", "B", "C") for dtype in ("float32", "bfloat16")]
-LENGTHS = {"A": [5, 17, 9, 64, 100, 33], "B": [1, 31, 12, 64, 65, 200], "C": [48, 7, 129, 2, 300, 70]}
+CASES = [(name, dtype) for name in ("A", "B", "C", "D") for dtype in ("float32", "bfloat16")]
+LENGTHS = {"A": [5, 17, 9, 64, 100, 33], "B": [1, 31, 12, 64, 65, 200], "C": [48, 7, 129, 2, 300, 70],
+           "D": [64, 3, 65, 129, 1, 40]}
 
 _engines = {}
 _refs = {}
@@ -101,7 +102,7 @@ def test_batches_of_unequal_lengths_one_after_another(model_dirs, name, dtype):
         assert eng.cache.kv_groups[0].table.pages.held_count == held_before
 
 
-@pytest.mark.parametrize("name,dtype", [("C", "float32"), ("C", "bfloat16"), ("B", "float32")])
+@pytest.mark.parametrize("name,dtype", [("C", "float32"), ("C", "bfloat16"), ("B", "float32"), ("D", "bfloat16")])
 def test_long_decoding(model_dirs, name, dtype):
     """A short prompt, then every further token one by one, across several pages."""
     from palm_infra_amd.engine import StepEntry
@@ -301,3 +302,21 @@ def test_decode_steps_of_more_sequences_than_a_recorded_step_takes(model_dirs, d
     for i in live:
         eng.close(slots[i])
     eng.cache.check()
+
+
+def test_which_decode_steps_take_the_attention_that_starts_from_the_projection(model_dirs, monkeypatch):
+    """Heads of 64 in bfloat16 do (once a layer), heads of 48 and float32 steps do not; prompts never."""
+    from palm_infra_amd.engine import Engine, StepEntry
+    from palm_infra_amd.kernels import ops
+    calls = []
+    real = ops.attention_decode_fused
+    monkeypatch.setattr(ops, "attention_decode_fused", lambda *a, **k: (calls.append(1), real(*a, **k))[1])
+    for name, dtype, expected in (("D", "bfloat16", tiny.CONFIGS["D"]["num_hidden_layers"]), ("D", "float32", 0), ("C", "bfloat16", 0)):
+        eng = Engine.from_dir(model_dirs[name][dtype], dtype=dtype, max_tokens=64 * 4, graphs=False)
+        slot = eng.open()
+        eng.step([StepEntry(slot, [1, 2, 3], [2])])
+        assert not calls
+        eng.step([StepEntry(slot, [4], [0])])
+        assert len(calls) == expected, (name, dtype)
+        calls.clear()
+        eng.close(slot)

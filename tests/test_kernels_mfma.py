@@ -1,6 +1,7 @@
 """The matrix-core kernels alone against their plain references: the thin linear product (with and
 without the gated epilogue) and the bfloat16 attention kernels, at sizes other than the tiny models'."""
 
+import numpy as np
 import pytest
 import torch
 
@@ -289,7 +290,7 @@ def test_linear_tile_refuses_what_it_does_not_serve(ops):
 
 # ---- attention on the matrix cores ------------------------------------------------------------------
 
-from test_kernels import _attention_case, _spike_case  # noqa: E402  (the cases and the cache filling are shared)
+from test_kernels import _attention_case, _fill_cache, _spike_case  # noqa: E402  (the cases and the cache filling are shared)
 
 
 def decode_fn(ops, n_slices):
@@ -375,3 +376,130 @@ def test_attention_mfma_refuses_what_it_was_not_built_for(ops):
     i32 = lambda xs: torch.tensor(xs, dtype=torch.int32).to(DEV)
     with pytest.raises(KernelError, match="bfloat16"):
         ops.attention_decode(q, kc, vc, i32([[0, 1]]), i32([0]), i32([3]), 2, 1, 32, 1.0, None, 1)
+
+
+# ---- decode attention that starts from the joined projection's rows -----------------------------------
+
+def _fused_case(ops, nh, nkv, hd, lengths, n_slices, planes, window=None, norm=True, rotate=True, seed=0):
+    """Sequences whose last token is new: its q/k/v row goes (a) through qk_norm_rope_store and attention_decode and
+    (b) through attention_decode_fused, each on its own copy of a cache that holds the earlier tokens and stale
+    values elsewhere.  Returns both outputs and both pairs of caches."""
+    B, W = len(lengths), (nh + 2 * nkv) * hd
+    n_pages = sum((L + 63) // 64 for L in lengths) + 2
+    perm = torch.randperm(n_pages - 1, generator=torch.Generator().manual_seed(seed)).tolist()
+    max_pages = max((L + 63) // 64 for L in lengths) + 1
+    slots = torch.randperm(B + 3, generator=torch.Generator().manual_seed(seed + 7)).tolist()[:B]
+    table = torch.full((B + 3, max_pages), n_pages - 1, dtype=torch.int32)
+    kc = rand(n_pages, nkv, 64, hd, seed=seed + 50).to(DEV)
+    vc = rand(n_pages, nkv, hd, 64, seed=seed + 51).to(DEV)
+    o = 0
+    for b, L in enumerate(lengths):
+        npg = (L + 63) // 64
+        table[slots[b], :npg] = torch.tensor(perm[o:o + npg], dtype=torch.int32)
+        o += npg
+        if L > 1:
+            _fill_cache(kc, vc, table, slots[b], rand(L - 1, nkv, hd, seed=seed + 10 * b + 1).to(DEV),
+                        rand(L - 1, nkv, hd, seed=seed + 10 * b + 2).to(DEV))
+    if planes == 0:
+        qkv = rand(B, W, seed=seed + 3, scale=1.5).to(DEV)
+    else:
+        qkv = rand(planes, B, W, seed=seed + 3, scale=1.5, dtype=F32).to(DEV)
+    i32 = lambda xs: torch.tensor(xs, dtype=torch.int32).to(DEV)
+    pos, slot = i32([L - 1 for L in lengths]), i32(slots)
+    kw = dict(q_norm_w=(1 + 0.3 * rand(hd, seed=seed + 4, dtype=F32)).to(DEV) if norm else None,
+              k_norm_w=(1 + 0.3 * rand(hd, seed=seed + 5, dtype=F32)).to(DEV) if norm else None, eps=1e-5 if norm else 0.0)
+    if rotate:
+        inv = torch.from_numpy((1.0 / np.power(10000.0, np.arange(hd // 2, dtype=np.float32) * 2 / hd)).astype(np.float32))
+        cos, sin = ops.rope_table(pos, inv.to(DEV))
+        kw.update(cos=cos, sin=sin, rotary_dim=hd, pairing=0)
+    ka, va, kb, vb = kc.clone(), vc.clone(), kc.clone(), vc.clone()
+    tab = table.to(DEV)
+    apart = torch.cat([qkv, torch.zeros_like(qkv)]) if planes == 1 else qkv          # the pass alone takes two planes or more
+    q = ops.qk_norm_rope_store(apart, nh, nkv, hd, pos, k_cache=ka, v_cache=va, block_table=tab, tok_slot=slot, out_dtype=BF16, **kw)
+    two = ops.attention_decode(q, ka, va, tab, slot, pos, nh, nkv, hd, hd ** -0.5, window, n_slices)
+    one = ops.attention_decode_fused(qkv, kb, vb, tab, slot, pos, nh, nkv, hd, hd ** -0.5, window, n_slices, **kw)
+    return one.float().cpu(), two.float().cpu(), (ka.cpu(), va.cpu()), (kb.cpu(), vb.cpu()), (kc.cpu(), vc.cpu())
+
+
+def _one_ulp(a, b):
+    """Both are rounded to bfloat16 from sums made in another order: a step of the last bit (2^-8 of the value, and
+    values here reach 8) on top of the attention kernels' own tolerance."""
+    return torch.allclose(a, b, rtol=2 ** -7, atol=2e-2)
+
+
+def _same_caches(a, b):
+    """Keys and values written by the two paths: the same but for an element's last bit now and then (the sums of
+    squares are added in another order)."""
+    for x, y in zip(a, b):
+        x, y = x.float(), y.float()
+        assert torch.allclose(x, y, rtol=2 ** -7, atol=1e-6), float((x - y).abs().max())
+        assert float((x != y).float().mean()) < 1e-3
+
+
+@pytest.mark.parametrize("nh,nkv,hd", [(4, 2, 128), (32, 8, 128), (6, 3, 64), (40, 2, 64), (3, 3, 256), (4, 1, 192)])
+@pytest.mark.parametrize("n_slices", [1, 3, 8])
+def test_attention_decode_fused_is_the_two_kernels_in_one(ops, nh, nkv, hd, n_slices):
+    """Lengths around page borders (the new token first in its page, last in it, the only one of its sequence), rows
+    as bfloat16 and as one, two and three planes."""
+    for planes, lengths in ((0, [300]), (1, [1]), (2, [64, 65, 700, 7, 128, 129, 1]), (3, [193, 2])):
+        one, two, ca, cb, before = _fused_case(ops, nh, nkv, hd, lengths, n_slices, planes, seed=hd + planes)
+        assert _one_ulp(one, two), (planes, lengths, float((one - two).abs().max()))
+        _same_caches(ca, cb)
+        assert not torch.equal(cb[0], before[0]) and not torch.equal(cb[1], before[1])      # it did write
+
+
+def test_attention_decode_fused_with_a_window_without_norm_and_without_rotation(ops):
+    for window in (1, 5, 64, 100):
+        for n_slices in (1, 4):
+            one, two, ca, cb, _ = _fused_case(ops, 4, 2, 64, [200, 150, 3, 65], n_slices, 2, window=window, seed=window)
+            assert _one_ulp(one, two), (window, n_slices, float((one - two).abs().max()))
+            _same_caches(ca, cb)
+    for norm, rotate in ((False, True), (True, False), (False, False)):
+        one, two, ca, cb, _ = _fused_case(ops, 8, 2, 128, [200, 64, 65], 3, 2, norm=norm, rotate=rotate, seed=9)
+        assert _one_ulp(one, two), (norm, rotate, float((one - two).abs().max()))
+        _same_caches(ca, cb)
+
+
+def test_attention_decode_fused_sees_its_own_key_and_leaves_a_read_only_cache_alone(ops):
+    """The new token's key is made to dominate: the output is its value, which only the step's row holds.  A layer
+    that reads another layer's cache writes nothing and reads the position from the cache."""
+    nh, nkv, hd = 4, 2, 128
+    W = (nh + 2 * nkv) * hd
+    i32 = lambda xs: torch.tensor(xs, dtype=torch.int32).to(DEV)
+    for L in (1, 64, 65, 300):
+        for n_slices in (1, 4):
+            table = torch.arange((L + 63) // 64 + 1, dtype=torch.int32).flip(0)[None, :].contiguous()
+            kc, vc = 0.1 * rand(table.shape[1], nkv, 64, hd, seed=1), rand(table.shape[1], nkv, hd, 64, seed=2)
+            row = 0.1 * rand(1, W, seed=3)
+            row[0, : (nh + nkv) * hd].reshape(nh + nkv, hd)[:, 5] = 8.0          # every q and k head: one large element
+            kd, vd = kc.to(DEV), vc.to(DEV)
+            got = ops.attention_decode_fused(row.to(DEV), kd, vd, table.to(DEV), i32([0]), i32([L - 1]), nh, nkv, hd, 1.0, None, n_slices)
+            v_new = row[0, (nh + nkv) * hd:].reshape(nkv, hd).float()
+            want = v_new.repeat_interleave(nh // nkv, 0).reshape(1, nh * hd)
+            assert torch.allclose(got.float().cpu(), want, atol=1e-2), (L, n_slices)
+            page = int(table[0, (L - 1) // 64])
+            assert torch.equal(vd[page, :, :, (L - 1) % 64].cpu(), row[0, (nh + nkv) * hd:].reshape(nkv, hd))
+            assert torch.equal(kd[page, :, (L - 1) % 64].cpu(), row[0, nh * hd:(nh + nkv) * hd].reshape(nkv, hd))
+            # read only: the cache as the writing call left it gives the same result, and stays as it is
+            k2, v2 = kd.clone(), vd.clone()
+            other = 0.1 * rand(1, W, seed=4)
+            other[0, : nh * hd] = row[0, : nh * hd]
+            again = ops.attention_decode_fused(other.to(DEV), k2, v2, table.to(DEV), i32([0]), i32([L - 1]), nh, nkv, hd, 1.0, None,
+                                               n_slices, write_cache=False)
+            assert torch.allclose(again.float().cpu(), want, atol=1e-2)
+            assert torch.equal(k2, kd) and torch.equal(v2, vd)
+
+
+def test_attention_decode_fused_says_what_it_serves(ops):
+    from palm_infra_amd.kernels import KernelError
+    planes = torch.zeros(2, 1, 4 * 128, dtype=F32, device=DEV)
+    assert ops.decode_fused_serves(planes, 128, BF16, 128, 0) and ops.decode_fused_serves(planes, 64, BF16, 0, 0)
+    assert not ops.decode_fused_serves(planes, 128, BF16, 64, 0)          # a rotation over half the head
+    assert not ops.decode_fused_serves(planes, 128, BF16, 128, 1)         # pairs side by side
+    assert not ops.decode_fused_serves(planes, 80, BF16, 80, 0)           # a pair would lie in two lanes
+    assert not ops.decode_fused_serves(planes, 128, F32, 128, 0)
+    qkv = torch.zeros(1, 4 * 80, dtype=BF16, device=DEV)
+    kc, vc = torch.zeros(2, 1, 64, 80, dtype=BF16, device=DEV), torch.zeros(2, 1, 80, 64, dtype=BF16, device=DEV)
+    i32 = lambda xs: torch.tensor(xs, dtype=torch.int32).to(DEV)
+    with pytest.raises(KernelError, match="multiple of 64"):
+        ops.attention_decode_fused(qkv, kc, vc, i32([[0, 1]]), i32([0]), i32([3]), 2, 1, 80, 1.0, None, 1)

@@ -3,7 +3,8 @@
 A and B differ in every size and option (layers, width, heads and groups, head size, heads*head_dim equal
 to the width or not, a feed-forward width that is no power of two, vocabulary, rotation base, eps, tied or
 untied head); C adds head sizes and widths that are no power of two at all, one kv head per head, and
-room for long sequences.
+room for long sequences; D has heads of 64, the smallest size at which a bfloat16 decode step takes the attention
+kernel that starts from the joined projection's rows, and two heads a kv head.
 
 The weights are the random-weights mode's, then sharpened so that faults show: matrices are four times
 larger (logits of order one instead of a tenth) and the q norm's weight is four times larger, which makes
@@ -32,8 +33,11 @@ CONFIGS = {
     "C": dict(_BASE, vocab_size=515, hidden_size=80, num_hidden_layers=2, num_attention_heads=5, num_key_value_heads=5,
               head_dim=48, intermediate_size=176, tie_word_embeddings=False, rope_theta=500000.0, rms_norm_eps=3e-6,
               max_position_embeddings=2048),
+    "D": dict(_BASE, vocab_size=300, hidden_size=88, num_hidden_layers=2, num_attention_heads=6, num_key_value_heads=3,
+              head_dim=64, intermediate_size=200, tie_word_embeddings=True, rope_theta=20000.0, rms_norm_eps=2e-6,
+              max_position_embeddings=512, eos_token_id=5),
 }
-SEEDS = {"A": 0, "B": 1, "C": 2}
+SEEDS = {"A": 0, "B": 1, "C": 2, "D": 3}
 
 
 def sharpened_tensors(name: str, store: str) -> dict[str, torch.Tensor]:
