@@ -14,6 +14,16 @@ PALM_API int palm_attention_decode(hipStream_t stream, const void* q, const void
                                    int n_seqs, int nh, int nkv, int hd, float scale, int window, int n_slices,
                                    float* work, void* out);
 
+// The same from the joined q/k/v projection's rows of the step's tokens (bfloat16 rows, or float32 planes of partial
+// sums to be added): per-head RMS norm of q and k, rotation, the new key and value into the cache, attention.
+PALM_API int palm_attention_decode_fused_serves(int rotary_dim, int pairing);
+PALM_API int palm_attention_decode_fused(hipStream_t stream, const void* qkv, int qkv_is_planes, int planes,
+                                         const float* q_norm_w, const float* k_norm_w, float eps, const float* cos_t,
+                                         const float* sin_t, int rotary_dim, int pairing, int write_cache, void* k_cache,
+                                         void* v_cache, const int* block_table, int max_pages, const int* seq_slot,
+                                         const int* seq_start, int n_seqs, int nh, int nkv, int hd, float scale,
+                                         int window, int n_slices, float* work, void* out);
+
 // The same computation for callers that cannot allocate: code under HIP graph capture, tight serving loops,
 // harnesses that forbid hipMalloc.  It has no counterpart in the reference (whose decode attention is a single
 // kernel without a workspace, engine/cuda_attention.cu).  It takes no workspace: the slices' partial results go

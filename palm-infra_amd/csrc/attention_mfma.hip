@@ -249,48 +249,58 @@ __global__ __launch_bounds__(WAVE) DECODE_WAVES_PER_SIMD void attention_decode_k
     finish_slice(c, valid, b, head, nh, slice, n_slices, p0 >= p1, g, work, out);
 }
 
-// One wave per (sequence, head): merge the slices in a fixed order.  Lane s first reads slice s's maximum
-// and sum (all at once), the wave agrees on the overall maximum and on each slice's weight, then lane d sums
-// output element d over the slices, eight reads in flight at a time.  Only the slices that hold pages of this
-// sequence are read: a launch is cut for the longest sequence a recorded step may serve, and a shorter one leaves
-// its last slices empty (one sequence of 2,048 tokens in a step recorded for 4,096: 33 of 64).
+// One wave per (sequence, head): merge the slices in a fixed order.  Lane s holds slice s's maximum and sum, the wave
+// agrees on the overall maximum and on each slice's weight, then lane d sums output element d over the slices,
+// AT_ONCE reads in flight at a time.  The kernel is a few KB of reads and its time is the round trips to memory
+// that follow each other, so the maxima, the sums and the first round of outputs (all of them in the usual step) are
+// asked for in the first instructions, before the sequence's length is known: a slice beyond those that hold pages
+// of this sequence is read like the others (a launch is cut for the longest sequence a recorded step may serve; a
+// shorter one's last records exist but hold what an earlier step left: one sequence of 2,048 tokens in a step
+// recorded for 4,096 fills 33 of 64) and counts as nothing by a select.  (8 sequences, 12 slices: a step of 36 layers
+// 4.04 ms against 4.12 with the reads where they are used.)
+template <int AT_ONCE>
 __global__ __launch_bounds__(WAVE) void attention_merge_kernel(const float* __restrict__ work, int n_slices, int nh,
                                                                const int* __restrict__ seq_start, int window,
                                                                bf16_t* __restrict__ out) {
+    constexpr int PER = (HD + WAVE - 1) / WAVE;
     const float* w = work + (size_t)blockIdx.x * n_slices * WORK_STRIDE;
     const int lane = threadIdx.x;
+    // asked for before the sequence's length is known: lane s's slice's maximum and sum, and the first round of outputs
+    const float2 mine = *reinterpret_cast<const float2*>(w + (size_t)min(lane, n_slices - 1) * WORK_STRIDE);
+    float v[AT_ONCE][PER];
+    auto ask = [&](int s0) {
+#pragma unroll
+        for (int u = 0; u < AT_ONCE; ++u) {
+            const float* rec = w + (size_t)min(s0 + u, n_slices - 1) * WORK_STRIDE + WORK_O;
+#pragma unroll
+            for (int i = 0; i < PER; ++i) v[u][i] = rec[min(lane + i * WAVE, HD - 1)];
+        }
+    };
+    ask(0);
     const int pos = seq_start[blockIdx.x / nh];
     const int first = window > 0 ? max(0, pos - window + 1) : 0;
     const int n_pages = pos / PAGE_TOKENS - first / PAGE_TOKENS + 1;
     const int per = (n_pages + n_slices - 1) / n_slices;
-    const int live = (n_pages + per - 1) / per;                 // as attention_decode_kernel cuts the range: <= n_slices
-    float m = -INFINITY;
-    for (int s = lane; s < live; s += WAVE) m = fmaxf(m, w[(size_t)s * WORK_STRIDE]);
+    const int live = (n_pages + per - 1) / per;                 // as the decode kernels cut the range: <= n_slices
+    float m = lane < live ? mine.x : -INFINITY, l = 0.f;
+    for (int s = lane + WAVE; s < live; s += WAVE) m = fmaxf(m, w[(size_t)s * WORK_STRIDE]);
     m = wave_max(m);
-    float l = 0.f;
-    for (int s = lane; s < live; s += WAVE) l += w[(size_t)s * WORK_STRIDE + 1] * exp2f(w[(size_t)s * WORK_STRIDE] - m);
+    float wt = lane < live ? exp2_weight(mine.x - m) : 0.f;     // slice `lane`'s weight
+    l = lane < live ? mine.y * wt : 0.f;
+    for (int s = lane + WAVE; s < live; s += WAVE) l += w[(size_t)s * WORK_STRIDE + 1] * exp2_weight(w[(size_t)s * WORK_STRIDE] - m);
     l = wave_sum(l);
-    constexpr int PER = (HD + WAVE - 1) / WAVE;
     float o[PER];
 #pragma unroll
     for (int i = 0; i < PER; ++i) o[i] = 0.f;
-    for (int s0 = 0; s0 < live; s0 += 8) {
-        float ms[8], v[8][PER];
+    for (int s0 = 0; s0 < live; s0 += AT_ONCE) {
+        if (s0 > 0) ask(s0);
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-            const int s = min(s0 + u, live - 1);
-            ms[u] = w[(size_t)s * WORK_STRIDE];
+        for (int u = 0; u < AT_ONCE; ++u) {
+            const int s = s0 + u;
+            float ws = 0.f;
+            if (s < live) ws = s < WAVE ? __shfl(wt, s, WAVE) : exp2_weight(w[(size_t)s * WORK_STRIDE] - m);
 #pragma unroll
-            for (int i = 0; i < PER; ++i) {
-                const int d = min(lane + i * WAVE, HD - 1);
-                v[u][i] = w[(size_t)s * WORK_STRIDE + WORK_O + d];
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < 8; ++u) {
-            const float wt = s0 + u < live ? exp2f(ms[u] - m) : 0.f;
-#pragma unroll
-            for (int i = 0; i < PER; ++i) o[i] += v[u][i] * wt;
+            for (int i = 0; i < PER; ++i) o[i] += s < live ? v[u][i] * ws : 0.f;
         }
     }
 #pragma unroll
@@ -298,6 +308,14 @@ __global__ __launch_bounds__(WAVE) void attention_merge_kernel(const float* __re
         const int d = lane + i * WAVE;
         if (d < HD) out[(size_t)blockIdx.x * HD + d] = f32_to_bf16(o[i] / l);
     }
+}
+
+// slices read together by the merge: all of a step's where they are few, never more than fit in registers
+static void launch_merge(hipStream_t stream, const float* work, int n_slices, int n_seqs, int nh, const int* seq_start,
+                         int window, bf16_t* out) {
+    if (n_slices <= 4) attention_merge_kernel<4><<<n_seqs * nh, WAVE, 0, stream>>>(work, n_slices, nh, seq_start, window, out);
+    else if (n_slices <= 8) attention_merge_kernel<8><<<n_seqs * nh, WAVE, 0, stream>>>(work, n_slices, nh, seq_start, window, out);
+    else attention_merge_kernel<16><<<n_seqs * nh, WAVE, 0, stream>>>(work, n_slices, nh, seq_start, window, out);
 }
 
 static int launch_attention_decode(hipStream_t stream, const void* q, const void* k_cache, const void* v_cache,
@@ -318,7 +336,7 @@ static int launch_attention_decode(hipStream_t stream, const void* q, const void
                                                       window, n_slices, work, (bf16_t*)out);
     PALM_LAUNCHED();
     if (n_slices > 1) {
-        attention_merge_kernel<<<n_seqs * nh, WAVE, 0, stream>>>(work, n_slices, nh, seq_start, window, (bf16_t*)out);
+        launch_merge(stream, work, n_slices, n_seqs, nh, seq_start, window, (bf16_t*)out);
         PALM_LAUNCHED();
     }
     return 0;
@@ -666,7 +684,7 @@ PALM_API int palm_attention_decode_fused(hipStream_t stream, const void* qkv, in
 #undef PALM_FUSED
     PALM_LAUNCHED();
     if (n_slices > 1) {
-        attention_merge_kernel<<<n_seqs * nh, WAVE, 0, stream>>>(work, n_slices, nh, seq_start, window, (bf16_t*)out);
+        launch_merge(stream, work, n_slices, n_seqs, nh, seq_start, window, (bf16_t*)out);
         PALM_LAUNCHED();
     }
     return 0;
