@@ -103,12 +103,15 @@ def plain_attention(h, w, nh, nkv, hd, eps, theta, window, qk_norm, position):
 
 
 @pytest.mark.parametrize("dtype", [F32, BF16])
-@pytest.mark.parametrize("kw", [dict(), dict(window=40), dict(qk_norm=False), dict(position=False), dict(qk_norm=False, position=False)])
+@pytest.mark.parametrize("kw", [dict(), dict(window=40), dict(qk_norm=False), dict(position=False), dict(qk_norm=False, position=False),
+                                dict(hd=64), dict(hd=64, window=40), dict(hd=64, qk_norm=False), dict(hd=64, position=False),
+                                dict(hd=128, nkv=1, window=3)])
 def test_attention_part_in_pieces_against_whole_sequences(dtype, kw):
-    """Plain attention without rotation or norm is one of the cases; each switch is a parameter of the part."""
+    """Plain attention without rotation or norm is one of the cases; each switch is a parameter of the part.  With
+    heads of 64 or 128 the single-token steps in bfloat16 take the kernel that starts from the projection's rows."""
     from palm_infra_amd.cache import ModelCache
     from palm_infra_amd.parts import cache_needs, make_context
-    H, nh, nkv, hd, eps, theta = 72, 6, 3, 48, 1e-5, 10000.0
+    H, nh, nkv, hd, eps, theta = 72, 6, kw.get("nkv", 3), kw.get("hd", 48), 1e-5, 10000.0
     window, qk_norm, position = kw.get("window"), kw.get("qk_norm", True), kw.get("position", True)
     T = Tensors()
     spec, w = attention_spec(T, H, nh, nkv, hd, eps, theta, window, qk_norm, position)
@@ -116,11 +119,13 @@ def test_attention_part_in_pieces_against_whole_sequences(dtype, kw):
     needs = cache_needs(spec)
     assert needs[0].num_kv_heads == nkv and needs[0].head_dim == hd and needs[0].window == window
     cache = ModelCache([needs], [None], 64 * 8, None, 4096, dtype, DEV)
-    seqs = [rand(150, H, seed=11), rand(70, H, seed=12)]
+    seqs = [rand(157, H, seed=11), rand(77, H, seed=12)]
     slots = [cache.open(), cache.open()]
     outs = [[], []]
     done = [0, 0]
-    for pieces in ([100, 64], [1, 0], [49, 6]):            # a prompt each, one token for the first only, the rest
+    # a prompt each, one token for the first only, a further piece, then both token by token (the second sequence's
+    # first single token opens a page)
+    for pieces in ([100, 64], [1, 0], [49, 0]) + ([1, 1],) * 7 + ([0, 6],):
         live = [b for b in range(2) if pieces[b] > 0]
         growth = [(slots[b], pieces[b]) for b in live]
         cache.reserve(growth)
