@@ -276,3 +276,22 @@ PALM_API int palm_swiglu(hipStream_t stream, const void* gate_up, int dtype, voi
     PALM_LAUNCHED();
     return 0;
 }
+
+// y[r, c] += bias[c]: a projection's bias, added to the product in 32-bit and rounded once more to y's type.  The
+// matrix-core kernels have no bias term in their epilogues (Qwen3's projections have none, models/qwen3.py:290-349);
+// a part whose projection has one pays this pass.
+template <typename T>
+__global__ void add_bias_kernel(T* __restrict__ y, const float* __restrict__ bias, size_t total, int cols) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x)
+        y[i] = from_float<T>(to_float(y[i]) + bias[i % cols]);
+}
+
+PALM_API int palm_add_bias(hipStream_t stream, void* y, int dtype, const float* bias, int n_rows, int cols) {
+    PALM_CHECK(n_rows >= 0 && cols > 0 && bias, "add_bias: rows=%d cols=%d", n_rows, cols);
+    if (n_rows == 0) return 0;
+    const size_t total = (size_t)n_rows * cols;
+    const int blocks = (int)((total + 255) / 256 < 65536 ? (total + 255) / 256 : 65536);
+    PALM_DTYPE_SWITCH(dtype, T, add_bias_kernel<T><<<blocks, 256, 0, stream>>>((T*)y, bias, total, cols));
+    PALM_LAUNCHED();
+    return 0;
+}

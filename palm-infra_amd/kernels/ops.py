@@ -23,6 +23,7 @@ _SIGNATURES = {
     "palm_rmsnorm": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p, c_float, c_void_p, c_int, c_int,
                      c_void_p, c_int, c_int, c_longlong],
     "palm_swiglu": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int],
+    "palm_add_bias": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int],
     "palm_convert": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_longlong],
     "palm_random_fill": [c_void_p, c_void_p, c_int, c_longlong, c_ulonglong, c_float, c_float],
     "palm_linear": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int],
@@ -158,6 +159,15 @@ def swiglu(gate_up: torch.Tensor) -> torch.Tensor:
     out = torch.empty((n, two_i // 2), dtype=gate_up.dtype, device=gate_up.device)
     library.call(core(), "palm_swiglu", _stream(), _p(gate_up), _code(gate_up, "swiglu"), _p(out), n, two_i // 2)
     return out
+
+
+def add_bias(y: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
+    """y[r, :] += bias, in place; y [n, out] float32 or bfloat16, bias [out] float32.  Returns y."""
+    _dev("add_bias", y, bias)
+    _need(y.dim() == 2 and y.is_contiguous() and bias.shape == (y.shape[1],) and bias.dtype == F32 and bias.is_contiguous(),
+          f"add_bias: y {tuple(y.shape)}, bias {tuple(bias.shape)} {bias.dtype} is not float32 [{y.shape[-1]}]")
+    library.call(core(), "palm_add_bias", _stream(), _p(y), _code(y, "add_bias"), _p(bias), y.shape[0], y.shape[1])
+    return y
 
 
 _STORED_CODES = {F32: 0, BF16: 1, torch.float16: 2, torch.float64: 3}

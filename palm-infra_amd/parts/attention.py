@@ -5,7 +5,8 @@ Order of operations as the reference builds it (models/qwen3.py:290-349): one jo
 per-head norm of q and k over head_dim with one weight vector for all heads; rotation of q and k; the
 step's k and v are appended to the cache; every query attends the cached keys of its own sequence up
 to its own position with scale ``scale`` (head_dim^-0.5 for Qwen3); head h reads kv head
-h // (heads / kv_heads) (kernels/attention.cpp:1161); output projection.  No bias anywhere.
+h // (heads / kv_heads) (kernels/attention.cpp:1161); output projection.  The reference's projections have no
+bias; a specification that names tensors ``qkv_bias`` / ``out_bias`` (float32 vectors) gets them added.
 """
 from __future__ import annotations
 
@@ -28,8 +29,9 @@ class Attention:
         self.window = int(p["window"]) if p.get("window") else None
         if self.nh % self.nkv:
             raise ValueError(f"{self.nh} heads are not a multiple of {self.nkv} kv heads")
-        self.qkv = Linear(builder.tensor(spec, "qkv"))
-        self.out = Linear(builder.tensor(spec, "out"))
+        bias = lambda name: builder.tensor(spec, name) if name in spec.tensors else None
+        self.qkv = Linear(builder.tensor(spec, "qkv"), bias("qkv_bias"))
+        self.out = Linear(builder.tensor(spec, "out"), bias("out_bias"))
         if self.qkv.weight.shape != ((self.nh + 2 * self.nkv) * self.hd, self.hidden):
             raise ValueError(f"attention: joined q/k/v weight {tuple(self.qkv.weight.shape)} does not fit "
                              f"{self.nh}+2*{self.nkv} heads of {self.hd} over hidden {self.hidden}")

@@ -13,8 +13,9 @@ class GatedSiluFeedForward:
     def __init__(self, spec, builder):
         self.hidden = int(spec.params["hidden_size"])
         self.inter = int(spec.params["intermediate_size"])
-        self.gate_up = Linear(builder.tensor(spec, "gate_up"))
-        self.down = Linear(builder.tensor(spec, "down"))
+        bias = lambda name: builder.tensor(spec, name) if name in spec.tensors else None
+        self.gate_up = Linear(builder.tensor(spec, "gate_up"), bias("gate_up_bias"))
+        self.down = Linear(builder.tensor(spec, "down"), bias("down_bias"))
         if self.gate_up.weight.shape != (2 * self.inter, self.hidden) or self.down.weight.shape != (self.hidden, self.inter):
             raise ValueError(f"feed-forward: weights {tuple(self.gate_up.weight.shape)}, {tuple(self.down.weight.shape)} "
                              f"do not fit hidden {self.hidden}, intermediate {self.inter}")

@@ -5,6 +5,9 @@
   bfloat16 x bfloat16, 17 to 64 rows (large decode batches)     the matrix-core kernel that shares the rows through LDS
   bfloat16 x bfloat16, many rows (prompts)                      the BLAS library, as the reference's GPU path
                                                                 does for its products (engine/cuda_matmul.cu:245-260)
+
+A bias (none of Qwen3's projections has one) is added by a pass of its own after the product, which then comes
+whole (no planes, no norm folded in): correct for any part that needs it, at the price of a launch.
 """
 from __future__ import annotations
 
@@ -20,11 +23,14 @@ THIN_ROWS = 16
 
 
 class Linear:
-    def __init__(self, weight: torch.Tensor):
+    def __init__(self, weight: torch.Tensor, bias: torch.Tensor | None = None):
         if weight.dim() != 2:
             raise ValueError(f"a linear weight must be [out, in], got {tuple(weight.shape)}")
         self.weight = weight
         self.out_features, self.in_features = weight.shape
+        if bias is not None and (bias.shape != (self.out_features,) or bias.dtype != torch.float32):
+            raise ValueError(f"a linear bias must be float32 [{self.out_features}], got {bias.dtype} {tuple(bias.shape)}")
+        self.bias = bias
 
     def __call__(self, x, out_dtype: torch.dtype | None = None, planes_ok: bool = False, sink=None):
         """x: rows [n, in], or ``Prenormed`` rows (their row factor is applied to the result).
@@ -37,6 +43,11 @@ class Linear:
         norm makes of the residual stream after the add, as a tensor or as ``Prenormed`` rows."""
         if sink is not None:
             return self._into(x, sink)
+        if self.bias is not None:
+            return ops.add_bias(self._product(x, out_dtype, False), self.bias)
+        return self._product(x, out_dtype, planes_ok)
+
+    def _product(self, x, out_dtype, planes_ok):
         w = self.weight
         if isinstance(x, Prenormed):
             if self._folds(x.values):
@@ -56,7 +67,7 @@ class Linear:
 
     def _into(self, x, sink):
         rows = x.values if isinstance(x, Prenormed) else x
-        if (sink.foldable and self._folds(rows) and sink.x.shape == (rows.shape[0], self.out_features)
+        if (self.bias is None and sink.foldable and self._folds(rows) and sink.x.shape == (rows.shape[0], self.out_features)
                 and rows.dtype == torch.bfloat16 and ops.fold_pays(rows.shape[0], self.out_features, self.in_features)):
             ss_in, eps_in = (x.ss, x.eps) if isinstance(x, Prenormed) else (None, 0.0)
             values, ss = ops.linear_thin_into_residual(rows, self.weight, sink.x, sink.norm.weight, row_ss=ss_in, row_eps=eps_in)
@@ -66,6 +77,8 @@ class Linear:
     def gated(self, x) -> torch.Tensor:
         """silu(x G^T) * (x U^T) for a weight that is [G rows | U rows]: in one kernel when the product is thin,
         else the product and then the activation."""
+        if self.bias is not None:
+            return ops.swiglu(self(x))
         if isinstance(x, Prenormed):
             if self._folds(x.values):
                 return ops.linear_thin(x.values, self.weight, x.dtype, gated=True, row_ss=x.ss, row_eps=x.eps)

@@ -69,7 +69,7 @@ def test_position_part_makes_its_tables_once_per_step():
         build(PartSpec("position", "rotary", {"rotary_dim": 8, "theta": 1.0, "pairing": "spiral"}), Tensors(), F32)
 
 
-def attention_spec(T, H, nh, nkv, hd, eps, theta, window=None, qk_norm=True, position=True, seed=0):
+def attention_spec(T, H, nh, nkv, hd, eps, theta, window=None, qk_norm=True, position=True, seed=0, bias=False):
     from palm_infra_amd.config import PartSpec, joined, tensor
     # without a q/k norm the scores' spread is set by these scales: kept near one so that bfloat16 rounding
     # cannot flip which key leads
@@ -82,30 +82,36 @@ def attention_spec(T, H, nh, nkv, hd, eps, theta, window=None, qk_norm=True, pos
         parts["k_norm"] = PartSpec("norm", "rms", {"width": hd, "eps": eps}, {"weight": T.add(tensor("kn", (hd,), "vector"), w["kn"])})
     if position:
         parts["position"] = PartSpec("position", "rotary", {"rotary_dim": hd, "theta": theta, "pairing": "half_split"})
+    tensors = {"qkv": T.add(joined(("q", "k", "v"), ((nh * hd, H), (nkv * hd, H), (nkv * hd, H))), torch.cat([w["q"], w["k"], w["v"]])),
+               "out": T.add(tensor("o", (H, nh * hd)), w["o"])}
+    if bias:           # a projection with a bias is no part of Qwen3; the part takes one if its specification names it
+        w.update(qb=rand(nh * hd, seed=seed + 7, scale=0.5), kb=rand(nkv * hd, seed=seed + 8, scale=0.5),
+                 vb=rand(nkv * hd, seed=seed + 9, scale=0.5), ob=rand(H, seed=seed + 10, scale=0.5))
+        tensors["qkv_bias"] = T.add(tensor("qkvb", ((nh + 2 * nkv) * hd,), "vector"), torch.cat([w["qb"], w["kb"], w["vb"]]))
+        tensors["out_bias"] = T.add(tensor("ob", (H,), "vector"), w["ob"])
     spec = PartSpec("mixer", "attention", {"hidden_size": H, "num_heads": nh, "num_kv_heads": nkv, "head_dim": hd,
-                                           "scale": hd ** -0.5, "window": window},
-                    {"qkv": T.add(joined(("q", "k", "v"), ((nh * hd, H), (nkv * hd, H), (nkv * hd, H))), torch.cat([w["q"], w["k"], w["v"]])),
-                     "out": T.add(tensor("o", (H, nh * hd)), w["o"])}, parts)
+                                           "scale": hd ** -0.5, "window": window}, tensors, parts)
     return spec, w
 
 
 def plain_attention(h, w, nh, nkv, hd, eps, theta, window, qk_norm, position):
     n = h.shape[0]
-    q = P.linear(h, w["q"]).reshape(n, nh, hd)
-    k = P.linear(h, w["k"]).reshape(n, nkv, hd)
-    v = P.linear(h, w["v"]).reshape(n, nkv, hd)
+    zero = torch.zeros(1, dtype=torch.float64)
+    q = (P.linear(h, w["q"]) + w.get("qb", zero).double()).reshape(n, nh, hd)
+    k = (P.linear(h, w["k"]) + w.get("kb", zero).double()).reshape(n, nkv, hd)
+    v = (P.linear(h, w["v"]) + w.get("vb", zero).double()).reshape(n, nkv, hd)
     if qk_norm:
         q, k = P.rms_norm(q, w["qn"], eps), P.rms_norm(k, w["kn"], eps)
     if position:
         cos, sin = P.rope_table(list(range(n)), hd, theta)
         q, k = P.rope_half_split(q, cos, sin), P.rope_half_split(k, cos, sin)
-    return P.linear(P.causal_attention(q, k, v, hd ** -0.5, window).reshape(n, nh * hd), w["o"])
+    return P.linear(P.causal_attention(q, k, v, hd ** -0.5, window).reshape(n, nh * hd), w["o"]) + w.get("ob", zero).double()
 
 
 @pytest.mark.parametrize("dtype", [F32, BF16])
 @pytest.mark.parametrize("kw", [dict(), dict(window=40), dict(qk_norm=False), dict(position=False), dict(qk_norm=False, position=False),
                                 dict(hd=64), dict(hd=64, window=40), dict(hd=64, qk_norm=False), dict(hd=64, position=False),
-                                dict(hd=128, nkv=1, window=3)])
+                                dict(hd=128, nkv=1, window=3), dict(bias=True), dict(hd=64, bias=True)])
 def test_attention_part_in_pieces_against_whole_sequences(dtype, kw):
     """Plain attention without rotation or norm is one of the cases; each switch is a parameter of the part.  With
     heads of 64 or 128 the single-token steps in bfloat16 take the kernel that starts from the projection's rows."""
@@ -114,7 +120,7 @@ def test_attention_part_in_pieces_against_whole_sequences(dtype, kw):
     H, nh, nkv, hd, eps, theta = 72, 6, kw.get("nkv", 3), kw.get("hd", 48), 1e-5, 10000.0
     window, qk_norm, position = kw.get("window"), kw.get("qk_norm", True), kw.get("position", True)
     T = Tensors()
-    spec, w = attention_spec(T, H, nh, nkv, hd, eps, theta, window, qk_norm, position)
+    spec, w = attention_spec(T, H, nh, nkv, hd, eps, theta, window, qk_norm, position, bias=kw.get("bias", False))
     att = build(spec, T, dtype)
     needs = cache_needs(spec)
     assert needs[0].num_kv_heads == nkv and needs[0].head_dim == hd and needs[0].window == window
@@ -148,7 +154,7 @@ def test_attention_part_in_pieces_against_whole_sequences(dtype, kw):
 
 def w_as(w, dtype):
     """The weights as the part holds them: matrices in the run's precision, norm vectors in float32."""
-    return {k: (v if k in ("qn", "kn") else v.to(dtype)) for k, v in w.items()}
+    return {k: (v if k in ("qn", "kn", "qb", "kb", "vb", "ob") else v.to(dtype)) for k, v in w.items()}
 
 
 @pytest.mark.parametrize("dtype", [F32, BF16])
@@ -165,6 +171,16 @@ def test_feed_forward_part(dtype):
     got = ff.forward(h.to(DEV), None).cpu().double()
     ref = P.swiglu_mlp(h, wg.to(dtype), wu.to(dtype), wd.to(dtype))
     assert torch.allclose(got, ref, atol=tol(dtype) * float(ref.abs().max()))
+    # with biases (no part of Qwen3; the part takes them if its specification names them)
+    bg, bd = rand(2 * I, seed=5, scale=0.5), rand(H, seed=6, scale=0.5)
+    biased = PartSpec("feed_forward", "gated_silu", {"hidden_size": H, "intermediate_size": I},
+                      dict(spec.tensors, gate_up_bias=T.add(tensor("gub", (2 * I,), "vector"), bg), down_bias=T.add(tensor("db", (H,), "vector"), bd)))
+    for rows in (9, 70):
+        h2 = rand(rows, H, seed=7).to(dtype)
+        g, u = P.linear(h2, wg.to(dtype)) + bg[:I].double(), P.linear(h2, wu.to(dtype)) + bg[I:].double()
+        ref2 = (g / (1 + torch.exp(-g)) * u) @ wd.to(dtype).double().T + bd.double()
+        got2 = build(biased, T, dtype).forward(h2.to(DEV), None).cpu().double()
+        assert torch.allclose(got2, ref2, atol=tol(dtype) * float(ref2.abs().max())), float((got2 - ref2).abs().max())
     # one expert of a routed feed-forward is this feed-forward: nothing else to reduce to here
     with pytest.raises(ValueError, match="do not fit"):
         build(PartSpec("feed_forward", "gated_silu", {"hidden_size": H, "intermediate_size": I + 1}, spec.tensors), T, dtype)
