@@ -5,6 +5,7 @@
 #include "common.h"
 
 PALM_API int palm_attention_head_dim();
+PALM_API int palm_attention_page_tokens();     // the cache's page size the library was built for
 
 // One query a sequence over the paged cache.  With more than one slice of the key range the partial results
 // (maximum, sum, unnormalised output of every slice) cross from the first kernel to the merging one through

@@ -43,6 +43,7 @@ __device__ inline float exp2_weight(float x) { return __builtin_amdgcn_exp2f(x);
 
 PALM_DEFINE_LAST_ERROR()
 PALM_API int palm_attention_head_dim() { return HD; }
+PALM_API int palm_attention_page_tokens() { return PAGE_TOKENS; }
 
 struct Columns {          // softmax state of this lane's query column, and its share of the output
     float m, l;

@@ -567,6 +567,9 @@ def attention_lib(hd: int):
             fn.argtypes, fn.restype = argtypes, c_int
         if lib.palm_attention_head_dim() != hd:
             raise KernelError(f"library attention_hd{hd} was built for head size {lib.palm_attention_head_dim()}")
+        if lib.palm_attention_page_tokens() != PAGE_TOKENS:
+            raise KernelError(f"library attention_hd{hd} was built for pages of {lib.palm_attention_page_tokens()} tokens, "
+                              f"the cache has pages of {PAGE_TOKENS}")
         _attention_libs[hd] = lib
     return _attention_libs[hd]
 

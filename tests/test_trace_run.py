@@ -89,11 +89,11 @@ def schedule_steps(reqs):
 # the last three: a folder stored in one precision and run in the other (a tensor stored in 32-bit stays so in
 # the bfloat16 mode; bfloat16 and float16 widen exactly for the float32 mode; float16 is re-rounded for bfloat16)
 @pytest.mark.parametrize("name,dtype,store", [("A", "float32", None), ("A", "bfloat16", None), ("B", "float32", None),
-                                              ("B", "bfloat16", None), ("B", "bfloat16", "float32"),
+                                              ("B", "bfloat16", None), ("D", "bfloat16", None), ("B", "bfloat16", "float32"),
                                               ("A", "float32", "bfloat16"), ("B", "float32", "float16"),
                                               ("A", "bfloat16", "float16")])
 def test_replay_schedules(model_dirs, tmp_path, name, dtype, store):
-    lengths = {"A": [5, 17, 9, 70, 40, 33], "B": [1, 31, 12, 64, 100, 45]}[name]
+    lengths = {"A": [5, 17, 9, 70, 40, 33], "B": [1, 31, 12, 64, 100, 45], "D": [64, 3, 97, 65, 128, 33]}[name]
     reqs = tiny.prompts(name, lengths, seed=8)
     steps, checks = schedule_steps(reqs)
     # the most that is live at once: the second batch, each request rounded up to 64
