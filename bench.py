@@ -137,14 +137,23 @@ def kernel_table(engine, cfg, slots, batch: int, context: int) -> dict:
     seq_slot = torch.tensor(slots, dtype=torch.int32, device=dev)
     seq_start = torch.tensor([cache.lengths[s] - 1 for s in slots], dtype=torch.int32, device=dev)
     n_slices = ops.decode_slices(batch, nh, nkv, engine._length_bucket(context + 1))
+    # what the attention part runs after its q/k/v projection in a decode step: the projection's planes of partial
+    # sums in, per-head norms, rotation, the new key and value into the cache, attention, the merge of the slices
+    mixer0 = layers[0].mixer
+    qkv = mixer0.qkv(h, planes_ok=True).clone()
+    cos, sin = ops.rope_table(seq_start, mixer0.position.inv_freq)
+
+    def attention_of(i):
+        m = layers[i].mixer
+        return ops.attention_decode_fused(qkv, kv.k[i], kv.v[i], kv.table_dev, seq_slot, seq_start, nh, nkv, hd, m.scale, None,
+                                          n_slices, q_norm_w=m.q_norm.weight, k_norm_w=m.k_norm.weight, eps=m.q_norm.eps,
+                                          cos=cos, sin=sin, rotary_dim=hd, pairing=0)
 
     def each_layer(fn):
         return lambda: [fn(i) for i in range(L)]
     work = {
         "qkv_proj": (each_layer(lambda i: layers[i].mixer.qkv(h, planes_ok=True)), (nh + 2 * nkv) * hd * H * 2, L),
-        "attention": (each_layer(lambda i: ops.attention_decode(attn, kv.k[i], kv.v[i], kv.table_dev, seq_slot, seq_start, nh, nkv, hd,
-                                                                hd ** -0.5, None, n_slices)),
-                      2 * nkv * hd * 2 * context * batch, L),
+        "attention": (each_layer(attention_of), 2 * nkv * hd * 2 * context * batch, L),
         "o_proj": (each_layer(lambda i: layers[i].mixer.out(attn, sink=ResidualSink(resid, layers[i].feed_forward_norm))),
                    nh * hd * H * 2, L),
         "gate_up_proj": (each_layer(lambda i: layers[i].feed_forward.gate_up.gated(h)), 2 * I * H * 2, L),
