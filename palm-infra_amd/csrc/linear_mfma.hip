@@ -161,8 +161,12 @@ struct RowNorm {
     float* ss_out;           // [M, strips]
 };
 
-constexpr int STREAM_WAVE_SLOTS = 4096;     // waves that run at once in the usual launch: 16 on each of 256 compute units
-constexpr int STREAM_WAVE_SLOTS_CUT = 6144; // with K cut into ranges a block's work is short: 24
+// Waves that run at once in the usual launch: 8 on each of 256 compute units, one block of eight waves each.  Two
+// blocks a unit (4096) were the rule once: measured at 8 rows, the gated product of 24576 x 4096 38.2 us against 36.6
+// and the head of 151936 rows 216 against 214 (a decode step of 36 layers 4.04 against 3.99 ms); anything between
+// (2560, 3072) leaves some units with twice the work of others and is much slower (4.58 ms).
+constexpr int STREAM_WAVE_SLOTS = 2048;
+constexpr int STREAM_WAVE_SLOTS_CUT = 6144; // with K cut into ranges a block's work is short: 24 waves a unit
 
 template <int NW, int U, int TREG, bool EXACT, typename TC, int EPI>
 __global__ __launch_bounds__(NW * WAVE) void linear_stream_kernel(const bf16_t* __restrict__ A,
@@ -376,8 +380,8 @@ static void launch_stream(hipStream_t stream, const void* a, const void* w, void
     T = (T + U - 1) / U * U;
     if (TREG > 0) T = TREG;
     // every block the same number of strips, as far as that goes
-    // (with six or eight steps of activations in registers half as many waves fit a compute unit)
-    const int wave_slots = TREG > 4 ? STREAM_WAVE_SLOTS / 2 : (parts > 1 ? STREAM_WAVE_SLOTS_CUT : STREAM_WAVE_SLOTS);
+    // (with six or eight steps of activations in registers more waves than the usual do not fit a compute unit)
+    const int wave_slots = parts > 1 && TREG <= 4 ? STREAM_WAVE_SLOTS_CUT : STREAM_WAVE_SLOTS;
     const int slots = max(1, wave_slots / NW / parts);
     const int rounds = (strips + slots - 1) / slots;
     const dim3 grid((strips + rounds - 1) / rounds, parts);
