@@ -37,6 +37,14 @@ class StepEntry:
     want: list = field(default_factory=list)
 
 
+@dataclass
+class FedTokens:
+    """Tokens that an earlier step's sampling left on the device, for a step of single tokens that is launched
+    before the host has seen them: the step's k-th sequence takes ``ids[rows[k]]``."""
+    ids: torch.Tensor            # int32 [m] on the engine's device
+    rows: list
+
+
 def resolve_dtype(dtype) -> torch.dtype:
     if isinstance(dtype, torch.dtype):
         if dtype not in (torch.bfloat16, torch.float32):
@@ -48,6 +56,8 @@ def resolve_dtype(dtype) -> torch.dtype:
 
 
 class Engine:
+    takes_fed = True             # step(entries, fed=..) takes tokens that are still on the device
+
     def __init__(self, config, spec, weights, dtype: torch.dtype, max_tokens: int, max_seqs: int | None = None,
                  device="cuda:0", graphs: bool = True, max_step_tokens: int = 32768):
         self.device = torch.device(device)
@@ -128,11 +138,17 @@ class Engine:
                 if not 0 <= int(w) < len(e.tokens):
                     raise StepError(f"slot {e.slot}: logits wanted at place {w} of {len(e.tokens)} tokens")
 
-    def step(self, entries) -> torch.Tensor:
+    def step(self, entries, fed: FedTokens | None = None) -> torch.Tensor:
         """Run the entries' tokens as one batch from the cache; float32 logits [wanted, vocab] in the
-        order of the entries and of each entry's ``want``.  Nothing changes if the step is refused."""
+        order of the entries and of each entry's ``want``.  Nothing changes if the step is refused.
+
+        ``fed``: every entry brings one token, and which one is not known on the host yet: entry k's is
+        ``fed.ids[fed.rows[k]]`` on the device (what its ``tokens`` holds is a stand-in).  The step is then launched
+        without waiting for the device, so that a caller can look at one step's tokens while the next one runs."""
         entries = [e if isinstance(e, StepEntry) else StepEntry(*e) for e in entries]
         self._validate(entries)
+        if fed is not None:
+            return self._run_fed(entries, fed)
         per_seq, per_step = self.step_tokens_per_seq, self.max_step_tokens
         total = sum(len(e.tokens) for e in entries)
         if (per_seq is None or all(len(e.tokens) <= per_seq for e in entries)) and total <= per_step:
@@ -196,7 +212,10 @@ class Engine:
         if state is None:
             while len(self._decode_graphs) >= self.GRAPH_LIMIT:          # a graph holds its activations and logits: bound them
                 self._decode_graphs.pop(next(iter(self._decode_graphs)))
-            state = {"buf": torch.zeros((context_ints(n_tokens, n_seqs),), dtype=torch.int32, device=self.device),
+            size = context_ints(n_tokens, n_seqs)
+            state = {"buf": torch.zeros((size,), dtype=torch.int32, device=self.device),
+                     "staging": [torch.zeros((size,), dtype=torch.int32, pin_memory=True) for _ in range(2)],
+                     "staged": [None, None], "turn": 0,
                      "rows": None if n_rows is None else torch.zeros((n_rows,), dtype=torch.int32, device=self.device),
                      "graph": None, "logits": None, "calls": 0}
         self._decode_graphs[key] = state
@@ -219,7 +238,20 @@ class Engine:
         state["calls"] += 1
         return logits
 
-    def _run_decode_graph(self, entries) -> torch.Tensor:
+    def _run_fed(self, entries, fed: FedTokens) -> torch.Tensor:
+        if any(len(e.tokens) != 1 for e in entries) or len(fed.rows) != len(entries):
+            raise StepError("a step fed from the device brings one token for each sequence and one row for each token")
+        if fed.ids.dtype != torch.int32 or fed.ids.device != self.device or fed.ids.dim() != 1:
+            raise StepError(f"fed tokens are int32 [m] on {self.device}, not {fed.ids.dtype} {tuple(fed.ids.shape)} on {fed.ids.device}")
+        if any(not 0 <= int(r) < fed.ids.shape[0] for r in fed.rows):
+            raise StepError(f"a fed row lies outside the {fed.ids.shape[0]} tokens given")
+        if self._graph_serves(entries):
+            return self._run_decode_graph(entries, fed)
+        # no recorded step serves these entries: the tokens come to the host first (which waits for them)
+        ids = fed.ids.tolist()
+        return self._run([StepEntry(e.slot, [ids[int(r)]], e.want) for e, r in zip(entries, fed.rows)])
+
+    def _run_decode_graph(self, entries, fed: FedTokens | None = None) -> torch.Tensor:
         cache = self.cache
         growth = [(e.slot, 1) for e in entries]
         cache.reserve(growth)
@@ -231,9 +263,23 @@ class Engine:
         state = self._recorded(key, Bb, Bb, None)
         # the step's arrays, laid out as for any step, at the addresses the recording reads; rows that pad the batch
         # belong to a slot of their own whose page is never read
+        # through pinned memory, so that the host need not wait for the device: two buffers in turn, each written
+        # again only after the copy that last read it has run
+        turn = state["turn"] = state["turn"] ^ 1
+        if state["staged"][turn] is not None:
+            state["staged"][turn].synchronize()
         ctx = make_context([e.slot for e in entries] + [cache.pad_slot] * pad, starts + [0] * pad,
                            [[int(e.tokens[0])] for e in entries] + [[0]] * pad, self.dtype, self.device,
-                           max_total=key[1], into=state["buf"])
+                           max_total=key[1], into=state["buf"], staging=state["staging"][turn])
+        state["staged"][turn] = torch.cuda.Event()
+        state["staged"][turn].record()
+        if fed is not None:
+            rows = [int(r) for r in fed.rows]
+            if rows == list(range(B)):
+                ctx.token_ids[:B].copy_(fed.ids[:B])
+            else:
+                index = torch.tensor(rows, dtype=torch.int64).pin_memory().to(self.device, non_blocking=True)
+                torch.index_select(fed.ids, 0, index, out=ctx.token_ids[:B])
         logits = self._replay(state, ctx)
         cache.commit(growth)
         wanted = [b for b, e in enumerate(entries) if e.want]

@@ -9,6 +9,13 @@ batches of requests with unequal prompts: all prompts of a batch in one step, th
 sequence that is still running; a sequence that ends leaves the batch at once and its slot goes back;
 batches follow one another until every request is served.
 
+Where the engine takes tokens that are still on the device (``takes_fed``) and the sampler's draw does not depend
+on earlier draws (no penalties), the loop runs one step ahead of itself: it launches step t+1 with the tokens
+that step t's sampling left on the device, and only then looks at step t's tokens, while the device is busy.  What
+can end a sequence without knowing its newest token (the lengths) is decided before the launch; a stop token shows
+one step late, and the one draw made for that sequence meanwhile is dropped.  The results are the same as
+without; the host's work between two steps no longer leaves the device idle.
+
 The loop only decides; the engine steps and the sampler chooses.  Both are handed in, so the decisions
 can be tested with stand-ins.
 """
@@ -19,7 +26,27 @@ from dataclasses import dataclass, field
 
 from ..cache.pool import PAGE_TOKENS, pages_for
 from ..sampling import SequenceSampling
-from .engine import StepEntry
+from .engine import FedTokens, StepEntry
+
+
+class TokenFetch:
+    """A step's drawn tokens on their way to the host: asked for at once (so that the copy stands before the next
+    step in the device's queue), looked at later."""
+
+    def __init__(self, ids):
+        self.ids, self.host, self.event = ids, None, None
+        if getattr(ids, "is_cuda", False):
+            import torch
+            self.host = torch.empty(ids.shape, dtype=ids.dtype, pin_memory=True)
+            self.host.copy_(ids, non_blocking=True)
+            self.event = torch.cuda.Event()
+            self.event.record()
+
+    def tokens(self) -> list:
+        if self.event is None:
+            return self.ids.tolist()
+        self.event.synchronize()
+        return self.host.tolist()
 
 
 @dataclass
@@ -159,6 +186,33 @@ def generate(engine, sampler, prompts, max_new_tokens: int = 2048, stop_token_id
 
             # ---- one token for each sequence that still runs ----
             t1 = timer()
+            if live and getattr(engine, "takes_fed", False) and not getattr(sampler, "needs_history", True):
+                def goes_on(i, n):
+                    """Whether request i runs on after its n-th token if that is no stop token (as take decides)."""
+                    return n < max_new_tokens and len(prompts[i]) + n <= max_seq
+
+                logits = engine.step([StepEntry(slots[i], [results[i].token_ids[-1]], [0]) for i in live])
+                for i in live:
+                    states[i].accept([results[i].token_ids[-1]])
+                pending = TokenFetch(sampler.sample(logits, [states[i] for i in live]))
+                order = [(i, row) for row, i in enumerate(live)]        # whose newest token is which row of `pending`
+                while order:
+                    ahead = [(i, row) for i, row in order if goes_on(i, len(results[i].token_ids) + 1)]
+                    following = None
+                    if ahead:
+                        logits = engine.step([StepEntry(slots[i], [0], [0]) for i, _ in ahead],
+                                             fed=FedTokens(pending.ids, [row for _, row in ahead]))
+                        following = TokenFetch(sampler.sample(logits, [states[i] for i, _ in ahead]))
+                    toks = pending.tokens()                              # the device runs the next step meanwhile
+                    alive = set()
+                    for i, row in order:
+                        states[i].accept([int(toks[row])])
+                        if take(i, int(toks[row])):
+                            alive.add(i)
+                    # a sequence that ended on a stop token was stepped once more: its draw is dropped with it
+                    order = [(i, row) for row, (i, _) in enumerate(ahead) if i in alive]
+                    pending = following
+                live = []
             while live:
                 last = {i: results[i].token_ids[-1] for i in live}
                 logits = engine.step([StepEntry(slots[i], [last[i]], [0]) for i in live])

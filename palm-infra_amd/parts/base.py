@@ -105,14 +105,16 @@ def context_ints(n_tokens: int, n_seqs: int) -> int:
 
 
 def make_context(slots, starts, new_tokens, dtype, device, max_total=None, into: torch.Tensor | None = None,
-                 max_new: int | None = None) -> StepContext:
+                 max_new: int | None = None, staging: torch.Tensor | None = None) -> StepContext:
     """A context from host lists: ``new_tokens[b]`` is the list of token ids of sequence b.  This is the one place
     where a step's arrays are laid out: a part that needs one more of them finds it here.
 
     ``into``: an int32 device buffer of ``context_ints(n, B)`` elements to lay the arrays in instead of a new
     one: a recorded step keeps its arrays at fixed addresses and gets new contents before every replay.
     ``max_new``, ``max_total``: bounds to size launches by instead of the step's own longest run and sequence (a
-    recorded step is sized for the largest step it will be replayed for)."""
+    recorded step is sized for the largest step it will be replayed for).
+    ``staging`` (with ``into``): a pinned host buffer of the same size through which the arrays go to the device
+    without the host waiting for the device; the caller must not write it again before that copy has run."""
     counts = [len(t) for t in new_tokens]
     ids = [t for seq in new_tokens for t in seq]
     pos = [starts[b] + j for b in range(len(slots)) for j in range(counts[b])]
@@ -129,7 +131,11 @@ def make_context(slots, starts, new_tokens, dtype, device, max_total=None, into:
         if into.shape != host.shape or into.dtype != torch.int32:
             raise ValueError(f"a step of {n} tokens in {B} sequences needs {host.numel()} int32, the buffer has {tuple(into.shape)}")
         flat = into
-        flat.copy_(host)
+        if staging is None:
+            flat.copy_(host)
+        else:
+            staging.copy_(host)
+            flat.copy_(staging, non_blocking=True)
     o = 0
     parts = []
     for size in (n, n, n, B, B, B, B + 1):

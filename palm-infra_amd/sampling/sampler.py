@@ -68,6 +68,12 @@ class DeviceSampler:
         self.params = params or SamplingParams()
         self.params.validate()
 
+    @property
+    def needs_history(self) -> bool:
+        """Whether a draw depends on the tokens drawn before (the penalties do): a loop may then not ask for a
+        sequence's next draw before the host has seen its last one."""
+        return bool(self.params.penalties_enabled)
+
     def sample(self, logits: torch.Tensor, states) -> torch.Tensor:
         from ..kernels import ops
         p = self.params
@@ -86,7 +92,9 @@ class DeviceSampler:
                                     p.frequency_penalty)
         if p.greedy:
             return ops.argmax(logits)
-        u = torch.tensor([uniform(p.seed, st.stream, st.draws) for st in states], dtype=torch.float32).to(logits.device)
+        # through pinned memory: the host does not wait for the device here
+        u = torch.tensor([uniform(p.seed, st.stream, st.draws) for st in states], dtype=torch.float32).pin_memory().to(
+            logits.device, non_blocking=True)
         for st in states:
             st.draws += 1
         top_k = p.top_k if 0 < p.top_k < V else 0

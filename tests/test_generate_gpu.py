@@ -208,3 +208,73 @@ def test_a_conversation_continues_from_the_cache(model_dirs, engine_a):
     assert r.returncode == 0, r.stderr[-2000:]
     got = [[int(t) for t in line.split()] for line in r.stdout.strip().splitlines()]
     assert got == lines + [lines[0]]                            # after /reset the first turn gives its first answer again
+
+
+# ---- tokens fed from the device, and the loop that runs one step ahead ---------------------------------
+
+@pytest.mark.parametrize("name,dtype,graphs", [("A", "float32", True), ("D", "bfloat16", True), ("B", "bfloat16", False)])
+def test_a_step_fed_from_the_device_is_the_step_fed_from_the_host(model_dirs, name, dtype, graphs):
+    """The same single-token steps with the tokens as host integers and as rows of a device tensor (in order, and
+    picked out of a longer one): the same bits; without recorded steps the tokens come to the host first."""
+    from palm_infra_amd.engine import Engine, FedTokens, StepEntry, StepError
+    a = Engine.from_dir(model_dirs[name][dtype], dtype=dtype, max_tokens=64 * 12, graphs=graphs)
+    b = Engine.from_dir(model_dirs[name][dtype], dtype=dtype, max_tokens=64 * 12, graphs=graphs)
+    reqs = tiny.prompts(name, [9, 3, 30, 64], seed=40)
+    sa, sb = [a.open() for _ in reqs], [b.open() for _ in reqs]
+    for eng, slots in ((a, sa), (b, sb)):
+        eng.step([StepEntry(s, r, []) for s, r in zip(slots, reqs)])
+    V = tiny.CONFIGS[name]["vocab_size"]
+    g = torch.Generator().manual_seed(5)
+    for t in range(6):
+        toks = torch.randint(0, V, (len(reqs),), generator=g).tolist()
+        if t % 2 == 0:                                          # row k for entry k
+            ids, rows = torch.tensor(toks, dtype=torch.int32).to("cuda:0"), list(range(len(reqs)))
+        else:                                                   # picked out of a longer tensor, not in order
+            spread = [V - 1] * (2 * len(reqs) + 1)
+            rows = [2 * k + 1 for k in range(len(reqs))][::-1]
+            for k, r in enumerate(rows):
+                spread[r] = toks[k]
+            ids = torch.tensor(spread, dtype=torch.int32).to("cuda:0")
+        host = a.step([StepEntry(s, [tok], [0]) for s, tok in zip(sa, toks)])
+        fed = b.step([StepEntry(s, [0], [0]) for s in sb], fed=FedTokens(ids, rows))
+        assert torch.equal(host, fed), t
+    with pytest.raises(StepError, match="one token for each sequence"):
+        b.step([StepEntry(sb[0], [1, 2], [1])], fed=FedTokens(ids, [0]))
+    with pytest.raises(StepError, match="outside"):
+        b.step([StepEntry(sb[0], [0], [0])], fed=FedTokens(ids, [ids.shape[0]]))
+    for eng, slots in ((a, sa), (b, sb)):
+        for s in slots:
+            eng.close(s)
+        eng.cache.check()
+
+
+@pytest.mark.parametrize("name,dtype", [("A", "float32"), ("D", "bfloat16")])
+@pytest.mark.parametrize("temperature", [0.0, 0.9])
+def test_the_loop_that_runs_ahead_generates_what_the_plain_loop_does(model_dirs, name, dtype, temperature):
+    """The engine's generation (whose loop launches a step before it has seen the last one's tokens) against the
+    same loop made to wait for every step's tokens: the same tokens and endings, with stop tokens that end
+    sequences at different steps, in batches that follow one another."""
+    import palm_infra_amd
+    from palm_infra_amd.engine.generate import generate
+    from palm_infra_amd.sampling import DeviceSampler, SamplingParams
+
+    class Waiting(DeviceSampler):
+        needs_history = True
+
+    eng = palm_infra_amd.load(model_dirs[name][dtype], dtype=dtype, max_tokens=64 * 16)
+    params = SamplingParams(temperature=temperature, top_k=20, seed=4)
+    prompts = tiny.prompts(name, [6, 3, 11, 70, 8, 1, 40], seed=41)
+    free, _ = generate(eng, Waiting(params), prompts, max_new_tokens=24, stop_token_ids=(), max_batch=3)
+    # stop tokens that some requests emit early, some late, some never
+    stop = {free[0].token_ids[2], free[3].token_ids[10], free[5].token_ids[-1]}
+    want, _ = generate(eng, Waiting(params), prompts, max_new_tokens=24, stop_token_ids=stop, max_batch=3)
+    seen = []
+    got, metrics = generate(eng, DeviceSampler(params), prompts, max_new_tokens=24, stop_token_ids=stop, max_batch=3,
+                            on_token=lambda i, t: seen.append((i, t)))
+    assert [r.token_ids for r in got] == [r.token_ids for r in want]
+    assert [r.finish_reason for r in got] == [r.finish_reason for r in want]
+    assert {r.finish_reason for r in got} == {"stop", "length"}
+    assert sorted(seen) == sorted((i, t) for i, r in enumerate(got) for t in r.token_ids)
+    assert metrics.generated_tokens == sum(len(r.token_ids) for r in want)
+    eng.cache.check()
+    assert eng.cache.slots.held_count == 0

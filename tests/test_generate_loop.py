@@ -191,3 +191,82 @@ def test_a_batch_holds_no_more_sequences_than_the_cache_has_slots_and_a_refused_
     with pytest.raises(NoSlots):
         generate(eng, ArgmaxSampler(), [[1], [2], [3]], max_new_tokens=2, max_batch=8)
     assert not eng.seen and sorted(eng.free) == [0, 1] and not eng.steps
+
+
+# ---- the loop that runs one step ahead of itself ------------------------------------------------------
+
+class FedScriptedEngine(ScriptedEngine):
+    """The same stand-in, which also takes a step's tokens from what an earlier draw left "on the device" (here a
+    tensor like any other): the loop may then launch a step before it has looked at the tokens it feeds."""
+    takes_fed = True
+
+    def __init__(self, *a, **k):
+        super().__init__(*a, **k)
+        self.fed_steps = 0
+
+    def step(self, entries, fed=None):
+        if fed is not None:
+            self.fed_steps += 1
+            ids = fed.ids.tolist()
+            assert len(fed.rows) == len(entries) and all(len(e.tokens) == 1 for e in entries)
+            entries = [type(e)(e.slot, [ids[r]], e.want) for e, r in zip(entries, fed.rows)]
+        for e in entries:
+            assert len(self.seen[e.slot]) + len(e.tokens) <= self.cache.max_seq_tokens, "stepped beyond the longest sequence"
+        return super().step(entries)
+
+
+class StatelessSampler(ArgmaxSampler):
+    needs_history = False
+
+
+@pytest.mark.parametrize("max_new", [1, 2, 5, 9])
+def test_the_loop_that_runs_ahead_gives_the_same_results_and_keeps_the_same_books(max_new):
+    prompts = [[3, 1, 1, 0], [1, 0], [5, 7, 7, 7, 7, 7, 0], [0, 0], [8, 0]]
+
+    def script(seen):
+        n_gen = len(seen) - (seen.index(0) + 1)
+        return 9 if n_gen >= seen[0] else 20 + n_gen
+    plain, ahead = ScriptedEngine(script), FedScriptedEngine(script)
+    tokens_plain, tokens_ahead = [], []
+    want, m0 = generate(plain, ArgmaxSampler(), prompts, max_new_tokens=max_new, stop_token_ids=[9],
+                        on_token=lambda i, t: tokens_plain.append((i, t)))
+    got, m1 = generate(ahead, StatelessSampler(), prompts, max_new_tokens=max_new, stop_token_ids=[9],
+                       on_token=lambda i, t: tokens_ahead.append((i, t)))
+    assert [r.token_ids for r in got] == [r.token_ids for r in want]
+    assert [r.finish_reason for r in got] == [r.finish_reason for r in want]
+    assert tokens_ahead == tokens_plain                         # every token reported once, in the same order
+    assert (m1.generated_tokens, m1.decode_tokens) == (m0.generated_tokens, m0.decode_tokens)
+    assert not ahead.seen and sorted(ahead.closed) == sorted(plain.closed)      # every slot given back once
+    # it did run ahead (where there was a second decode step to run), and a sequence that ended on a stop token was
+    # stepped at most once more than in the plain loop; one that ended by its length never
+    if max_new > 2:
+        assert ahead.fed_steps > 0
+    fed_plain = sum(n for s in plain.steps[1:] for _, n in s)
+    fed_ahead = sum(n for s in ahead.steps[1:] for _, n in s)
+    stopped = sum(1 for r in want if r.finish_reason == "stop" and len(r.token_ids) > 1)
+    assert fed_plain <= fed_ahead <= fed_plain + stopped
+
+
+def test_the_loop_that_runs_ahead_never_steps_beyond_the_longest_sequence():
+    eng = FedScriptedEngine(lambda seen: 1, max_seq_tokens=6)
+    results, _ = generate(eng, StatelessSampler(), [[2, 2, 2, 2], [2, 2]], max_new_tokens=50)
+    assert [r.finish_reason for r in results] == ["context", "context"]
+    assert [len(r.token_ids) for r in results] == [3, 5] and not eng.seen
+
+
+def test_a_sampler_that_needs_the_history_keeps_the_plain_loop():
+    eng = FedScriptedEngine(lambda seen: 30 + len(seen))
+    results, _ = generate(eng, ArgmaxSampler(), [[1, 2, 3]], max_new_tokens=4)
+    assert results[0].token_ids == [33, 34, 35, 36] and eng.fed_steps == 0
+
+
+def test_slots_come_back_when_a_step_launched_ahead_fails():
+    class Failing(FedScriptedEngine):
+        def step(self, entries, fed=None):
+            if len(self.steps) == 3:
+                raise RuntimeError("boom")
+            return super().step(entries, fed)
+    eng = Failing(lambda seen: 1)
+    with pytest.raises(RuntimeError, match="boom"):
+        generate(eng, StatelessSampler(), [[1, 2], [3]], max_new_tokens=8)
+    assert not eng.seen and sorted(eng.closed) == [0, 1]
