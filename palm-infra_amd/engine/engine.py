@@ -12,6 +12,7 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from pathlib import Path
 
+import numpy as np
 import torch
 
 from ..cache import ModelCache
@@ -119,6 +120,20 @@ class Engine:
         return self.cache.lengths[slot]
 
     # ---- the step ----------------------------------------------------------------------------
+    @staticmethod
+    def _entry(e) -> StepEntry:
+        """The entry with its tokens as an array of integers (a long prompt is checked and laid out by numpy, not
+        token by token)."""
+        if not isinstance(e, StepEntry):
+            e = StepEntry(*e)
+        try:
+            tokens = np.asarray(e.tokens)
+        except Exception as exc:
+            raise StepError(f"slot {e.slot}: the tokens are no list of integers ({exc})") from None
+        if tokens.ndim != 1 or (tokens.size and tokens.dtype.kind not in "iu"):
+            raise StepError(f"slot {e.slot}: the tokens are no list of integers (they come as {tokens.dtype}, {tokens.ndim} axes)")
+        return StepEntry(e.slot, tokens.astype(np.int64, copy=False), list(e.want))
+
     def _validate(self, entries) -> None:
         if not entries:
             raise StepError("a step needs at least one sequence")
@@ -131,9 +146,9 @@ class Engine:
                 raise StepError(f"slot {e.slot} is not open")
             if len(e.tokens) == 0:
                 raise StepError(f"slot {e.slot} brings no tokens")
-            for t in e.tokens:
-                if not 0 <= int(t) < self.vocab_size:
-                    raise StepError(f"token id {t} lies outside the vocabulary of {self.vocab_size}")
+            lo, hi = int(e.tokens.min()), int(e.tokens.max())
+            if lo < 0 or hi >= self.vocab_size:
+                raise StepError(f"token id {lo if lo < 0 else hi} lies outside the vocabulary of {self.vocab_size}")
             for w in e.want:
                 if not 0 <= int(w) < len(e.tokens):
                     raise StepError(f"slot {e.slot}: logits wanted at place {w} of {len(e.tokens)} tokens")
@@ -145,7 +160,7 @@ class Engine:
         ``fed``: every entry brings one token, and which one is not known on the host yet: entry k's is
         ``fed.ids[fed.rows[k]]`` on the device (what its ``tokens`` holds is a stand-in).  The step is then launched
         without waiting for the device, so that a caller can look at one step's tokens while the next one runs."""
-        entries = [e if isinstance(e, StepEntry) else StepEntry(*e) for e in entries]
+        entries = [self._entry(e) for e in entries]
         self._validate(entries)
         if fed is not None:
             return self._run_fed(entries, fed)
@@ -310,7 +325,7 @@ class Engine:
         cache.reserve(growth)
         start = cache.lengths[e.slot]
         state = self._recorded(("prompt", bucket), bucket, 2, 1)
-        ctx = make_context([e.slot, cache.pad_slot], [start, 0], [list(map(int, e.tokens)), [0] * (bucket - n)], self.dtype,
+        ctx = make_context([e.slot, cache.pad_slot], [start, 0], [e.tokens, [0] * (bucket - n)], self.dtype,
                            self.device, into=state["buf"], max_new=bucket)
         state["rows"].copy_(torch.tensor([int(e.want[0])], dtype=torch.int32))
         logits = self._replay(state, ctx)
@@ -343,7 +358,7 @@ class Engine:
         growth = [(e.slot, len(e.tokens)) for e in entries]
         cache.reserve(growth)
         starts = [cache.lengths[e.slot] for e in entries]
-        ctx = make_context([e.slot for e in entries], starts, [list(map(int, e.tokens)) for e in entries],
+        ctx = make_context([e.slot for e in entries], starts, [e.tokens for e in entries],
                            self.dtype, self.device)
         want_rows = [ctx.host["cu"][b] + int(w) for b, e in enumerate(entries) for w in e.want]
         if want_rows:

@@ -27,6 +27,7 @@ from __future__ import annotations
 
 from dataclasses import dataclass, field
 
+import numpy as np
 import torch
 
 from ..config.spec import PartSpec
@@ -115,16 +116,24 @@ def make_context(slots, starts, new_tokens, dtype, device, max_total=None, into:
     recorded step is sized for the largest step it will be replayed for).
     ``staging`` (with ``into``): a pinned host buffer of the same size through which the arrays go to the device
     without the host waiting for the device; the caller must not write it again before that copy has run."""
+    # laid out with numpy: a prompt of some thousand tokens as Python lists costs the host a millisecond before the
+    # first kernel is launched
     counts = [len(t) for t in new_tokens]
-    ids = [t for seq in new_tokens for t in seq]
-    pos = [starts[b] + j for b in range(len(slots)) for j in range(counts[b])]
-    tslot = [slots[b] for b in range(len(slots)) for _ in range(counts[b])]
     cu = [0]
     for c in counts:
         cu.append(cu[-1] + c)
-    n, B = len(ids), len(slots)
-    # one transfer for all index arrays
-    host = torch.tensor(ids + pos + tslot + list(slots) + list(starts) + counts + cu, dtype=torch.int32)
+    n, B = cu[-1], len(slots)
+    packed = np.empty((context_ints(n, B),), dtype=np.int32)
+    for b in range(B):
+        lo, hi = cu[b], cu[b + 1]
+        packed[lo:hi] = new_tokens[b]
+        packed[n + lo:n + hi] = np.arange(starts[b], starts[b] + counts[b], dtype=np.int32)
+        packed[2 * n + lo:2 * n + hi] = slots[b]
+    o = 3 * n
+    for arr in (slots, starts, counts, cu):
+        packed[o:o + len(arr)] = arr
+        o += len(arr)
+    host = torch.from_numpy(packed)
     if into is None:
         flat = host.to(device)
     else:
