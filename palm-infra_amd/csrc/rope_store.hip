@@ -41,6 +41,20 @@ __global__ __launch_bounds__(WAVE) void qk_norm_rope_store_kernel(
     const int kind = head < nh ? 0 : (head < nh + nkv ? 1 : 2);
     if (kind != 0 && !write_cache) return;
     const TIN* src = qkv + ((size_t)t * (nh + 2 * nkv) + head) * hd;
+    // What does not depend on the row is asked for first (the position, its page, the first rotation pair's cos and
+    // sin, the norm weight): the kernel's time is the round trips to memory that follow each other.
+    const int pos = positions[t];
+    const bool rotate = kind != 2 && cos_t && rotary_dim > 0;
+    const int half = rotary_dim / 2;
+    float c0 = 1.f, s0 = 0.f;
+    if (rotate && lane < half) {
+        c0 = cos_t[(size_t)t * half + lane];
+        s0 = sin_t[(size_t)t * half + lane];
+    }
+    int page = 0;
+    if (kind != 0) page = block_table[(size_t)tok_slot[t] * max_pages + pos / PAGE_TOKENS];
+    const float* norm_w = kind == 0 ? q_norm_w : (kind == 1 ? k_norm_w : nullptr);
+    const float w0 = norm_w && lane < hd ? norm_w[lane] : 1.f;
 
     float ss = 0.f;
     for (int d = lane; d < hd; d += WAVE) {
@@ -49,21 +63,18 @@ __global__ __launch_bounds__(WAVE) void qk_norm_rope_store_kernel(
         vals[d] = v;
         ss += v * v;
     }
-    const float* norm_w = kind == 0 ? q_norm_w : (kind == 1 ? k_norm_w : nullptr);
     if (norm_w) {
         ss = wave_sum(ss);
         const float inv = 1.0f / sqrtf(ss / (float)hd + eps);
-        for (int d = lane; d < hd; d += WAVE) vals[d] = vals[d] * inv * norm_w[d];
+        for (int d = lane; d < hd; d += WAVE) vals[d] = vals[d] * inv * (d == lane ? w0 : norm_w[d]);
     }
     __syncthreads();
 
-    const int pos = positions[t];
-    if (kind != 2 && cos_t && rotary_dim > 0) {
-        const int half = rotary_dim / 2;
+    if (rotate) {
         for (int i = lane; i < half; i += WAVE) {
             const int a = pairing == 0 ? i : 2 * i;
             const int b = pairing == 0 ? i + half : 2 * i + 1;
-            const float c = cos_t[(size_t)t * half + i], s = sin_t[(size_t)t * half + i];
+            const float c = i == lane ? c0 : cos_t[(size_t)t * half + i], s = i == lane ? s0 : sin_t[(size_t)t * half + i];
             const float x0 = vals[a], x1 = vals[b];
             vals[a] = x0 * c - x1 * s;
             vals[b] = x0 * s + x1 * c;
@@ -73,7 +84,6 @@ __global__ __launch_bounds__(WAVE) void qk_norm_rope_store_kernel(
 
     if (kind == 2) {
         const int g = head - nh - nkv;
-        const int page = block_table[(size_t)tok_slot[t] * max_pages + pos / PAGE_TOKENS];
         T* dst = v_cache + ((size_t)page * nkv + g) * hd * PAGE_TOKENS + pos % PAGE_TOKENS;
         for (int d = lane; d < hd; d += WAVE) dst[(size_t)d * PAGE_TOKENS] = from_float<T>(vals[d]);
         return;
@@ -83,7 +93,6 @@ __global__ __launch_bounds__(WAVE) void qk_norm_rope_store_kernel(
         dst = q_out + ((size_t)t * nh + head) * hd;
     } else {
         const int g = head - nh;
-        const int page = block_table[(size_t)tok_slot[t] * max_pages + pos / PAGE_TOKENS];
         dst = k_cache + (((size_t)page * nkv + g) * PAGE_TOKENS + pos % PAGE_TOKENS) * hd;
     }
     for (int d = lane; d < hd; d += WAVE) dst[d] = from_float<T>(vals[d]);
