@@ -440,8 +440,8 @@ def _same_caches(a, b):
 @pytest.mark.parametrize("n_slices", [1, 3, 8])
 def test_attention_decode_fused_is_the_two_kernels_in_one(ops, nh, nkv, hd, n_slices):
     """Lengths around page borders (the new token first in its page, last in it, the only one of its sequence), rows
-    as bfloat16 and as one, two and three planes."""
-    for planes, lengths in ((0, [300]), (1, [1]), (2, [64, 65, 700, 7, 128, 129, 1]), (3, [193, 2])):
+    as bfloat16 and as one to five planes."""
+    for planes, lengths in ((0, [300]), (1, [1]), (2, [64, 65, 700, 7, 128, 129, 1]), (3, [193, 2]), (4, [130, 64, 1]), (5, [66])):
         one, two, ca, cb, before = _fused_case(ops, nh, nkv, hd, lengths, n_slices, planes, seed=hd + planes)
         assert _one_ulp(one, two), (planes, lengths, float((one - two).abs().max()))
         _same_caches(ca, cb)
