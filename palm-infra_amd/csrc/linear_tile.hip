@@ -13,9 +13,9 @@
 // eight 16-byte chunks are permuted by the row number (chunk ^ ((row >> 1) & 7)) so that the 16-byte reads of a
 // matrix instruction's operand, consecutive rows at the same k, spread over the banks.  The lane that fills a place
 // fetches the chunk that belongs there, so the permutation costs nothing.
-// What bounds it: a compute unit reads at most some 45 GB/s from L2 (measured with the products and the LDS reads
-// taken out, through registers or straight into LDS, with one, two or three stages in flight), 11 to 12 TB/s for
-// the chip; a tile of 256 x 256 needs 128 KB for every 64 k-values, which is 270 us for the gate/up product of
+// What bounds it: a compute unit reads at most some 45 GB/s of what its die's L2 does not hold (measured with the
+// products and the LDS reads taken out, through registers or straight into LDS, with one, two or three stages in
+// flight; a long prompt's operands are far larger than L2), 11 to 12 TB/s for the chip; a tile of 256 x 256 needs 128 KB for every 64 k-values, which is 270 us for the gate/up product of
 // 2,048 rows, about what the library's kernel of the same tile takes in all.  This kernel overlaps its products
 // and its reads less well (360 us), so prompts keep the library; it serves where a library call cannot: float32
 // results of many rows (logits at many places), and the epilogues below.
