@@ -503,3 +503,37 @@ def test_attention_decode_fused_says_what_it_serves(ops):
     i32 = lambda xs: torch.tensor(xs, dtype=torch.int32).to(DEV)
     with pytest.raises(KernelError, match="multiple of 64"):
         ops.attention_decode_fused(qkv, kc, vc, i32([[0, 1]]), i32([0]), i32([3]), 2, 1, 80, 1.0, None, 1)
+
+
+def test_attention_decode_fused_finds_a_far_key_and_respects_the_window_edge(ops):
+    """One cached key among hundreds dominates the new token's query (the new token's own key does not): the output
+    is that key's value, wherever it lies (first, last before the new one, on a page's border, in any slice); just
+    outside a window it is out of reach."""
+    nh, nkv, hd = 4, 2, 128
+    W = (nh + 2 * nkv) * hd
+    i32 = lambda xs: torch.tensor(xs, dtype=torch.int32).to(DEV)
+
+    def run(L, at, n_slices, window=None):
+        k = rand(L - 1, nkv, hd, seed=1, scale=0.1)
+        v = rand(L - 1, nkv, hd, seed=2)
+        k[at] = 0
+        k[at, :, 5] = 8.0
+        row = rand(1, W, seed=3, scale=0.1)
+        row[0, : nh * hd].reshape(nh, hd)[:, 5] = 8.0                    # every query head looks for element 5
+        table = torch.arange((L + 63) // 64 + 1, dtype=torch.int32).flip(0)[None, :].contiguous()
+        kc = rand(table.shape[1], nkv, 64, hd, seed=4).to(DEV)           # stale values everywhere else
+        vc = rand(table.shape[1], nkv, hd, 64, seed=5).to(DEV)
+        _fill_cache(kc, vc, table, 0, k.to(DEV), v.to(DEV))
+        got = ops.attention_decode_fused(row.to(DEV), kc, vc, table.to(DEV), i32([0]), i32([L - 1]), nh, nkv, hd, 1.0, window,
+                                         n_slices)
+        return got.float().cpu().reshape(nh, hd), v[at].float().repeat_interleave(nh // nkv, 0)
+
+    for n_slices in (1, 5):
+        for L, at in ((700, 13), (700, 0), (700, 698), (513, 448), (65, 63), (66, 64), (130, 31), (2, 0)):
+            got, want = run(L, at, n_slices)
+            assert torch.allclose(got, want, atol=1e-2), (L, at, n_slices)
+        L, w = 300, 70                                                   # the query sits at L-1 and reads keys L-w .. L-1
+        got, want = run(L, L - w, n_slices, window=w)
+        assert torch.allclose(got, want, atol=1e-2), n_slices
+        got, want = run(L, L - w - 1, n_slices, window=w)
+        assert not torch.allclose(got, want, atol=0.2), n_slices
