@@ -326,7 +326,11 @@ def main(argv=None) -> int:
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": round(achieved / PEAK_HBM_GBS, 4),
                      # the step's dominant kernels alone (a launch for each layer in a recorded graph, event-timed)
-                     "kernels": kernels, **{f"frac_{k}": v["frac"] for k, v in kernels.items()}},
+                     "kernels": kernels, **{f"frac_{k}": v["frac"] for k, v in kernels.items()},
+                     # the same fraction for the steps of one and of 64 sequences (their bytes over their time)
+                     **{f"frac_{name}": round(decode_bytes(cfg, b, mid_context) * tps / b / 1e9 / PEAK_HBM_GBS, 4)
+                        for name, b, tps in (("decode_b1", 1, points.get("decode_b1")), ("decode_b64", 64, points.get("decode_b64")))
+                        if tps}},
         "points": points,
     }
     print(json.dumps(record), flush=True)
