@@ -18,6 +18,9 @@ from __future__ import annotations
 
 from dataclasses import dataclass
 
+import copy
+
+import numpy as np
 import torch
 
 from .pool import PAGE_TOKENS, CacheFull, CacheMisuse, FreeList, PageTable, pages_for
@@ -30,8 +33,11 @@ from .pool import PAGE_TOKENS, CacheFull, CacheMisuse, FreeList, PageTable, page
 # need by name: a mixer with storage of another shape brings a need and a group class of its own.
 #
 # A group has: ``need``, ``n_entries``; ``table`` (a ``PageTable`` if the storage grows with the sequence, else
-# None); ``sync()`` (bring device copies of host bookkeeping up to date); ``on_open(slot)``; ``nbytes()``;
-# ``attach(layer_cache, entry)``.
+# None; its ``window`` says whether pages are given back as a sequence grows); ``sync()`` (bring device copies of
+# host bookkeeping up to date, without making the host wait for the device); ``on_open(slot)``; ``nbytes()``;
+# ``attach(layer_cache, entry)``, which hangs what the part is to see on the entry's ``LayerCache`` under a field of
+# the need's choosing (the shipped ones use ``kv``, ``rows[name]`` and ``states[name]``).  Storage in pages derives
+# from ``PagedGroup``, which reads one thing of its need: ``window`` (absent or None: every position is kept).
 
 @dataclass(frozen=True)
 class KVNeed:
@@ -76,26 +82,44 @@ class PagedGroup:
 
     def __init__(self, need, n_entries: int, n_pages: int, n_slots: int, max_pages_per_slot: int, device):
         self.need, self.n_entries, self.n_pages = need, n_entries, n_pages
-        self.table = PageTable(n_pages, n_slots, max_pages_per_slot, need.window)
+        self.table = PageTable(n_pages, n_slots, max_pages_per_slot, getattr(need, "window", None))
         self.pad_page = n_pages
         self.table_host = torch.full((n_slots + 1, max_pages_per_slot), self.pad_page, dtype=torch.int32)
         self.table_dev = self.table_host.to(device)
+        # Stale rows go to the device through pinned memory, two buffers in turn, each written again only after the
+        # copy that last read it has run: the host never waits for the step that is still running (a step launched
+        # ahead of its predecessor's results would otherwise stop at every page border of every sequence).
+        self._pinned = torch.device(device).type == "cuda"
+        self._staging: list = [None, None]           # int32 [rows, pages of a slot + 1]: a slot's pages, then its number
+        self._staged: list = [None, None]
+        self._turn = 0
 
     def sync(self) -> None:
-        """Bring the device's copy of the page lists up to date: all stale rows in one indexed copy.
-        The rows travel in fresh host tensors, so a later change on the host cannot reach a copy that
-        the device has not run yet."""
+        """Bring the device's copy of the page lists up to date: all stale rows in one indexed copy, queued on
+        the stream like the step that reads them."""
         if not self.table.dirty:
             return
         slots = sorted(self.table.dirty)
-        rows = torch.full((len(slots), self.table_host.shape[1]), self.pad_page, dtype=torch.int32)
+        k, width = len(slots), self.table_host.shape[1]
+        turn = self._turn = self._turn ^ 1
+        if self._staged[turn] is not None:
+            self._staged[turn].synchronize()
+        buf = self._staging[turn]
+        if buf is None or buf.shape[0] < k:
+            buf = self._staging[turn] = torch.empty((max(k, 16), width + 1), dtype=torch.int32, pin_memory=self._pinned)
+        rows = buf.numpy()[:k]
+        rows[:, :width] = self.pad_page
         for i, slot in enumerate(slots):
             pages = self.table.slot_pages[slot]
             if pages:
-                rows[i, :len(pages)] = torch.tensor([p if p >= 0 else self.pad_page for p in pages], dtype=torch.int32)
-            self.table_host[slot] = rows[i]
-        index = torch.tensor(slots, dtype=torch.long)
-        self.table_dev.index_copy_(0, index.to(self.table_dev.device), rows.to(self.table_dev.device))
+                rows[i, :len(pages)] = np.where(np.asarray(pages, dtype=np.int32) >= 0, pages, self.pad_page)
+            rows[i, width] = slot
+        self.table_host[slots] = buf[:k, :width]
+        up = buf[:k].to(self.table_dev.device, non_blocking=True)
+        self.table_dev.index_copy_(0, up[:, width].long(), up[:, :width])
+        if self._pinned:
+            self._staged[turn] = torch.cuda.Event()
+            self._staged[turn].record()
         self.table.dirty.clear()
 
     def on_open(self, slot: int) -> None:
@@ -217,8 +241,6 @@ class ModelCache:
         self.groups = [need.make_group(len(m), n_pages, self.max_seqs, max_pages_per_slot, dtype, device)
                        for need, m in members.items()]
         self.paged_groups = [g for g in self.groups if g.table is not None]       # storage that grows: pages to manage
-        self.kv_groups = [g for g in self.groups if isinstance(g, KVGroup)]
-        self.state_groups = [g for g in self.groups if isinstance(g, StateGroup)]
 
         self.layer_caches: list[LayerCache] = [LayerCache() for _ in needs]
         for group, entries in zip(self.groups, members.values()):
@@ -229,8 +251,12 @@ class ModelCache:
                     raise ValueError(f"run-order entry {i}: {e}") from None
         for i, src in enumerate(shares):
             if src is not None:
-                s = self.layer_caches[src]
-                self.layer_caches[i] = LayerCache(kv=s.kv, kv_entry=s.kv_entry, writes=False, states=s.states, rows=s.rows)
+                self.layer_caches[i] = copy.copy(self.layer_caches[src])      # whatever its groups hung on it
+                self.layer_caches[i].writes = False
+
+    def groups_of(self, need_type) -> list:
+        """The groups whose need is of the given class, in the order in which the run order first asked for them."""
+        return [g for g in self.groups if isinstance(g.need, need_type)]
 
     # ---- sequences ---------------------------------------------------------------------------
     def open(self) -> int:
@@ -259,7 +285,7 @@ class ModelCache:
                 raise CacheFull(f"slot {slot}: {self.lengths[slot]} + {n_new} tokens exceed the longest sequence "
                                 f"the cache takes ({self.max_seq_tokens})")
         for g in self.paged_groups:
-            if in_pieces and g.need.window:
+            if in_pieces and g.table.window:
                 continue
             need = sum(g.table.pages_needed(slot, self.lengths[slot] + n) for slot, n in growth)
             if need > g.table.pages.free_count:

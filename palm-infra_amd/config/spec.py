@@ -18,13 +18,40 @@ ROLES = ("matrix", "table", "vector", "integer")
 
 
 @dataclass(frozen=True)
+class Stored:
+    """How a piece of a parameter lies in the checkpoint when it is not a whole tensor in the parameter's own layout:
+    the stored tensor has shape ``shape``; of it the rows ``rows = (a, b)`` are taken (None: all); ``transposed``: what
+    was taken is the transpose of the piece (a matrix that the checkpoint keeps as [in, out]).  So a checkpoint that
+    stores q, k and v fused in one tensor, in any order, is three pieces with three row ranges of one name."""
+    shape: tuple[int, ...]
+    rows: tuple[int, int] | None = None
+    transposed: bool = False
+
+    def piece_shape(self) -> tuple[int, ...]:
+        shape = tuple(self.shape)
+        if self.rows is not None:
+            a, b = self.rows
+            if not shape or not 0 <= a < b <= shape[0]:
+                raise ValueError(f"rows {a}:{b} do not lie in a stored tensor of shape {shape}")
+            shape = (b - a,) + shape[1:]
+        if self.transposed:
+            if len(shape) != 2:
+                raise ValueError(f"only a matrix can be stored transposed, not a tensor of shape {shape}")
+            shape = (shape[1], shape[0])
+        return shape
+
+
+@dataclass(frozen=True)
 class TensorRef:
-    """One parameter of a part: one or more tensors of the checkpoint, joined along their rows."""
+    """One parameter of a part: one or more pieces, joined along their rows.  Piece i is the checkpoint tensor
+    ``names[i]`` and has shape ``shapes[i]`` in the parameter; usually it is that tensor whole and as stored, else
+    ``stored[i]`` says how it lies in the tensor (a range of its rows, transposed)."""
     names: tuple[str, ...]
     shapes: tuple[tuple[int, ...], ...]
     role: str = "matrix"
     # how the random-weights writer fills it: ("normal", mean, std)
     init: tuple = ("normal", 0.0, 0.02)
+    stored: tuple = ()          # empty, or one ``Stored`` or None for each piece
 
     def __post_init__(self):
         if self.role not in ROLES:
@@ -34,19 +61,40 @@ class TensorRef:
         tail = self.shapes[0][1:]
         if any(s[1:] != tail for s in self.shapes):
             raise ValueError(f"tensors {self.names} cannot be joined along rows: shapes {self.shapes}")
+        if self.stored:
+            if len(self.stored) != len(self.names):
+                raise ValueError("TensorRef needs one entry of `stored` (or None) for each name")
+            for name, shape, how in zip(self.names, self.shapes, self.stored):
+                if how is not None and tuple(how.piece_shape()) != tuple(shape):
+                    raise ValueError(f"piece {name}: what is taken of the stored tensor has shape {how.piece_shape()}, "
+                                     f"the parameter expects {tuple(shape)}")
 
     @property
     def shape(self) -> tuple[int, ...]:
         rows = sum(s[0] for s in self.shapes)
         return (rows,) + tuple(self.shapes[0][1:])
 
+    @property
+    def key(self) -> tuple:
+        """What tells this parameter from every other one (two parameters may take different rows of one tensor)."""
+        return (self.names, self.stored) if any(h is not None for h in self.stored) else self.names
 
-def tensor(name: str, shape, role: str = "matrix", init=("normal", 0.0, 0.02)) -> TensorRef:
-    return TensorRef((name,), (tuple(int(s) for s in shape),), role, tuple(init))
+    def pieces(self):
+        """(name, shape in the parameter, Stored or None) for each piece, in the order of the rows."""
+        stored = self.stored or (None,) * len(self.names)
+        return list(zip(self.names, self.shapes, stored))
+
+    def stored_shapes(self):
+        """(name, shape as the checkpoint stores the tensor) for each piece."""
+        return [(name, tuple(how.shape) if how is not None else tuple(shape)) for name, shape, how in self.pieces()]
 
 
-def joined(names, shapes, role: str = "matrix", init=("normal", 0.0, 0.02)) -> TensorRef:
-    return TensorRef(tuple(names), tuple(tuple(int(x) for x in s) for s in shapes), role, tuple(init))
+def tensor(name: str, shape, role: str = "matrix", init=("normal", 0.0, 0.02), stored: Stored | None = None) -> TensorRef:
+    return TensorRef((name,), (tuple(int(s) for s in shape),), role, tuple(init), (stored,) if stored is not None else ())
+
+
+def joined(names, shapes, role: str = "matrix", init=("normal", 0.0, 0.02), stored=()) -> TensorRef:
+    return TensorRef(tuple(names), tuple(tuple(int(x) for x in s) for s in shapes), role, tuple(init), tuple(stored))
 
 
 @dataclass(frozen=True)
@@ -114,16 +162,16 @@ class ModelSpec:
         seen, out = set(), []
         for part in self.parts():
             for ref in part.tensors.values():
-                if ref.names not in seen:
-                    seen.add(ref.names)
+                if ref.key not in seen:
+                    seen.add(ref.key)
                     out.append(ref)
         return out
 
     def expected_tensors(self) -> dict[str, tuple[tuple[int, ...], str]]:
-        """Checkpoint tensor name -> (shape, role)."""
+        """Checkpoint tensor name -> (shape as stored, role)."""
         out = {}
         for ref in self.tensor_refs():
-            for name, shape in zip(ref.names, ref.shapes):
+            for name, shape in ref.stored_shapes():
                 if name in out and out[name][0] != shape:
                     raise ValueError(f"tensor {name} is used with two shapes: {out[name][0]} and {shape}")
                 out[name] = (shape, ref.role)

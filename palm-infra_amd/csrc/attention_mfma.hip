@@ -130,6 +130,21 @@ __device__ inline float score_page(const PageOperands& ops, const bf16x8 (&qv)[K
     return alpha;
 }
 
+// A key beyond `hi` (an in-page index) has weight zero, but its column of V^T would still be multiplied, and pages
+// are handed out uncleared: what an earlier request left there (a NaN or an infinity, if its activations overflowed)
+// times zero is NaN.  So the values of such keys are taken as zero.  Only the page that holds the column's last key
+// has any; this lane's fragments hold keys 32 h + 8 g + e.
+__device__ inline void blank_values_after(PageOperands& ops, int hi, int g) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const bool seen = h * 32 + g * 8 + e <= hi;
+#pragma unroll
+            for (int dt = 0; dt < DTILES; ++dt) ops.v[dt][h][e] = seen ? ops.v[dt][h][e] : (__bf16)0.0f;
+        }
+}
+
 __device__ inline void weigh_values(const PageOperands& ops, const bf16x8 (&pv)[2], float alpha, Columns& c) {
 #pragma unroll
     for (int dt = 0; dt < DTILES; ++dt) {
@@ -165,6 +180,7 @@ __device__ inline void attend_pages(const bf16_t* __restrict__ k_cache, const bf
         bf16x8 pv[2];
         const float alpha = score_page(ops, qv, first - p * PAGE_TOKENS, last - p * PAGE_TOKENS, scale_log2, c, g, pv);
         if (more) load_keys(k_cache + next, r, g, ops);
+        if (last - p * PAGE_TOKENS < PAGE_TOKENS - 1) blank_values_after(ops, last - p * PAGE_TOKENS, g);   // the same in every lane
         weigh_values(ops, pv, alpha, c);
         if (more) load_values(v_cache + next, r, g, ops);
         base = next;
@@ -182,6 +198,25 @@ __device__ inline void load_query(const bf16_t* qrow, bool valid, int g, bf16x8 
 }
 
 // ---- decode ---------------------------------------------------------------------------------------
+// How a query at position `pos` cuts its key range into slices of whole pages.  The decode kernels and the merge
+// must agree on it (the merge reads only the records of slices that hold pages), so it is written once.
+struct SliceCut {
+    int first;            // the first key the query sees
+    int page_lo;          // the page that holds it
+    int n_pages;          // pages from there to the query's own
+    int per;              // pages a slice
+    int live;             // slices that hold pages: 1 <= live <= n_slices
+    __device__ SliceCut(int pos, int window, int n_slices) {
+        first = window > 0 ? max(0, pos - window + 1) : 0;
+        page_lo = first / PAGE_TOKENS;
+        n_pages = pos / PAGE_TOKENS - page_lo + 1;
+        per = (n_pages + n_slices - 1) / n_slices;
+        live = (n_pages + per - 1) / per;
+    }
+    __device__ int begin(int slice) const { return page_lo + slice * per; }
+    __device__ int end(int slice) const { return min(begin(slice) + per, page_lo + n_pages); }
+};
+
 // grid (slices, nkv * query groups, sequences), one wave each.  Workspace per (sequence, head, slice):
 // m, l, two floats unused, then HD floats of the unnormalised output (which so start on 16 bytes).
 constexpr int WORK_O = 4, WORK_STRIDE = HD + WORK_O;
@@ -229,10 +264,8 @@ __global__ __launch_bounds__(WAVE) DECODE_WAVES_PER_SIMD void attention_decode_k
     const int kvh = blockIdx.y / groups, qg = blockIdx.y % groups;
     const int lane = threadIdx.x, r = lane % 16, g = lane / 16;
     const int pos = seq_start[b];                       // the query's position; keys 0..pos are in the cache
-    const int first = window > 0 ? max(0, pos - window + 1) : 0;
-    const int page_lo = first / PAGE_TOKENS, n_pages = pos / PAGE_TOKENS - page_lo + 1;
-    const int per = (n_pages + n_slices - 1) / n_slices;
-    const int p0 = page_lo + slice * per, p1 = min(p0 + per, page_lo + n_pages);
+    const SliceCut cut(pos, window, n_slices);
+    const int first = cut.first, p0 = cut.begin(slice), p1 = cut.end(slice);
     const int head = kvh * G + qg * 16 + r;             // this lane's query head (column r)
     const bool valid = qg * 16 + r < G;
 
@@ -278,11 +311,7 @@ __global__ __launch_bounds__(WAVE) void attention_merge_kernel(const float* __re
         }
     };
     ask(0);
-    const int pos = seq_start[blockIdx.x / nh];
-    const int first = window > 0 ? max(0, pos - window + 1) : 0;
-    const int n_pages = pos / PAGE_TOKENS - first / PAGE_TOKENS + 1;
-    const int per = (n_pages + n_slices - 1) / n_slices;
-    const int live = (n_pages + per - 1) / per;                 // as the decode kernels cut the range: <= n_slices
+    const int live = SliceCut(seq_start[blockIdx.x / nh], window, n_slices).live;       // as the decode kernels cut the range
     float m = lane < live ? mine.x : -INFINITY, l = 0.f;
     for (int s = lane + WAVE; s < live; s += WAVE) m = fmaxf(m, w[(size_t)s * WORK_STRIDE]);
     m = wave_max(m);
@@ -620,10 +649,8 @@ __global__ __launch_bounds__(WAVE) DECODE_WAVES_PER_SIMD void attention_decode_f
         start.ask();
 
         const int pos = seq_start[b];
-        const int first = window > 0 ? max(0, pos - window + 1) : 0;
-        const int page_lo = first / PAGE_TOKENS, n_pages = pos / PAGE_TOKENS - page_lo + 1;
-        const int per = (n_pages + n_slices - 1) / n_slices;
-        const int p0 = page_lo + slice * per, p1 = min(p0 + per, page_lo + n_pages);
+        const SliceCut cut(pos, window, n_slices);
+        const int first = cut.first, p0 = cut.begin(slice), p1 = cut.end(slice);
         const int* pages = block_table + (size_t)seq_slot[b] * max_pages;
         const int page = pos / PAGE_TOKENS;
         start.owner = write_cache && page >= p0 && page < p1;
@@ -858,6 +885,22 @@ __device__ inline void page_into_lds(const bf16_t* __restrict__ kp, const bf16_t
         load_16_bytes_a_lane_into_lds(reinterpret_cast<const char*>(vp) + src.v[i], lds_address(v_lds + (i * PF_WAVES + wave) * KB));
 }
 
+// The page that holds a sequence's last key also holds, beyond it, what an earlier owner of the page left there
+// (pages are handed out uncleared).  Those keys have weight zero in every column, but their columns of V^T are
+// multiplied all the same, and zero times a NaN or an infinity is NaN: they are made zero in LDS, once, before the
+// page is used.  `tail`: the last key of the sequence, as an index into the page.  (A barrier must follow.)
+__device__ inline void blank_values_after(bf16_t* v_lds, int tail) {
+    for (int idx = threadIdx.x; idx < HD * (PAGE_TOKENS / 8); idx += PF_THREADS) {
+        const int d = idx / (PAGE_TOKENS / 8), chunk = idx % (PAGE_TOKENS / 8);
+        if (chunk * 8 + 7 <= tail) continue;
+        bf16x8* at = reinterpret_cast<bf16x8*>(v_lds + d * V_STRIDE + (chunk ^ v_swizzle(d)) * 8);
+        bf16x8 v = *at;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = chunk * 8 + e <= tail ? v[e] : (__bf16)0.0f;
+        *at = v;
+    }
+}
+
 struct Unit {                 // one (head, 16 query positions): the wave's share of it
     bool live;                // false: the wave has no such unit (fewer units than slots)
     bool active;              // the page at hand holds keys that some column of the unit sees
@@ -1029,6 +1072,7 @@ __global__ __launch_bounds__(PF_THREADS) PF_WAVES_PER_SIMD void attention_prefil
     const int lane = threadIdx.x % WAVE, r = lane % 16, g = lane / 16;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);      // the same in every lane: what follows from it stays scalar
     const int start = seq_start[b];
+    const int seq_tail = start + n_new - 1;                     // the sequence's last key
     const int heads_here = min(hg, G - hgi * hg);
     const int n_units = heads_here * subs;
     const int* pages = block_table + (size_t)seq_slot[b] * max_pages;
@@ -1099,6 +1143,10 @@ __global__ __launch_bounds__(PF_THREADS) PF_WAVES_PER_SIMD void attention_prefil
         for (int p = p_lo; p <= p_hi; ++p) {
             const int buf = (p - p_lo) & 1;
             const bool more = p < p_hi;
+            if (seq_tail - p * PAGE_TOKENS < PAGE_TOKENS - 1) {     // the sequence's last page (no page follows it)
+                blank_values_after(v_lds + buf * V_TILE, seq_tail - p * PAGE_TOKENS);
+                __syncthreads();
+            }
             if (more) {                                         // in flight while this page is used
                 const size_t next = ((size_t)pages[p + 1] * nkv + kvh) * PAGE_TOKENS * HD;
                 if constexpr (PF_DMA) {     // straight into the other buffer, whose last readers passed the barrier a page ago
@@ -1144,6 +1192,10 @@ __global__ __launch_bounds__(PF_THREADS) PF_WAVES_PER_SIMD void attention_prefil
             __syncthreads();
             stage_values(pf, v_lds);
             __syncthreads();
+            if (seq_tail - p * PAGE_TOKENS < PAGE_TOKENS - 1) {
+                blank_values_after(v_lds, seq_tail - p * PAGE_TOKENS);
+                __syncthreads();
+            }
             unit_values(v_lds, u, r, g, pv, alpha, rescale);
             if (more) prefetch_values(v_cache + next, pf);
         }

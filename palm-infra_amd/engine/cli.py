@@ -7,7 +7,8 @@ Options keep the reference's names and meanings where it has them (examples/cli_
 ``--presence-penalty``, ``--frequency-penalty``, ``--seed``, ``--output kv|human``, ``--profile``,
 ``--trace``.  ``--package`` names a
 model folder here (``--model`` is the same): there is no packaging step.  New: ``--dtype``, ``--batch``, ``--stop-token-ids``, ``--ignore-eos``,
-``--prompt-ids``, ``--prompt-lengths``, ``--random-config`` (random weights from a config.json or a named size).  Options of
+``--prompt-ids``, ``--prompt-lengths``, ``--random-config`` (random weights from a config.json or a named size),
+``--allow-extra-tensors`` (tensors the model does not name are listed and left alone instead of refused).  Options of
 the reference that select a backend, offload, vision or speculation have no meaning here and are
 refused by the parser.
 
@@ -32,6 +33,8 @@ def build_parser(prog: str, bench: bool) -> argparse.ArgumentParser:
     ap.add_argument("--package", "--model", dest="model", help="model folder: config.json + safetensors")
     ap.add_argument("--random-config", "--random", dest="random_config",
                     help="instead of --package: a config.json, or a named size, to fill with random weights")
+    ap.add_argument("--allow-extra-tensors", action="store_true",
+                    help="load a checkpoint that holds tensors the model does not name (they are listed and left alone)")
     ap.add_argument("--prompt", action="append", default=[], help="prompt text (needs tokenizer.json); may repeat")
     ap.add_argument("--prompt-file", help="read prompt text from a file")
     ap.add_argument("--prompt-ids", action="append", default=[], help="prompt as comma-separated token ids; may repeat")
@@ -118,7 +121,7 @@ def collect_prompts(args, tokenizer, vocab_size: int):
 def make_engine(args):
     from .engine import Engine
     if args.model:
-        return Engine.from_dir(args.model, dtype=args.dtype, max_tokens=args.n_ctx)
+        return Engine.from_dir(args.model, dtype=args.dtype, max_tokens=args.n_ctx, strict_weights=not args.allow_extra_tensors)
     if args.random_config:
         return Engine.from_config(config_source(args.random_config), seed=args.seed, dtype=args.dtype, max_tokens=args.n_ctx)
     raise SystemExit("--package <model folder> (or --random-config <config.json>) is required")

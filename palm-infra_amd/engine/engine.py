@@ -76,7 +76,7 @@ class Engine:
         self._decode_graphs: dict = {}            # (batch bucket, length bucket) -> recorded step, least recently used first
         self._graph_pool_handle = None
         # a windowed group gives pages back only between steps, so long prompts go through it in pieces
-        windows = [g.need.window for g in self.cache.paged_groups if g.need.window]
+        windows = [g.table.window for g in self.cache.paged_groups if g.table.window]
         self.step_tokens_per_seq = max(1024, 2 * max(windows)) if windows else None
         # the most tokens that run through the layers at once: longer steps go through in pieces, so that a step's
         # activations (the widest: tokens x twice the feed-forward width) stay within a few gigabytes
@@ -86,14 +86,17 @@ class Engine:
 
     # ---- construction ------------------------------------------------------------------------
     @classmethod
-    def from_dir(cls, model_dir, dtype="bfloat16", max_tokens: int | None = None, device="cuda:0", **options):
-        """A folder with config.json and safetensors; the model class is chosen by config.json."""
+    def from_dir(cls, model_dir, dtype="bfloat16", max_tokens: int | None = None, device="cuda:0",
+                 strict_weights: bool = True, **options):
+        """A folder with config.json and safetensors; the model class is chosen by config.json.  ``strict_weights``
+        false: tensors of the checkpoint that the model does not name are listed on standard error and left alone
+        instead of refused."""
         dt = resolve_dtype(dtype)
         model_dir = Path(model_dir)
         config = config_from_dir(model_dir)
         files = ModelFiles(model_dir)
         spec = config.spec(files.names())
-        weights = load_weights(spec, files, dt, device)
+        weights = load_weights(spec, files, dt, device, strict=strict_weights)
         return cls(config, spec, weights, dt, max_tokens or 16384, device=device, **options)
 
     @classmethod
@@ -159,7 +162,10 @@ class Engine:
 
         ``fed``: every entry brings one token, and which one is not known on the host yet: entry k's is
         ``fed.ids[fed.rows[k]]`` on the device (what its ``tokens`` holds is a stand-in).  The step is then launched
-        without waiting for the device, so that a caller can look at one step's tokens while the next one runs."""
+        without waiting for the device, so that a caller can look at one step's tokens while the next one runs.
+        Fed tokens are meant to be a sampler's draws, which lie in the vocabulary; the host cannot look at them
+        without waiting, so a recorded step takes them unchecked, and an id outside the table is not read from
+        memory but makes that sequence's logits NaN (the embedding kernel's rule)."""
         entries = [self._entry(e) for e in entries]
         self._validate(entries)
         if fed is not None:
@@ -219,14 +225,24 @@ class Engine:
         return (self.graphs_enabled and self.model.capturable and len(entries) <= self.GRAPH_MAX_BATCH
                 and all(len(e.tokens) == 1 for e in entries) and profile.active() is None)
 
-    GRAPH_LIMIT = 24        # recorded steps kept at once; the least recently used one goes when another is recorded
+    # Recorded steps kept at once, decode steps and short prompts counted apart (a burst of prompts of many lengths
+    # must not push out the decode steps that run between them); the least recently used of its kind goes when
+    # another is recorded.
+    GRAPH_LIMIT = 24
+    PROMPT_GRAPH_LIMIT = 8
 
     def _recorded(self, key, n_tokens: int, n_seqs: int, n_rows: int | None) -> dict:
         """The state of the recorded step ``key`` (made if new; the most recently used is kept last)."""
         state = self._decode_graphs.pop(key, None)
         if state is None:
-            while len(self._decode_graphs) >= self.GRAPH_LIMIT:          # a graph holds its activations and logits: bound them
-                self._decode_graphs.pop(next(iter(self._decode_graphs)))
+            is_prompt = key[0] == "prompt"
+            kin = [k for k in self._decode_graphs if (k[0] == "prompt") == is_prompt]
+            limit = self.PROMPT_GRAPH_LIMIT if is_prompt else self.GRAPH_LIMIT
+            if len(kin) >= limit:                 # a graph holds its activations and logits: bound them
+                # a step launched ahead may still be queued or running: its graph and buffers go only when it is done
+                torch.cuda.current_stream().synchronize()
+                for k in kin[:len(kin) - limit + 1]:
+                    self._decode_graphs.pop(k)
             size = context_ints(n_tokens, n_seqs)
             state = {"buf": torch.zeros((size,), dtype=torch.int32, device=self.device),
                      "staging": [torch.zeros((size,), dtype=torch.int32, pin_memory=True) for _ in range(2)],
@@ -262,9 +278,12 @@ class Engine:
             raise StepError(f"a fed row lies outside the {fed.ids.shape[0]} tokens given")
         if self._graph_serves(entries):
             return self._run_decode_graph(entries, fed)
-        # no recorded step serves these entries: the tokens come to the host first (which waits for them)
+        # no recorded step serves these entries: the tokens come to the host first (which waits for them) and are
+        # checked like any others
         ids = fed.ids.tolist()
-        return self._run([StepEntry(e.slot, [ids[int(r)]], e.want) for e, r in zip(entries, fed.rows)])
+        entries = [self._entry(StepEntry(e.slot, [ids[int(r)]], e.want)) for e, r in zip(entries, fed.rows)]
+        self._validate(entries)
+        return self._run(entries)
 
     def _run_decode_graph(self, entries, fed: FedTokens | None = None) -> torch.Tensor:
         cache = self.cache

@@ -594,14 +594,29 @@ def _attention_checks(what, q, k_cache, v_cache, block_table, nh, nkv, hd, *inde
     _need(k_cache.dtype == BF16, f"{what}: the cache is {k_cache.dtype}, not bfloat16")
 
 
+def _slices_workspace(what: str, work, B: int, nh: int, n_slices: int, hd: int, device):
+    """Where the slices' partial results cross to the merging kernel: the caller's, or a new one."""
+    need = B * nh * n_slices * (hd + 4)
+    if n_slices <= 1:
+        return None
+    if work is None:
+        return torch.empty((need,), dtype=F32, device=device)
+    _dev(what, work)
+    _need(work.dtype == F32 and work.numel() >= need, f"{what}: the workspace holds {work.numel()} {work.dtype}, "
+          f"{B} sequences x {nh} heads x {n_slices} slices need {need} float32")
+    return work
+
+
 def attention_decode(q, k_cache, v_cache, block_table, seq_slot, seq_start, nh: int, nkv: int, hd: int, scale: float,
-                     window: int | None, n_slices: int) -> torch.Tensor:
-    """One query for each sequence (row b of q, at position seq_start[b]) over keys 0..seq_start[b]."""
+                     window: int | None, n_slices: int, work: torch.Tensor | None = None) -> torch.Tensor:
+    """One query for each sequence (row b of q, at position seq_start[b]) over keys 0..seq_start[b].  ``work``: a
+    float32 workspace of B * nh * n_slices * (hd + 4) elements for the slices' partial results (made here if None;
+    nothing in it has to be cleared)."""
     _attention_checks("attention_decode", q, k_cache, v_cache, block_table, nh, nkv, hd, seq_slot, seq_start)
     B = seq_slot.shape[0]
     _need(q.shape[0] == B and seq_start.shape == (B,), "attention_decode: one query, slot and start for each sequence")
     out = torch.empty_like(q)
-    work = torch.empty((B * nh * n_slices * (hd + 4),), dtype=F32, device=q.device) if n_slices > 1 else None
+    work = _slices_workspace("attention_decode", work, B, nh, n_slices, hd, q.device)
     library.call(attention_lib(hd), "palm_attention_decode", _stream(), _p(q), _p(k_cache), _p(v_cache), _p(block_table),
                  block_table.shape[1], _p(seq_slot), _p(seq_start), B, nh, nkv, hd, float(scale), int(window or 0),
                  int(n_slices), _p(work), _p(out))
@@ -620,7 +635,8 @@ def decode_fused_serves(qkv: torch.Tensor, hd: int, out_dtype, rotary_dim: int, 
 
 def attention_decode_fused(qkv, k_cache, v_cache, block_table, seq_slot, seq_start, nh: int, nkv: int, hd: int, scale: float,
                            window: int | None, n_slices: int, *, q_norm_w=None, k_norm_w=None, eps: float = 0.0, cos=None,
-                           sin=None, rotary_dim: int = 0, pairing: int = 0, write_cache: bool = True) -> torch.Tensor:
+                           sin=None, rotary_dim: int = 0, pairing: int = 0, write_cache: bool = True,
+                           work: torch.Tensor | None = None) -> torch.Tensor:
     """A decode step's attention from the joined projection's rows: qk_norm_rope_store and attention_decode in one
     launch.  qkv is [B, (nh + 2 nkv) hd] bfloat16 or float32 planes [P, B, (nh + 2 nkv) hd]; sequence b's token is
     row b, at position seq_start[b]; cos, sin are [B, hd / 2] rows of those positions.  Returns [B, nh hd] bfloat16."""
@@ -643,7 +659,7 @@ def attention_decode_fused(qkv, k_cache, v_cache, block_table, seq_slot, seq_sta
         _need(tab is None or (tab.dtype == F32 and tab.shape == (B, hd // 2) and tab.is_contiguous() and rotary_dim == hd),
               f"{what}: a rotation table is float32 [{B}, {hd // 2}] over the whole head")
     out = torch.empty((B, nh * hd), dtype=BF16, device=qkv.device)
-    work = torch.empty((B * nh * n_slices * (hd + 4),), dtype=F32, device=qkv.device) if n_slices > 1 else None
+    work = _slices_workspace(what, work, B, nh, n_slices, hd, qkv.device)
     library.call(attention_lib(hd), "palm_attention_decode_fused", _stream(), _p(qkv), int(as_planes),
                  qkv.shape[0] if as_planes else 1, _p(q_norm_w), _p(k_norm_w), float(eps), _p(cos), _p(sin),
                  int(rotary_dim if cos is not None else 0), int(pairing), int(write_cache), _p(k_cache), _p(v_cache),

@@ -6,8 +6,9 @@
   bfloat16 x bfloat16, many rows (prompts)                      the BLAS library, as the reference's GPU path
                                                                 does for its products (engine/cuda_matmul.cu:245-260)
 
-A bias (none of Qwen3's projections has one) is added by a pass of its own after the product, which then comes
-whole (no planes, no norm folded in): correct for any part that needs it, at the price of a launch.
+A bias (none of Qwen3's projections has one) is added by a pass of its own to the product's 32-bit result, which
+then comes whole (no planes, no norm folded in) and is rounded once, after the add: correct for any part that needs
+it, at the price of two launches.
 """
 from __future__ import annotations
 
@@ -44,7 +45,14 @@ class Linear:
         if sink is not None:
             return self._into(x, sink)
         if self.bias is not None:
-            return ops.add_bias(self._product(x, out_dtype, False), self.bias)
+            rows = x.values if isinstance(x, Prenormed) else x
+            out_dtype = out_dtype or rows.dtype
+            y = ops.add_bias(self._product(x, torch.float32, False), self.bias)         # added where the sum still is 32-bit
+            if out_dtype == torch.float32:
+                return y
+            out = torch.empty(y.shape, dtype=out_dtype, device=y.device)
+            ops.convert_into(y, out)
+            return out
         return self._product(x, out_dtype, planes_ok)
 
     def _product(self, x, out_dtype, planes_ok):

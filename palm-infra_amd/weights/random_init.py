@@ -26,7 +26,9 @@ def random_tensors(spec, seed: int, dtype: str = "bfloat16") -> dict[str, torch.
         raise ValueError(f"dtype {dtype!r} is not one of {sorted(_STORE)}")
     out = {}
     for ref in spec.tensor_refs():
-        for name, shape in zip(ref.names, ref.shapes):
+        for name, shape in ref.stored_shapes():          # the tensors as the checkpoint stores them, each once
+            if name in out:
+                continue
             if ref.role == "integer":
                 out[name] = torch.zeros(shape, dtype=torch.int32)
                 continue

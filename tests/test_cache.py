@@ -43,7 +43,7 @@ def test_pages_follow_lengths_and_come_back():
     a, b = c.open(), c.open()
     c.reserve([(a, 70), (b, 1)])
     c.commit([(a, 70), (b, 1)])
-    g = c.kv_groups[0]
+    g = c.groups_of(KVNeed)[0]
     assert g.table.slot_pages[a] == [0, 1] and g.table.slot_pages[b] == [2]
     assert c.lengths[a] == 70 and c.lengths[b] == 1
     for _ in range(58):                              # 70 -> 128: still two pages
@@ -71,16 +71,16 @@ def test_a_step_that_does_not_fit_takes_nothing():
     c = _cache(max_tokens=64 * 4)
     a, b = c.open(), c.open()
     c.reserve([(a, 64)]); c.commit([(a, 64)])
-    free = c.kv_groups[0].table.pages.free_count
+    free = c.groups_of(KVNeed)[0].table.pages.free_count
     with pytest.raises(CacheFull, match="more pages"):
         c.reserve([(a, 65), (b, 100)])               # 2 + 2 pages wanted, 3 free
-    assert c.kv_groups[0].table.pages.free_count == free and c.lengths[a] == 64
+    assert c.groups_of(KVNeed)[0].table.pages.free_count == free and c.lengths[a] == 64
     with pytest.raises(CacheFull, match="longest sequence"):
         c.reserve([(b, 64 * 4 + 1)])
     with pytest.raises(CacheFull, match="more pages"):
         c.check_room([(a, 65), (b, 100)])            # the same question without taking anything
     c.check_room([(a, 64), (b, 100)])
-    assert c.kv_groups[0].table.pages.free_count == free and c.lengths[a] == 64 and c.lengths[b] == 0
+    assert c.groups_of(KVNeed)[0].table.pages.free_count == free and c.lengths[a] == 64 and c.lengths[b] == 0
     with pytest.raises(CacheMisuse, match="not open"):
         c.reserve([(3, 1)])
     c.check()
@@ -96,8 +96,8 @@ def test_longest_sequence_is_bounded_by_positions_and_by_the_cache():
 def test_groups_have_storage_of_their_own():
     needs = [[KVNeed(2, 16)], [KVNeed(1, 32, window=100)], [KVNeed(2, 16)], [KVNeed(1, 32, window=100), StateNeed("s", (3, 2))]]
     c = _cache(needs)
-    assert len(c.kv_groups) == 2 and len(c.state_groups) == 1
-    full, win = c.kv_groups
+    assert len(c.groups_of(KVNeed)) == 2 and len(c.groups_of(StateNeed)) == 1
+    full, win = c.groups_of(KVNeed)
     assert full.k.shape == (2, 13, 2, PAGE_TOKENS, 16) and win.k.shape == (2, 13, 1, PAGE_TOKENS, 32)
     assert full.v.shape == (2, 13, 2, 16, PAGE_TOKENS)                  # values are kept transposed
     assert full.k.data_ptr() != win.k.data_ptr() and full.table is not win.table
@@ -109,7 +109,7 @@ def test_groups_have_storage_of_their_own():
 
 def test_a_window_gives_pages_back_as_the_sequence_grows():
     c = _cache([[KVNeed(1, 16, window=70)], [KVNeed(1, 16)]])
-    win, full = c.kv_groups
+    win, full = c.groups_of(KVNeed)
     s = c.open()
     c.reserve([(s, 200)]); c.commit([(s, 200)])
     # the next query sits at 200 and reads keys 131..200: pages 0 and 1 (positions 0..127) are out of reach
@@ -126,17 +126,17 @@ def test_a_window_gives_pages_back_as_the_sequence_grows():
 def test_state_is_zero_for_a_new_sequence():
     c = _cache([[StateNeed("h", (4,))]])
     s = c.open()
-    c.state_groups[0].data[0, s] = 5.0
+    c.groups_of(StateNeed)[0].data[0, s] = 5.0
     c.close(s)
     assert c.open() == s
-    assert float(c.state_groups[0].data[0, s].abs().sum()) == 0.0
+    assert float(c.groups_of(StateNeed)[0].data[0, s].abs().sum()) == 0.0
 
 
 def test_an_entry_can_read_another_entrys_cache():
     c = _cache([[KVNeed(2, 16)], []], shares=[None, 0])
     a, b = c.layer_caches
     assert b.kv is a.kv and b.kv_entry == a.kv_entry and a.writes and not b.writes
-    assert c.kv_groups[0].k.shape[0] == 1
+    assert c.groups_of(KVNeed)[0].k.shape[0] == 1
 
 
 def test_random_traffic_keeps_the_books():
@@ -164,7 +164,7 @@ def test_random_traffic_keeps_the_books():
         c.check()
         for s, n in live.items():
             assert c.lengths[s] == n
-            for g in c.kv_groups:
+            for g in c.groups_of(KVNeed):
                 pages = g.table.slot_pages[s]
                 assert len(pages) >= pages_for(n)
                 first = 0 if g.need.window is None else max(0, n - g.need.window + 1) // PAGE_TOKENS
@@ -173,7 +173,7 @@ def test_random_traffic_keeps_the_books():
     for s in list(live):
         c.close(s)
     c.check()
-    assert all(g.table.pages.free_count == g.n_pages for g in c.kv_groups) and c.slots.free_count == 9
+    assert all(g.table.pages.free_count == g.n_pages for g in c.groups_of(KVNeed)) and c.slots.free_count == 9
 
 
 def test_rows_of_a_part_s_own_shape_grow_in_pages_beside_keys_and_values():
@@ -182,7 +182,7 @@ def test_rows_of_a_part_s_own_shape_grow_in_pages_beside_keys_and_values():
              [RowsNeed("codes", (2, 5), dtype="int32", window=70)]]
     c = _cache(needs)
     rows = [g for g in c.groups if isinstance(g, RowsGroup)]
-    assert len(rows) == 2 and len(c.kv_groups) == 1 and len(c.paged_groups) == 3 and len(c.state_groups) == 1
+    assert len(rows) == 2 and len(c.groups_of(KVNeed)) == 1 and len(c.paged_groups) == 3 and len(c.groups_of(StateNeed)) == 1
     latent, codes = rows
     assert latent.data.shape == (2, 13, PAGE_TOKENS, 24) and latent.data.dtype == torch.float32       # two entries share the group
     assert codes.data.shape == (1, 13, PAGE_TOKENS, 2, 5) and codes.data.dtype == torch.int32

@@ -7,6 +7,7 @@ import torch
 
 import plain_qwen3 as P
 import tiny
+from palm_infra_amd.cache import KVNeed, StateNeed
 
 pytestmark = pytest.mark.gpu
 
@@ -70,7 +71,7 @@ def test_batches_of_unequal_lengths_one_after_another(model_dirs, name, dtype):
     once), so later steps are smaller."""
     from palm_infra_amd.engine import StepEntry
     eng = engine_for(model_dirs, name, dtype)
-    held_before = eng.cache.kv_groups[0].table.pages.held_count
+    held_before = eng.cache.groups_of(KVNeed)[0].table.pages.held_count
     for round_no, (seed, tails) in enumerate([(2, [3, 0, 9, 1, 20, 5]), (3, [1, 12, 0, 2, 7, 30])]):
         reqs = tiny.prompts(name, LENGTHS[name] if round_no == 0 else LENGTHS[name][::-1], seed=seed)
         tails = [min(t, len(r) - 1) for t, r in zip(tails, reqs)]
@@ -99,7 +100,7 @@ def test_batches_of_unequal_lengths_one_after_another(model_dirs, name, dtype):
             tiny.assert_logits_close(torch.cat(got[i]), reference(model_dirs, name, dtype, r), dtype,
                                      f"{name} batch {round_no} request {i} ({len(r)} tokens, {tails[i]} one by one)")
         eng.cache.check()
-        assert eng.cache.kv_groups[0].table.pages.held_count == held_before
+        assert eng.cache.groups_of(KVNeed)[0].table.pages.held_count == held_before
 
 
 @pytest.mark.parametrize("name,dtype", [("C", "float32"), ("C", "bfloat16"), ("B", "float32"), ("D", "bfloat16")])

@@ -408,8 +408,17 @@ def _fill_cache(kc, vc, table, slot, k, v):
         vc[page, :, :, p % 64] = v[p].to(vc.dtype)
 
 
-def _attention_case(ops, fn, dtype, nh, nkv, hd, lens_new, window, seed=0, scale=None):
-    """Sequences (total length, new tokens): queries are the last `new` positions."""
+def _poison(t):
+    """What a request whose activations overflowed may leave in its pages: NaN, +inf and -inf in turn."""
+    flat = t.view(-1)
+    flat[0::3], flat[1::3], flat[2::3] = float("nan"), float("inf"), float("-inf")
+    return t
+
+
+def _attention_case(ops, fn, dtype, nh, nkv, hd, lens_new, window, seed=0, scale=None, poison=False):
+    """Sequences (total length, new tokens): queries are the last `new` positions.  Every place of the cache that
+    belongs to no sequence (other pages, the last page's tail) holds stale values: random numbers, or with
+    ``poison`` NaN and infinities."""
     scale = scale if scale is not None else hd ** -0.5
     B = len(lens_new)
     n_pages = sum((L + 63) // 64 for L, _ in lens_new) + 2
@@ -419,6 +428,8 @@ def _attention_case(ops, fn, dtype, nh, nkv, hd, lens_new, window, seed=0, scale
     table = torch.full((B + 4, max_pages), n_pages - 1, dtype=torch.int32)
     kc = rand(n_pages, nkv, 64, hd, seed=seed + 50, dtype=dtype).to(DEV)      # stale values everywhere
     vc = rand(n_pages, nkv, hd, 64, seed=seed + 51, dtype=dtype).to(DEV)
+    if poison:
+        _poison(kc), _poison(vc)
     qs, refs, o = [], [], 0
     for b, (L, new) in enumerate(lens_new):
         npg = (L + 63) // 64
@@ -447,6 +458,15 @@ def test_attention_exact_prompts_decode_and_mixed_lengths(ops, dtype, nh, nkv, h
     for lens in cases:
         got, ref = _attention_case(ops, ops.attention_exact, dtype, nh, nkv, hd, lens, None, seed=len(lens))
         assert torch.allclose(got, ref, atol=1e-5 if dtype == F32 else 2e-2), lens
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_attention_exact_takes_nothing_from_what_lies_beyond_a_sequence(ops, dtype):
+    """Pages are handed out uncleared: NaN and infinities beyond a sequence's length must not reach its output."""
+    got, ref = _attention_case(ops, ops.attention_exact, dtype, 4, 2, 32, [(64, 64), (65, 1), (130, 70), (7, 7)], None, seed=5, poison=True)
+    assert torch.isfinite(got).all() and torch.allclose(got, ref, atol=1e-5 if dtype == F32 else 2e-2)
+    got, ref = _attention_case(ops, ops.attention_exact, dtype, 4, 2, 32, [(200, 1), (150, 150), (3, 1)], 70, seed=6, poison=True)
+    assert torch.isfinite(got).all() and torch.allclose(got, ref, atol=1e-5 if dtype == F32 else 2e-2)
 
 
 def test_attention_exact_over_thousands_of_keys(ops):

@@ -290,7 +290,7 @@ def test_linear_tile_refuses_what_it_does_not_serve(ops):
 
 # ---- attention on the matrix cores ------------------------------------------------------------------
 
-from test_kernels import _attention_case, _fill_cache, _spike_case  # noqa: E402  (the cases and the cache filling are shared)
+from test_kernels import _attention_case, _fill_cache, _poison, _spike_case  # noqa: E402  (the cases and the cache filling are shared)
 
 
 def decode_fn(ops, n_slices):
@@ -360,6 +360,39 @@ def test_attention_mfma_finds_a_far_key_and_respects_the_window_edge(ops):
         assert not torch.allclose(got, v[L - w - 1, 0].float().expand(2, -1), atol=0.2)
 
 
+@pytest.mark.parametrize("nh,nkv,hd", [(32, 8, 128), (6, 3, 64), (6, 1, 80), (3, 3, 256), (4, 2, 192), (40, 2, 32)])
+def test_attention_mfma_takes_nothing_from_what_lies_beyond_a_sequence(ops, nh, nkv, hd):
+    """Pages are handed out uncleared, and a key beyond a sequence's length has weight zero: but zero times the NaN
+    or the infinity that an earlier request may have left as its value is NaN.  Every place of the cache that
+    belongs to no sequence is filled with NaN and infinities; the outputs must be finite and right.  (Every head
+    size's way of bringing a page into LDS, prompts whose last page is partly filled and exactly filled, a
+    continuation, single queries in one and in several slices, with and without a window.)"""
+    prompts = [[(20, 20)], [(64, 64)], [(1, 1)], [(300, 44)], [(64, 64), (65, 1), (130, 70), (7, 7), (200, 17), (129, 129)]]
+    for window in (None, 70):
+        for lens in prompts:
+            got, ref = _attention_case(ops, ops.attention_prefill, BF16, nh, nkv, hd, lens, window, seed=len(lens) + hd, poison=True)
+            assert torch.isfinite(got).all(), (lens, window)
+            assert torch.allclose(got, ref, atol=2e-2), (lens, window, float((got - ref).abs().max()))
+        for n_slices in (1, 3, 8):
+            for lens in ([(300, 1)], [(1, 1)], [(64, 1), (65, 1), (700, 1), (7, 1), (128, 1)]):
+                got, ref = _attention_case(ops, decode_fn(ops, n_slices), BF16, nh, nkv, hd, lens, window, seed=len(lens) + hd, poison=True)
+                assert torch.isfinite(got).all(), (lens, window, n_slices)
+                assert torch.allclose(got, ref, atol=2e-2), (lens, window, n_slices, float((got - ref).abs().max()))
+
+
+def test_attention_decode_reads_no_record_of_a_slice_without_pages(ops):
+    """A step is cut into slices for its longest sequence; a shorter sequence's last slices hold no page, write no
+    record, and the merge must read none of theirs: the workspace is handed in full of NaN."""
+    nh, nkv, hd = 8, 2, 64
+    for n_slices in (4, 9, 40):
+        def fn(q, kc, vc, table, slots, starts, news, cu, max_new, nh_, nkv_, hd_, scale, window):
+            work = torch.full((q.shape[0] * nh * n_slices * (hd + 4),), float("nan"), device=DEV)
+            return ops.attention_decode(q, kc, vc, table, slots, starts, nh, nkv, hd, scale, window, n_slices, work=work)
+        for window in (None, 100):
+            got, ref = _attention_case(ops, fn, BF16, nh, nkv, hd, [(2000, 1), (3, 1), (65, 1), (700, 1)], window, seed=n_slices)
+            assert torch.isfinite(got).all() and torch.allclose(got, ref, atol=2e-2), (n_slices, window)
+
+
 def test_attention_mfma_agrees_with_the_exact_kernel_on_the_same_cache(ops):
     """Both read the same cache (keys as rows, values transposed): the layouts cannot drift apart."""
     got_m, ref = _attention_case(ops, ops.attention_prefill, BF16, 8, 2, 64, [(190, 190), (64, 5)], None, seed=3)
@@ -380,7 +413,7 @@ def test_attention_mfma_refuses_what_it_was_not_built_for(ops):
 
 # ---- decode attention that starts from the joined projection's rows -----------------------------------
 
-def _fused_case(ops, nh, nkv, hd, lengths, n_slices, planes, window=None, norm=True, rotate=True, seed=0):
+def _fused_case(ops, nh, nkv, hd, lengths, n_slices, planes, window=None, norm=True, rotate=True, seed=0, poison=False):
     """Sequences whose last token is new: its q/k/v row goes (a) through qk_norm_rope_store and attention_decode and
     (b) through attention_decode_fused, each on its own copy of a cache that holds the earlier tokens and stale
     values elsewhere.  Returns both outputs and both pairs of caches."""
@@ -392,6 +425,8 @@ def _fused_case(ops, nh, nkv, hd, lengths, n_slices, planes, window=None, norm=T
     table = torch.full((B + 3, max_pages), n_pages - 1, dtype=torch.int32)
     kc = rand(n_pages, nkv, 64, hd, seed=seed + 50).to(DEV)
     vc = rand(n_pages, nkv, hd, 64, seed=seed + 51).to(DEV)
+    if poison:
+        _poison(kc), _poison(vc)
     o = 0
     for b, L in enumerate(lengths):
         npg = (L + 63) // 64
@@ -446,6 +481,18 @@ def test_attention_decode_fused_is_the_two_kernels_in_one(ops, nh, nkv, hd, n_sl
         assert _one_ulp(one, two), (planes, lengths, float((one - two).abs().max()))
         _same_caches(ca, cb)
         assert not torch.equal(cb[0], before[0]) and not torch.equal(cb[1], before[1])      # it did write
+
+
+def test_attention_decode_fused_takes_nothing_from_what_lies_beyond_a_sequence(ops):
+    """As for the other attention kernels: NaN and infinities wherever the cache belongs to no sequence, also at the
+    new token's own place, which the kernel may read before or after it writes it."""
+    for nh, nkv, hd in ((32, 8, 128), (6, 3, 64), (3, 3, 256)):
+        for n_slices in (1, 3, 8):
+            for window in (None, 70):
+                one, two, *_ = _fused_case(ops, nh, nkv, hd, [64, 65, 700, 7, 128, 129, 1, 300], n_slices, 2, window=window,
+                                           seed=hd, poison=True)
+                assert torch.isfinite(one).all() and torch.isfinite(two).all(), (hd, n_slices, window)
+                assert _one_ulp(one, two), (hd, n_slices, window, float((one - two).abs().max()))
 
 
 def test_attention_decode_fused_with_a_window_without_norm_and_without_rotation(ops):

@@ -19,8 +19,8 @@ NAME = "ToyMixedForCausalLM"
 
 
 def register():
-    from palm_infra_amd.config import (LayerCall, ModelSpec, PartSpec, joined, register_architecture, registered_architectures,
-                                       tensor)
+    from palm_infra_amd.config import (LayerCall, ModelSpec, PartSpec, Stored, joined, register_architecture,
+                                       registered_architectures, tensor)
     toy.register_toy_mixer()
     if NAME in registered_architectures():
         return
@@ -61,9 +61,14 @@ def register():
                     nh, nkv, hd = b["heads"], b["kv_heads"], b["head_size"]
                     mixer = PartSpec("mixer", "attention",
                                      {"hidden_size": H, "num_heads": nh, "num_kv_heads": nkv, "head_dim": hd, "scale": hd ** -0.5, "window": None},
-                                     {"qkv": joined((p + "attn.wq", p + "attn.wk", p + "attn.wv"), ((nh * hd, H), (nkv * hd, H), (nkv * hd, H)),
-                                                    init=("normal", 0.0, 0.1)),
-                                      "out": tensor(p + "attn.wo", (H, nh * hd), init=("normal", 0.0, 0.1))},
+                                     # the checkpoint keeps v, k and q fused in one tensor, in that order, and the output
+                                     # matrix as [in, out]: the description says so, the loader needs no change
+                                     {"qkv": joined((p + "attn.wvkq",) * 3, ((nh * hd, H), (nkv * hd, H), (nkv * hd, H)), init=("normal", 0.0, 0.1),
+                                                    stored=(Stored(((nh + 2 * nkv) * hd, H), rows=(2 * nkv * hd, (nh + 2 * nkv) * hd)),
+                                                            Stored(((nh + 2 * nkv) * hd, H), rows=(nkv * hd, 2 * nkv * hd)),
+                                                            Stored(((nh + 2 * nkv) * hd, H), rows=(0, nkv * hd)))),
+                                      "out": tensor(p + "attn.wo_t", (H, nh * hd), init=("normal", 0.0, 0.1),
+                                                    stored=Stored((nh * hd, H), transposed=True))},
                                      {"position": PartSpec("position", "rotary", {"rotary_dim": b["rotary"], "theta": self.theta,
                                                                                   "pairing": "interleaved"})})      # no q/k norm here
                 else:
@@ -100,12 +105,13 @@ def plain_logits(raw, w, ids):
         h = P.rms_norm(x, w[p + "n1.weight"], eps)
         if b["mixer"] == "attention":
             nh, nkv, hd, rot = b["heads"], b["kv_heads"], b["head_size"], b["rotary"]
-            q = P.linear(h, w[p + "attn.wq"]).reshape(n, nh, hd)
-            k = P.linear(h, w[p + "attn.wk"]).reshape(n, nkv, hd)
-            v = P.linear(h, w[p + "attn.wv"]).reshape(n, nkv, hd)
+            vkq = w[p + "attn.wvkq"]                     # rows: v heads, then k heads, then q heads
+            v = P.linear(h, vkq[:nkv * hd]).reshape(n, nkv, hd)
+            k = P.linear(h, vkq[nkv * hd:2 * nkv * hd]).reshape(n, nkv, hd)
+            q = P.linear(h, vkq[2 * nkv * hd:]).reshape(n, nh, hd)
             cos, sin = P.rope_table(list(range(n)), rot, raw["theta"])
             q, k = toy._rope_interleaved(q, cos, sin, rot), toy._rope_interleaved(k, cos, sin, rot)
-            x = x + P.linear(P.causal_attention(q, k, v, hd ** -0.5).reshape(n, nh * hd), w[p + "attn.wo"])
+            x = x + P.causal_attention(q, k, v, hd ** -0.5).reshape(n, nh * hd) @ w[p + "attn.wo_t"].double()     # stored [in, out]
         else:
             u = h @ w[p + "mix.w_in"].double().T
             s, mixed = torch.zeros(b["state"], dtype=torch.float64), []
@@ -133,7 +139,8 @@ def test_an_architecture_registered_from_outside_loads_steps_and_generates(tmp_p
     assert type(config_from_dir(folder)).__name__ == "ToyMixedConfig"
     engine = palm_infra_amd.load(folder, dtype=dtype, max_tokens=64 * 8)
     # three runs of two layers: two key/value stores for the layer that runs twice, one state for the toy mixer
-    assert [g.n_entries for g in engine.cache.kv_groups] == [2] and len(engine.cache.state_groups) == 1
+    kinds = sorted((type(g.need).__name__, g.n_entries) for g in engine.cache.groups)
+    assert kinds == [("KVNeed", 2), ("StateNeed", 1)]
     assert not engine.model.capturable                                          # the toy mixer plans on the host
     raw, w = P.read_model(folder)
     reqs = [torch.randint(0, raw["vocab"], (n,), generator=torch.Generator().manual_seed(60 + n)).tolist() for n in (70, 9, 33)]

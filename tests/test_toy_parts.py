@@ -8,6 +8,7 @@ import torch
 
 import plain_qwen3 as P
 import tiny
+from palm_infra_amd.cache import KVNeed, StateNeed
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -106,7 +107,7 @@ def test_a_mixer_with_state_of_its_own(model_dirs, dtype):
     weights = ExtraWeights(load_weights(base, files, tdt, DEV), {("toy.w_in",): w_in.to(DEV), ("toy.w_out",): w_out.to(DEV)})
     eng = Engine(config, spec, weights, tdt, max_tokens=64 * 8)
     # the cache has one key/value group (layer 0) and one state group (layer 1)
-    assert [g_.n_entries for g_ in eng.cache.kv_groups] == [1] and len(eng.cache.state_groups) == 1
+    assert [g_.n_entries for g_ in eng.cache.groups_of(KVNeed)] == [1] and len(eng.cache.groups_of(StateNeed)) == 1
     assert eng.cache.layer_caches[1].kv is None and "decay_state" in eng.cache.layer_caches[1].states
 
     cfg, w = P.read_model(d)
@@ -146,7 +147,7 @@ def test_run_order_names_a_layer_twice_and_shares_a_cache(model_dirs, dtype):
     base = config.spec(files.names())
     spec = dataclasses.replace(base, order=(LayerCall(0), LayerCall(1), LayerCall(0), LayerCall(1, cache_of=1)))
     eng = Engine(config, spec, load_weights(base, files, tdt, DEV), tdt, max_tokens=64 * 4)
-    assert eng.cache.kv_groups[0].n_entries == 3                   # three stores for four runs
+    assert eng.cache.groups_of(KVNeed)[0].n_entries == 3                   # three stores for four runs
 
     cfg, w = P.read_model(d)
     S = P.sizes(cfg)
@@ -198,7 +199,7 @@ def test_layers_with_and_without_a_window_in_one_model(model_dirs, dtype):
     parts["mixer"] = dataclasses.replace(mixer, params=dict(mixer.params, window=37))
     spec = dataclasses.replace(base, layers=(base.layers[0], dataclasses.replace(layer, parts=parts)))
     eng = Engine(config, spec, load_weights(base, files, tdt, DEV), tdt, max_tokens=64 * 12)
-    assert sorted(str(g.need.window) for g in eng.cache.kv_groups) == ["37", "None"]
+    assert sorted(str(g.need.window) for g in eng.cache.groups_of(KVNeed)) == ["37", "None"]
     eng.step_tokens_per_seq = 50                                     # force long prompts through in pieces
 
     cfg, w = P.read_model(d)
@@ -221,7 +222,7 @@ def test_layers_with_and_without_a_window_in_one_model(model_dirs, dtype):
         out = eng.step([StepEntry(slots[i], [reqs[i][fed[i]]], [0]) for i in live])
         for r_, i in enumerate(live):
             got[i].append(out[r_:r_ + 1]); fed[i] += 1
-    win = [g for g in eng.cache.kv_groups if g.need.window][0]
+    win = [g for g in eng.cache.groups_of(KVNeed) if g.need.window][0]
     assert win.table.slot_pages[slots[0]][:2] == [-1, -1]            # pages below the window went back
     for i in range(2):
         tiny.assert_logits_close(torch.cat(got[i]), plain(reqs[i]), dtype, f"window model request {i}")
@@ -460,7 +461,7 @@ def test_a_mixer_that_keeps_one_latent_row_for_each_position(model_dirs, dtype):
     eng = Engine(config, spec, weights, tdt, max_tokens=64 * 6)
     rows_groups = [g_ for g_ in eng.cache.groups if isinstance(g_, RowsGroup)]
     assert len(rows_groups) == 1 and rows_groups[0].data.shape == (1, 7, 64, width) and rows_groups[0].data.dtype == torch.float32
-    assert len(eng.cache.kv_groups) == 1 and len(eng.cache.paged_groups) == 2
+    assert len(eng.cache.groups_of(KVNeed)) == 1 and len(eng.cache.paged_groups) == 2
     assert not eng.model.capturable
 
     cfg, w = P.read_model(d)

@@ -12,9 +12,9 @@ from palm_infra_amd.weights import (ModelFiles, SafetensorsError, SafetensorsFil
                                     random_tensors, write_random_model, write_safetensors)
 
 
-def host_copy(stored, part):
+def host_copy(stored, part, transposed=False):
     """Stands in for the device's conversion kernel where only the binding is tested (no GPU here)."""
-    part.copy_(stored)
+    part.copy_(stored.t() if transposed else stored)
 
 
 def test_round_trip_is_bit_exact(tmp_path):
@@ -81,6 +81,68 @@ def test_one_error_lists_missing_unexpected_and_misshapen(tmp_path):
     text = str(err)
     for word in ("missing", "unexpected", "wrong shapes", "k_proj", "inv_freq", "expected [64, 128], file has [64, 100]"):
         assert word in text, word
+
+
+def test_tensors_the_model_does_not_name_are_a_warning_list_when_asked(tmp_path):
+    """The reference's converter passes over names it does not know (models/qwen3.py:105-106).  Here they are an
+    error by default; with strict=False they come back as a list and the model loads; what is missing or
+    misshapen stays an error either way."""
+    tensors = tiny.sharpened_tensors("A", "float32")
+    tensors["rotary.inv_freq"] = torch.zeros(8)
+    tensors["model.layers.7.mlp.up_proj.weight"] = torch.zeros(2, 2)
+    (tmp_path / "config.json").write_text(json.dumps(tiny.CONFIGS["A"]))
+    write_safetensors(tmp_path / "model.safetensors", tensors)
+    files = ModelFiles(tmp_path)
+    spec = config_from_dir(tmp_path).spec(files.names())
+    with pytest.raises(WeightError) as e:
+        load_weights(spec, files, torch.float32, "cpu", place=host_copy)
+    assert sorted(e.value.unexpected) == ["model.layers.7.mlp.up_proj.weight", "rotary.inv_freq"] and not e.value.missing
+    told = []
+    w = load_weights(spec, files, torch.float32, "cpu", place=host_copy, strict=False, warn=told.extend)
+    assert sorted(told) == ["model.layers.7.mlp.up_proj.weight", "rotary.inv_freq"]
+    assert torch.equal(w.get(spec.final_norm.tensors["weight"]), tensors["model.norm.weight"])
+    del tensors["model.norm.weight"]
+    write_safetensors(tmp_path / "model.safetensors", tensors)
+    files = ModelFiles(tmp_path)
+    with pytest.raises(WeightError) as e:
+        load_weights(spec, files, torch.float32, "cpu", place=host_copy, strict=False, warn=told.extend)
+    assert e.value.missing == ["model.norm.weight"]
+
+
+def test_a_parameter_may_be_rows_of_a_stored_tensor_or_its_transpose(tmp_path):
+    """A checkpoint that stores q, k and v fused in one tensor (here in the order v, k, q) and a matrix as [in, out]
+    is a matter of the model's description, not of the loader: pieces say which rows of which stored tensor they
+    are, and whether what is stored is their transpose."""
+    from palm_infra_amd.config import Stored, joined, tensor
+    from palm_infra_amd.config.spec import LayerCall, ModelSpec, PartSpec
+    g = torch.Generator().manual_seed(3)
+    fused, w_io = torch.randn(4 + 4 + 8, 6, generator=g), torch.randn(6, 10, generator=g)
+    qkv = joined(("att.fused",) * 3, ((8, 6), (4, 6), (4, 6)),
+                 stored=(Stored((16, 6), rows=(8, 16)), Stored((16, 6), rows=(4, 8)), Stored((16, 6), rows=(0, 4))))
+    out = tensor("att.out_io", (10, 6), stored=Stored((6, 10), transposed=True))
+    assert qkv.shape == (16, 6) and out.shape == (10, 6) and qkv.key != joined(("att.fused",) * 3, ((8, 6), (4, 6), (4, 6))).key
+    with pytest.raises(ValueError, match="expects"):
+        tensor("x", (5, 6), stored=Stored((6, 10), transposed=True))
+    with pytest.raises(ValueError, match="rows"):
+        tensor("x", (5, 6), stored=Stored((4, 6), rows=(0, 5)))
+    part = PartSpec("mixer", "anything", {}, {"qkv": qkv, "out": out})
+    norm = PartSpec("norm", "rms", {}, {"weight": tensor("n", (6,), "vector")})
+    spec = ModelSpec("T", 3, 6, None, PartSpec("embedding", "token_table", {}, {"table": tensor("emb", (3, 6), "table")}),
+                     (part,), (LayerCall(0),), norm, PartSpec("head", "linear", {}, {"weight": tensor("emb", (3, 6), "table")}))
+    assert spec.expected_tensors()["att.fused"] == ((16, 6), "matrix") and spec.expected_tensors()["att.out_io"] == ((6, 10), "matrix")
+    write_safetensors(tmp_path / "model.safetensors", {"att.fused": fused, "att.out_io": w_io, "n": torch.ones(6), "emb": torch.zeros(3, 6)})
+    w = load_weights(spec, ModelFiles(tmp_path), torch.float32, "cpu", place=host_copy)
+    assert torch.equal(w.get(qkv), torch.cat([fused[8:16], fused[4:8], fused[0:4]]))
+    assert torch.equal(w.get(out), w_io.t())
+    # the random-weights mode writes the tensors as the checkpoint stores them, each once
+    from palm_infra_amd.weights import random_tensors
+    made = random_tensors(spec, 1, "float32")
+    assert made["att.fused"].shape == (16, 6) and made["att.out_io"].shape == (6, 10) and set(made) == {"att.fused", "att.out_io", "n", "emb"}
+    # a wrong stored shape is named like any other
+    write_safetensors(tmp_path / "model.safetensors", {"att.fused": fused[:12], "att.out_io": w_io, "n": torch.ones(6), "emb": torch.zeros(3, 6)})
+    with pytest.raises(WeightError) as e:
+        load_weights(spec, ModelFiles(tmp_path), torch.float32, "cpu", place=host_copy)
+    assert [n for n, _, _ in e.value.wrong_shape] == ["att.fused"]
 
 
 def test_a_stored_head_is_used_whatever_the_config_says(tmp_path):
