@@ -42,7 +42,10 @@ PALM_API int palm_attention_decode_static(hipStream_t stream, const void* q, con
                                           int window, int n_slices, void* out);
 PALM_API long long palm_attention_decode_static_limit();
 
+// q_prescaled: the queries come multiplied by scale * log2(e) already and `scale` is not applied again; only where
+// palm_attention_prefill_takes_prescaled() says so (the head sizes whose kernel gains from it).
 PALM_API int palm_attention_prefill(hipStream_t stream, const void* q, const void* k_cache, const void* v_cache,
                                     const int* block_table, int max_pages, const int* seq_slot, const int* seq_start,
                                     const int* seq_new, const int* cu_new, int n_seqs, int max_new, int nh, int nkv,
-                                    int hd, float scale, int window, void* out);
+                                    int hd, float scale, int window, int q_prescaled, void* out);
+PALM_API int palm_attention_prefill_takes_prescaled();

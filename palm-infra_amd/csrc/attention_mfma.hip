@@ -1218,10 +1218,283 @@ __global__ __launch_bounds__(PF_THREADS) PF_WAVES_PER_SIMD void attention_prefil
     }
 }
 
+// ---- prefill for the head sizes whose pages go straight into LDS (64, 128) --------------------------
+// The same block of four waves, eight units and pages staged once in LDS, arranged so that the page loop is one
+// stretch of arithmetic without a branch around any matrix instruction:
+//  * a wave's two units lie next to each other (the same head's neighbouring 16 queries where a kv head has four
+//    query heads), so both see almost the same pages, and there is no unit to switch on and off: a page that a unit
+//    does not see at all is simply a page whose every key is masked for it;
+//  * a block has one tile of queries, and a late tile has many more pages to walk than an early one.  Where the
+//    launch has more blocks than the chip holds at once, the long ones simply go first.  Where all its blocks run at
+//    once (a prompt of a few thousand tokens), two share a compute unit, and the numbering makes blocks k and k + 256,
+//    which the dispatcher is expected to place together, a tile from the back and its partner from the front, so
+//    that every unit gets about the same work;
+//  * the scores come out of the matrix cores already taken against the column's reference (the accumulator starts at
+//    minus the reference instead of zero; with queries that come multiplied by scale * log2(e), q_prescaled, no
+//    multiplication is left either), so a weight is one exp2 and one rounding;
+//  * the reference follows the running maximum only when a column's scores have risen more than 2^PF_LAZY_LOG2 above
+//    it.  Whether any column of the wave has to move is one vote over the lanes' own sixteen scores; the exchange
+//    between the four lanes of a column, the shift and the rescaling of the outputs stand behind that vote, off the
+//    usual path;
+//  * STAGES pages of K and V^T lie in LDS, STAGES - 1 of them on their way while one is used: two where many blocks
+//    share a compute unit, four where a short prompt leaves a unit one block, whose loads then need a longer lead.
+//    The barrier between pages waits for LDS and for the one page that is needed next, not for the younger loads.
+template <int N> __device__ __forceinline__ void wait_for_all_but_the_youngest_loads() {
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));          // s_waitcnt vmcnt(N)
+}
+__device__ __forceinline__ void page_barrier() {     // LDS reads done, then the block's barrier; loads stay in flight
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+struct PairedUnit {           // one (head, 16 query positions): the wave's share of it
+    bool live, valid;         // the wave has such a unit; this lane's column is a real query
+    int pos, first;           // the column's position and the first key it sees
+    size_t row;               // the column's row in q and out
+    int head;
+    float m;                  // the reference the column's weights are taken against (-inf before its first key)
+    bf16x8 qv[KSTEPS];
+    f32x4 o[DTILES];
+    f32x4 weights;            // the sum of the column's weights, four times
+};
+
+// masked (the same in every lane): some column of the wave does not see every key of the page
+template <bool PRESCALED>
+__device__ __forceinline__ void paired_page(const bf16_t* k_lds, const bf16_t* v_lds, PairedUnit (&u)[PF_UNITS], int page_first_key,
+                                            float scale_log2, int r, int g, bool masked) {
+    f32x4 s[PF_UNITS][4];
+    float sub[PF_UNITS];
+#pragma unroll
+    for (int x = 0; x < PF_UNITS; ++x) sub[x] = u[x].m == -INFINITY ? 0.f : u[x].m;
+    bf16x8 kf[2][KSTEPS];
+    read_key_fragments(k_lds, 0, r, g, kf[0]);
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        if (t < 3) read_key_fragments(k_lds, t + 1, r, g, kf[(t + 1) & 1]);
+#pragma unroll
+        for (int x = 0; x < PF_UNITS; ++x) {
+            const float from = PRESCALED ? -sub[x] : 0.f;
+            f32x4 acc = f32x4{from, from, from, from};
+#pragma unroll
+            for (int j = 0; j < KSTEPS; ++j) acc = mfma_16x16x32(kf[t & 1][j], u[x].qv[j], acc);
+            s[x][t] = acc;
+        }
+        __builtin_amdgcn_sched_barrier(0);          // or every tile's fragments are asked for at once and the registers run out
+    }
+    // the first values are asked for now and arrive while the weights are made
+    bf16x8 vf[2][2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) vf[0][h] = *reinterpret_cast<const bf16x8*>(v_lds + r * V_STRIDE + ((h * 4 + g) ^ v_swizzle(r)) * 8);
+
+    bool vote = masked;
+    float mx[PF_UNITS];
+#pragma unroll
+    for (int x = 0; x < PF_UNITS; ++x) {
+        if (!PRESCALED) {
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) s[x][t][i] = fmaf(s[x][t][i], scale_log2, -sub[x]);
+        }
+        if (masked) {
+            const int lo = u[x].first - page_first_key, hi = u[x].pos - page_first_key;
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int key = tile_key(t, 4 * g + i);
+                    s[x][t][i] = (key >= lo && key <= hi) ? s[x][t][i] : -INFINITY;
+                }
+        }
+        float top = s[x][0][0];
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) top = fmaxf(top, s[x][t][i]);
+        mx[x] = top;
+        vote = vote || top > PF_LAZY_LOG2 || u[x].m == -INFINITY;
+    }
+    if (__any(vote)) {
+#pragma unroll
+        for (int x = 0; x < PF_UNITS; ++x) {
+            float top = mx[x];                                          // of the column: its four lanes agree
+            top = fmaxf(top, __shfl_xor(top, 16, WAVE));
+            top = fmaxf(top, __shfl_xor(top, 32, WAVE));
+            const bool fresh = u[x].m == -INFINITY;                     // no key yet: outputs and sums are still zero
+            const bool jump = top > PF_LAZY_LOG2 || (fresh && top > -INFINITY);
+            const float shift = jump ? top : 0.f;
+            const float alpha = jump && !fresh ? exp2_weight(-top) : 1.0f;
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) s[x][t][i] -= shift;
+            if (jump) u[x].m = sub[x] + top;
+            if (__any(alpha != 1.0f)) {
+#pragma unroll
+                for (int dt = 0; dt < DTILES; ++dt) u[x].o[dt] = u[x].o[dt] * alpha;
+                u[x].weights = u[x].weights * alpha;
+            }
+        }
+    }
+    bf16x8 pv[PF_UNITS][2];
+#pragma unroll
+    for (int x = 0; x < PF_UNITS; ++x)
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) pv[x][h][e] = (__bf16)exp2_weight(s[x][2 * h + e / 4][e % 4]);
+
+    // the sum of a column's weights comes from the matrix cores too: a row of ones in place of a row of V^T
+    bf16x8 ones;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ones[e] = (__bf16)1.0f;
+#pragma unroll
+    for (int x = 0; x < PF_UNITS; ++x)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) u[x].weights = mfma_16x16x32(ones, pv[x][h], u[x].weights);
+#pragma unroll
+    for (int dt = 0; dt < DTILES; ++dt) {
+        if (dt + 1 < DTILES) {
+            const bf16_t* vrow = v_lds + ((dt + 1) * 16 + r) * V_STRIDE;
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+                vf[(dt + 1) & 1][h] = *reinterpret_cast<const bf16x8*>(vrow + ((h * 4 + g) ^ v_swizzle((dt + 1) * 16 + r)) * 8);
+        }
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int x = 0; x < PF_UNITS; ++x) u[x].o[dt] = mfma_16x16x32(vf[dt & 1][h], pv[x][h], u[x].o[dt]);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+}
+
+template <int STAGES, bool PRESCALED>
+__global__ __launch_bounds__(PF_THREADS) PF_WAVES_PER_SIMD void attention_prefill_paired_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+    const int* __restrict__ block_table, int max_pages, const int* __restrict__ seq_slot,
+    const int* __restrict__ seq_start, const int* __restrict__ seq_new, const int* __restrict__ cu_new, int nh,
+    int nkv, float scale_log2, int window, int qb, int hg, int partners_follow, bf16_t* __restrict__ out) {
+    if constexpr (PF_DMA) {
+        constexpr int K_TILE = PAGE_TOKENS * K_STRIDE, V_TILE = HD * V_STRIDE;
+        constexpr int PAGE_LOADS = 2 * PF_LOADS;                    // a wave's instructions for one page of K and V^T
+        __shared__ __attribute__((aligned(16))) bf16_t k_lds[STAGES * K_TILE];
+        __shared__ __attribute__((aligned(16))) bf16_t v_lds[STAGES * V_TILE];
+
+        const int b = blockIdx.z;
+        const int G = nh / nkv, n_hg = (G + hg - 1) / hg;
+        const int kvh = blockIdx.x / n_hg, hgi = blockIdx.x % n_hg;   // the kv head runs fastest over the blocks, see the launch
+        const int n_new = seq_new[b];
+        const int subs = qb / 16, n_q = (n_new + qb - 1) / qb;        // tiles of qb queries in this sequence
+        if ((int)blockIdx.y >= n_q) return;
+        // first the tiles from the back (the long ones), the last first; then, where the launch asks for it, their
+        // partners from the front in the same order, else the rest from the back too
+        const int half = (n_q + 1) / 2, y = blockIdx.y;
+        const int tile = y < half || !partners_follow ? n_q - 1 - y : y - half;
+        const int lane = threadIdx.x % WAVE, r = lane % 16, g = lane / 16;
+        const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
+        const int start = seq_start[b];
+        const int seq_tail = start + n_new - 1;                       // the sequence's last key
+        const int heads_here = min(hg, G - hgi * hg);
+        const int n_units = heads_here * subs;
+        const int* pages = block_table + (size_t)seq_slot[b] * max_pages;
+        const PageSources sources = page_sources();
+
+        {
+            const int tile_first = tile * qb;                         // the tile's first query, within the step
+            PairedUnit u[PF_UNITS];
+#pragma unroll
+            for (int x = 0; x < PF_UNITS; ++x) {
+                const int unit = wave + x * PF_WAVES;
+                const int sub = unit / heads_here;                    // the unit's 16 queries within the tile
+                const int q_first = tile_first + sub * 16;
+                u[x].live = unit < n_units && q_first < n_new;
+                const int qi = q_first + r;
+                u[x].head = kvh * G + hgi * hg + (unit < n_units ? unit % heads_here : 0);
+                u[x].valid = u[x].live && qi < n_new;
+                const int qc = min(qi, n_new - 1);
+                u[x].pos = start + qc;
+                u[x].first = window > 0 ? max(0, u[x].pos - window + 1) : 0;
+                u[x].row = (size_t)cu_new[b] + qc;
+                load_query(q + (u[x].row * nh + u[x].head) * HD, true, g, u[x].qv);
+                u[x].m = -INFINITY;
+                u[x].weights = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int dt = 0; dt < DTILES; ++dt) u[x].o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+            }
+            // the pages any query of the tile sees (the same for all waves)
+            const int tile_last = min(tile_first + qb - 1, n_new - 1);
+            const int p_hi = (start + tile_last) / PAGE_TOKENS;
+            const int p_lo = window > 0 ? max(0, start + tile_first - window + 1) / PAGE_TOKENS : 0;
+            auto load_page = [&](int p) {
+                const size_t at = ((size_t)pages[p] * nkv + kvh) * PAGE_TOKENS * HD;
+                const int stage = (p - p_lo) % STAGES;
+                page_into_lds(k_cache + at, v_cache + at, sources, k_lds + stage * K_TILE, v_lds + stage * V_TILE);
+            };
+            // is every key of page p visible to every column of this wave?
+            auto interior = [&](int p) -> bool {
+                bool inside = true;
+#pragma unroll
+                for (int x = 0; x < PF_UNITS; ++x)
+                    inside = inside && (!u[x].live || (u[x].first <= p * PAGE_TOKENS && u[x].pos >= p * PAGE_TOKENS + PAGE_TOKENS - 1));
+                return __all(inside);
+            };
+            wait_for_all_but_the_youngest_loads<0>();                 // the queries
+#pragma unroll
+            for (int ahead = 0; ahead < STAGES - 1; ++ahead)
+                if (p_lo + ahead <= p_hi) load_page(p_lo + ahead);
+            // the first page has landed when at most the pages after it are on their way
+            if constexpr (STAGES > 2) {
+                const int young = min(p_hi - p_lo, STAGES - 2);
+                if (young >= 2) wait_for_all_but_the_youngest_loads<2 * PAGE_LOADS>();
+                else if (young == 1) wait_for_all_but_the_youngest_loads<PAGE_LOADS>();
+                else wait_for_all_but_the_youngest_loads<0>();
+            } else {
+                wait_for_all_but_the_youngest_loads<0>();
+            }
+            page_barrier();
+            for (int p = p_lo; p <= p_hi; ++p) {
+                const int stage = (p - p_lo) % STAGES;
+                if (p + STAGES - 1 <= p_hi) load_page(p + STAGES - 1);      // into the stage whose readers passed the barrier a page ago
+                bf16_t* v_page = v_lds + stage * V_TILE;
+                if (seq_tail - p * PAGE_TOKENS < PAGE_TOKENS - 1) {          // the sequence's last page: no page follows it
+                    blank_values_after(v_page, seq_tail - p * PAGE_TOKENS);
+                    __syncthreads();
+                }
+                paired_page<PRESCALED>(k_lds + stage * K_TILE, v_page, u, p * PAGE_TOKENS, scale_log2, r, g, !interior(p));
+                // the next page has landed when at most the pages after it are on their way
+                if constexpr (STAGES > 2) {
+                    const int young = min(p_hi, p + STAGES - 1) - (p + 1);
+                    if (young >= 2) wait_for_all_but_the_youngest_loads<2 * PAGE_LOADS>();
+                    else if (young == 1) wait_for_all_but_the_youngest_loads<PAGE_LOADS>();
+                    else wait_for_all_but_the_youngest_loads<0>();
+                } else {
+                    wait_for_all_but_the_youngest_loads<0>();
+                }
+                page_barrier();
+            }
+#pragma unroll
+            for (int x = 0; x < PF_UNITS; ++x) {
+                if (u[x].valid) {
+                    const float inv = 1.0f / u[x].weights[0];
+                    bf16_t* o = out + (u[x].row * nh + u[x].head) * HD;
+#pragma unroll
+                    for (int dt = 0; dt < DTILES; ++dt) {           // the lane's four elements of a tile lie side by side: one store
+                        uint2 four;
+                        four.x = (uint32_t)f32_to_bf16(u[x].o[dt][0] * inv).bits | ((uint32_t)f32_to_bf16(u[x].o[dt][1] * inv).bits << 16);
+                        four.y = (uint32_t)f32_to_bf16(u[x].o[dt][2] * inv).bits | ((uint32_t)f32_to_bf16(u[x].o[dt][3] * inv).bits << 16);
+                        *reinterpret_cast<uint2*>(o + dt * 16 + 4 * g) = four;
+                    }
+                }
+            }
+        }
+    }
+}
+
+// q_prescaled: the queries come multiplied by scale * log2(e) already (by the pass that rounds them), so a score is
+// the exponent of its weight as it leaves the matrix cores; `scale` is then not applied again.
 PALM_API int palm_attention_prefill(hipStream_t stream, const void* q, const void* k_cache, const void* v_cache,
                                     const int* block_table, int max_pages, const int* seq_slot, const int* seq_start,
                                     const int* seq_new, const int* cu_new, int n_seqs, int max_new, int nh, int nkv,
-                                    int hd, float scale, int window, void* out) {
+                                    int hd, float scale, int window, int q_prescaled, void* out) {
     PALM_CHECK(hd == HD, "attention_prefill: this library was built for head size %d, not %d", HD, hd);
     PALM_CHECK(n_seqs >= 0 && max_new >= 0 && nh > 0 && nkv > 0 && nh % nkv == 0,
                "attention_prefill: seqs=%d max_new=%d heads=%d kv=%d", n_seqs, max_new, nh, nkv);
@@ -1233,16 +1506,37 @@ PALM_API int palm_attention_prefill(hipStream_t stream, const void* q, const voi
     const int qb = 16 * (UNITS / hg > 0 ? UNITS / hg : 1);     // query positions in a tile
     const int n_hg = (G + hg - 1) / hg;
     PALM_CHECK(nkv * n_hg <= 65535 && n_seqs <= 65535, "attention_prefill: grid too large");
-    const int n16 = (max_new + 15) / 16, subs = qb / 16;
+    const float scale_log2 = q_prescaled ? 1.0f : scale * LOG2E;
     // Blocks are handed to the chip's eight dies in turn by their number, and each die has an L2 of its own.  With
     // the kv head as the fastest index, the blocks that a die gets belong to few kv heads (one, with eight of
     // them), whose keys and values then stay in that die's L2 for all the query tiles that read them.
+    if constexpr (PF_DMA) {
+        const int n_q = (max_new + qb - 1) / qb;
+        PALM_CHECK(n_q <= 65535, "attention_prefill: %d new tokens are more than one launch takes", max_new);
+        dim3 grid(nkv * n_hg, n_q, n_seqs);
+        const long long blocks = (long long)grid.x * grid.y * grid.z;
+        // four pages in LDS leave a compute unit room for one block: where the launch has no second block for it anyway
+        const bool few = blocks <= 256;
+        const int partners_follow = blocks <= 512 && n_seqs == 1;     // all blocks run at once, two a unit
+#define PALM_PAIRED(STAGES, PRE) attention_prefill_paired_kernel<STAGES, PRE><<<grid, PF_THREADS, 0, stream>>>( \
+        (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages, seq_slot, seq_start, seq_new, \
+        cu_new, nh, nkv, scale_log2, window, qb, hg, partners_follow, (bf16_t*)out)
+        if (few) { if (q_prescaled) PALM_PAIRED(4, true); else PALM_PAIRED(4, false); }
+        else { if (q_prescaled) PALM_PAIRED(2, true); else PALM_PAIRED(2, false); }
+#undef PALM_PAIRED
+        PALM_LAUNCHED();
+        return 0;
+    }
+    PALM_CHECK(!q_prescaled, "attention_prefill: head size %d takes its queries as they are and applies the scale itself", HD);
+    const int n16 = (max_new + 15) / 16, subs = qb / 16;
     const int n_tiles = subs > 1 ? ((n16 + 1) / 2 + subs / 2 - 1) / (subs / 2) : n16;
     PALM_CHECK(n_tiles <= 65535, "attention_prefill: %d new tokens are more than one launch takes", max_new);
     dim3 grid(nkv * n_hg, n_tiles, n_seqs);
     attention_prefill_kernel<<<grid, PF_THREADS, 0, stream>>>((const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache,
                                                              block_table, max_pages, seq_slot, seq_start, seq_new, cu_new, nh,
-                                                             nkv, scale * LOG2E, window, qb, hg, (bf16_t*)out);
+                                                             nkv, scale_log2, window, qb, hg, (bf16_t*)out);
     PALM_LAUNCHED();
     return 0;
 }
+
+PALM_API int palm_attention_prefill_takes_prescaled() { return PF_DMA ? 1 : 0; }

@@ -546,7 +546,8 @@ _ATTENTION_SIGNATURES = {
     "palm_attention_decode": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int,
                               c_int, c_int, c_float, c_int, c_int, c_void_p, c_void_p],
     "palm_attention_prefill": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
-                               c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
+                               c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p],
+    "palm_attention_prefill_takes_prescaled": [],
     "palm_attention_decode_fused": [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_int,
                                     c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int,
                                     c_int, c_int, c_float, c_int, c_int, c_void_p, c_void_p],
@@ -668,9 +669,22 @@ def attention_decode_fused(qkv, k_cache, v_cache, block_table, seq_slot, seq_sta
     return out
 
 
+LOG2E = 1.4426950408889634
+
+
+def prefill_q_scale(hd: int, dtype, scale: float) -> float:
+    """What the pass that rounds a prompt's queries should multiply them by first: scale * log2(e) where the prompt
+    attention kernel of this head size takes its queries so (a score is then the exponent of its weight as it leaves
+    the matrix cores), else 1."""
+    if dtype == BF16 and hd in MFMA_HEAD_DIMS and attention_lib(hd).palm_attention_prefill_takes_prescaled():
+        return float(scale) * LOG2E
+    return 1.0
+
+
 def attention_prefill(q, k_cache, v_cache, block_table, seq_slot, seq_start, seq_new, cu_new, max_new: int, nh: int,
-                      nkv: int, hd: int, scale: float, window: int | None) -> torch.Tensor:
-    """The step's queries (several for each sequence) over the cache, on the matrix cores."""
+                      nkv: int, hd: int, scale: float, window: int | None, q_prescaled: bool = False) -> torch.Tensor:
+    """The step's queries (several for each sequence) over the cache, on the matrix cores.  ``q_prescaled``: the
+    queries come multiplied by ``prefill_q_scale`` already, and ``scale`` is not applied again."""
     _attention_checks("attention_prefill", q, k_cache, v_cache, block_table, nh, nkv, hd, seq_slot, seq_start, seq_new, cu_new)
     B = seq_slot.shape[0]
     _need(seq_start.shape == (B,) and seq_new.shape == (B,) and cu_new.shape == (B + 1,),
@@ -678,7 +692,7 @@ def attention_prefill(q, k_cache, v_cache, block_table, seq_slot, seq_start, seq
     out = torch.empty_like(q)
     library.call(attention_lib(hd), "palm_attention_prefill", _stream(), _p(q), _p(k_cache), _p(v_cache), _p(block_table),
                  block_table.shape[1], _p(seq_slot), _p(seq_start), _p(seq_new), _p(cu_new), B, int(max_new), nh, nkv, hd,
-                 float(scale), int(window or 0), _p(out))
+                 float(scale), int(window or 0), int(bool(q_prescaled)), _p(out))
     return out
 
 
