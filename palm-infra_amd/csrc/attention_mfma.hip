@@ -1258,6 +1258,7 @@ struct PairedUnit {           // one (head, 16 query positions): the wave's shar
 };
 
 // masked (the same in every lane): some column of the wave does not see every key of the page
+constexpr int VALUES_AHEAD = DTILES / 2;       // value tiles whose fragments are asked for before the weights are made
 template <bool PRESCALED>
 __device__ __forceinline__ void paired_page(const bf16_t* k_lds, const bf16_t* v_lds, PairedUnit (&u)[PF_UNITS], int page_first_key,
                                             float scale_log2, int r, int g, bool masked) {
@@ -1265,25 +1266,32 @@ __device__ __forceinline__ void paired_page(const bf16_t* k_lds, const bf16_t* v
     float sub[PF_UNITS];
 #pragma unroll
     for (int x = 0; x < PF_UNITS; ++x) sub[x] = u[x].m == -INFINITY ? 0.f : u[x].m;
-    bf16x8 kf[2][KSTEPS];
-    read_key_fragments(k_lds, 0, r, g, kf[0]);
+    // A fragment read from LDS takes longer than the few matrix instructions it feeds, so fragments are asked for
+    // well ahead: all of a page's keys at once (the weights' and values' registers are free then), and the values
+    // as soon as the scores are done, so that they arrive while the weights are made.
+    bf16x8 kf[4][KSTEPS];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) read_key_fragments(k_lds, t, r, g, kf[t]);
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
-        if (t < 3) read_key_fragments(k_lds, t + 1, r, g, kf[(t + 1) & 1]);
 #pragma unroll
         for (int x = 0; x < PF_UNITS; ++x) {
             const float from = PRESCALED ? -sub[x] : 0.f;
             f32x4 acc = f32x4{from, from, from, from};
 #pragma unroll
-            for (int j = 0; j < KSTEPS; ++j) acc = mfma_16x16x32(kf[t & 1][j], u[x].qv[j], acc);
+            for (int j = 0; j < KSTEPS; ++j) acc = mfma_16x16x32(kf[t][j], u[x].qv[j], acc);
             s[x][t] = acc;
         }
-        __builtin_amdgcn_sched_barrier(0);          // or every tile's fragments are asked for at once and the registers run out
     }
-    // the first values are asked for now and arrive while the weights are made
-    bf16x8 vf[2][2];
+    __builtin_amdgcn_sched_barrier(0);
+    bf16x8 vf[DTILES][2];
 #pragma unroll
-    for (int h = 0; h < 2; ++h) vf[0][h] = *reinterpret_cast<const bf16x8*>(v_lds + r * V_STRIDE + ((h * 4 + g) ^ v_swizzle(r)) * 8);
+    for (int dt = 0; dt < VALUES_AHEAD; ++dt) {
+        const int row = dt * 16 + r;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) vf[dt][h] = *reinterpret_cast<const bf16x8*>(v_lds + row * V_STRIDE + ((h * 4 + g) ^ v_swizzle(row)) * 8);
+    }
+    __builtin_amdgcn_sched_barrier(0);
 
     bool vote = masked;
     float mx[PF_UNITS];
@@ -1351,20 +1359,19 @@ __device__ __forceinline__ void paired_page(const bf16_t* k_lds, const bf16_t* v
     for (int x = 0; x < PF_UNITS; ++x)
 #pragma unroll
         for (int h = 0; h < 2; ++h) u[x].weights = mfma_16x16x32(ones, pv[x][h], u[x].weights);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int dt = 0; dt < DTILES; ++dt) {
-        if (dt + 1 < DTILES) {
-            const bf16_t* vrow = v_lds + ((dt + 1) * 16 + r) * V_STRIDE;
+    for (int dt = VALUES_AHEAD; dt < DTILES; ++dt) {        // the rest of the values, now that the scores' registers are free
+        const int row = dt * 16 + r;
 #pragma unroll
-            for (int h = 0; h < 2; ++h)
-                vf[(dt + 1) & 1][h] = *reinterpret_cast<const bf16x8*>(vrow + ((h * 4 + g) ^ v_swizzle((dt + 1) * 16 + r)) * 8);
-        }
+        for (int h = 0; h < 2; ++h) vf[dt][h] = *reinterpret_cast<const bf16x8*>(v_lds + row * V_STRIDE + ((h * 4 + g) ^ v_swizzle(row)) * 8);
+    }
+#pragma unroll
+    for (int dt = 0; dt < DTILES; ++dt)
 #pragma unroll
         for (int h = 0; h < 2; ++h)
 #pragma unroll
-            for (int x = 0; x < PF_UNITS; ++x) u[x].o[dt] = mfma_16x16x32(vf[dt & 1][h], pv[x][h], u[x].o[dt]);
-        __builtin_amdgcn_sched_barrier(0);
-    }
+            for (int x = 0; x < PF_UNITS; ++x) u[x].o[dt] = mfma_16x16x32(vf[dt][h], pv[x][h], u[x].o[dt]);
 }
 
 template <int STAGES, bool PRESCALED>

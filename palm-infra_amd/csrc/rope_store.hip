@@ -33,7 +33,7 @@ __global__ __launch_bounds__(WAVE) void qk_norm_rope_store_kernel(
     const int* __restrict__ positions, const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w,
     float eps, const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rotary_dim, int pairing,
     int nh, int nkv, int hd,
-    int write_cache) {
+    int write_cache, float q_scale) {
     __shared__ float vals[MAX_HEAD_DIM];
     const int t = blockIdx.x;
     const int head = blockIdx.y;                 // 0..nh-1: q, then nkv k heads, then nkv v heads
@@ -89,13 +89,15 @@ __global__ __launch_bounds__(WAVE) void qk_norm_rope_store_kernel(
         return;
     }
     T* dst;
+    float scale = 1.0f;
     if (kind == 0) {
         dst = q_out + ((size_t)t * nh + head) * hd;
+        scale = q_scale;                         // what the attention kernel wants folded into the queries before they are rounded
     } else {
         const int g = head - nh;
         dst = k_cache + (((size_t)page * nkv + g) * PAGE_TOKENS + pos % PAGE_TOKENS) * hd;
     }
-    for (int d = lane; d < hd; d += WAVE) dst[d] = from_float<T>(vals[d]);
+    for (int d = lane; d < hd; d += WAVE) dst[d] = from_float<T>(vals[d] * scale);
 }
 
 // ---- the same for many tokens (prompts) -------------------------------------------------------------
@@ -187,7 +189,7 @@ __global__ __launch_bounds__(4 * WAVE) void qk_norm_rope_fast_kernel(
     const int* __restrict__ block_table, int max_pages, const int* __restrict__ tok_slot,
     const int* __restrict__ positions, const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w,
     float eps, const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rotary_dim, int pairing,
-    int nh, int nkv, int hd, int L, int write_cache) {
+    int nh, int nkv, int hd, int L, int write_cache, float q_scale) {
     constexpr int U = FAST_HEADS_AT_ONCE;
     const int t = blockIdx.x;
     const int per_wave = WAVE / L;
@@ -265,6 +267,10 @@ __global__ __launch_bounds__(4 * WAVE) void qk_norm_rope_fast_kernel(
                         x[u][e + 1] = turn ? x0 * sn[e] + x1 * c[e] : x1;
                     }
                 }
+            }
+            if (!is_k) {
+#pragma unroll
+                for (int e = 0; e < E; ++e) x[u][e] *= q_scale;
             }
             if (head[u] < n_heads) {
                 T* dst = is_k ? k_cache + k_row + (size_t)(head[u] - nh) * PAGE_TOKENS * hd : q_out + ((size_t)t * nh + head[u]) * hd;
@@ -346,12 +352,13 @@ __global__ __launch_bounds__(4 * WAVE) void v_store_tile_kernel(
 }
 
 // dtype: the element type of q_out and of the cache, and of qkv if planes == 1; with planes > 1 qkv is
-// [planes, n_tokens, (nh + 2 nkv) * hd] float32.
+// [planes, n_tokens, (nh + 2 nkv) * hd] float32.  q_scale: a factor on the queries (not the keys), applied in 32-bit
+// before they are rounded: 1, or what the attention kernel that reads them wants folded in.
 PALM_API int palm_qk_norm_rope_store(hipStream_t stream, const void* qkv, int dtype, int planes, void* q_out, void* k_cache,
                                      void* v_cache, const int* block_table, int max_pages, const int* tok_slot,
                                      const int* positions, const float* q_norm_w, const float* k_norm_w, float eps,
                                      const float* cos_t, const float* sin_t, int rotary_dim, int pairing,
-                                     int n_tokens, int nh, int nkv, int hd, int write_cache) {
+                                     int n_tokens, int nh, int nkv, int hd, int write_cache, float q_scale) {
     PALM_CHECK(n_tokens >= 0 && nh > 0 && nkv > 0 && hd > 0, "qk_norm_rope_store: tokens=%d heads=%d kv=%d hd=%d",
                n_tokens, nh, nkv, hd);
     PALM_CHECK(hd <= MAX_HEAD_DIM, "qk_norm_rope_store: head_dim %d exceeds %d", hd, MAX_HEAD_DIM);
@@ -374,7 +381,7 @@ PALM_API int palm_qk_norm_rope_store(hipStream_t stream, const void* qkv, int dt
 #define PALM_ROPE_FAST_E(TIN, T, EE) case EE: \
         qk_norm_rope_fast_kernel<TIN, T, EE><<<qk_grid, 4 * WAVE, 0, stream>>>( \
             (const TIN*)qkv, (T*)q_out, (T*)k_cache, block_table, max_pages, tok_slot, positions, \
-            q_norm_w, k_norm_w, eps, cos_t, sin_t, rotary_dim, pairing, nh, nkv, hd, L, write_cache); break;
+            q_norm_w, k_norm_w, eps, cos_t, sin_t, rotary_dim, pairing, nh, nkv, hd, L, write_cache, q_scale); break;
 #define PALM_ROPE_FAST(TIN, T) do { \
         switch (hd / L) { \
             PALM_ROPE_FAST_E(TIN, T, 1) PALM_ROPE_FAST_E(TIN, T, 2) PALM_ROPE_FAST_E(TIN, T, 3) PALM_ROPE_FAST_E(TIN, T, 4) \
@@ -393,12 +400,12 @@ PALM_API int palm_qk_norm_rope_store(hipStream_t stream, const void* qkv, int dt
         PALM_DTYPE_SWITCH(dtype, T,
             (qk_norm_rope_store_kernel<float, T><<<grid, WAVE, 0, stream>>>(
                 (const float*)qkv, planes, plane_stride, (T*)q_out, (T*)k_cache, (T*)v_cache, block_table, max_pages,
-                tok_slot, positions, q_norm_w, k_norm_w, eps, cos_t, sin_t, rotary_dim, pairing, nh, nkv, hd, write_cache)));
+                tok_slot, positions, q_norm_w, k_norm_w, eps, cos_t, sin_t, rotary_dim, pairing, nh, nkv, hd, write_cache, q_scale)));
     } else {
         PALM_DTYPE_SWITCH(dtype, T,
             (qk_norm_rope_store_kernel<T, T><<<grid, WAVE, 0, stream>>>(
                 (const T*)qkv, 1, plane_stride, (T*)q_out, (T*)k_cache, (T*)v_cache, block_table, max_pages,
-                tok_slot, positions, q_norm_w, k_norm_w, eps, cos_t, sin_t, rotary_dim, pairing, nh, nkv, hd, write_cache)));
+                tok_slot, positions, q_norm_w, k_norm_w, eps, cos_t, sin_t, rotary_dim, pairing, nh, nkv, hd, write_cache, q_scale)));
     }
     PALM_LAUNCHED();
     return 0;

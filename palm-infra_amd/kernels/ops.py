@@ -29,7 +29,7 @@ _SIGNATURES = {
     "palm_linear": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int],
     "palm_qk_norm_rope_store": [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                                 c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
-                                c_int, c_int, c_int],
+                                c_int, c_int, c_int, c_float],
     "palm_rope_table": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int],
     "palm_attention_simple": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                               c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
@@ -224,10 +224,11 @@ def _check_cache(what, k_cache, v_cache, block_table, nkv, hd):
 def qk_norm_rope_store(qkv: torch.Tensor, nh: int, nkv: int, hd: int, positions: torch.Tensor, *, q_norm_w=None,
                        k_norm_w=None, eps: float = 0.0, cos=None, sin=None, rotary_dim: int = 0, pairing: int = 0,
                        k_cache=None, v_cache=None, block_table=None, tok_slot=None, write_cache: bool = True,
-                       out_dtype: torch.dtype | None = None) -> torch.Tensor:
+                       out_dtype: torch.dtype | None = None, q_scale: float = 1.0) -> torch.Tensor:
     """qkv [n, (nh + 2 nkv) hd] -> q [n, nh hd], normed and rotated by the cos/sin rows [n, rotary_dim/2];
     k (normed, rotated) and v go to the cache page of (tok_slot[t], positions[t]).  qkv may also be float32
-    planes [P, n, (nh + 2 nkv) hd] to be added up; ``out_dtype`` then names the type of q and of the cache."""
+    planes [P, n, (nh + 2 nkv) hd] to be added up; ``out_dtype`` then names the type of q and of the cache.
+    ``q_scale``: a factor on q (not k), applied before the rounding (see ``prefill_q_scale``)."""
     _dev("qk_norm_rope_store", qkv, positions, q_norm_w, k_norm_w, cos, sin, k_cache, v_cache, block_table, tok_slot)
     _i32("qk_norm_rope_store", positions, block_table, tok_slot)
     planes = 1
@@ -264,7 +265,8 @@ def qk_norm_rope_store(qkv: torch.Tensor, nh: int, nkv: int, hd: int, positions:
     q_out = torch.empty((n, nh * hd), dtype=out_dtype, device=qkv.device)
     library.call(core(), "palm_qk_norm_rope_store", _stream(), _p(qkv), _code(q_out, "qkv"), planes, _p(q_out), _p(k_cache), _p(v_cache),
                  _p(block_table), max_pages, _p(tok_slot), _p(positions), _p(q_norm_w), _p(k_norm_w), float(eps),
-                 _p(cos), _p(sin), int(rotary_dim if cos is not None else 0), int(pairing), n, nh, nkv, hd, int(write_cache))
+                 _p(cos), _p(sin), int(rotary_dim if cos is not None else 0), int(pairing), n, nh, nkv, hd, int(write_cache),
+                 float(q_scale))
     return q_out
 
 
@@ -702,8 +704,14 @@ def slices_of_step(ctx, nh: int, nkv: int, window: int | None) -> int:
     return ctx.decode_slices or decode_slices(ctx.n_seqs, nh, nkv, keys)
 
 
-def attention(q, k_cache, v_cache, block_table, ctx, nh: int, nkv: int, hd: int, scale: float, window: int | None):
-    """The step's queries over the cache; picks the kernel by element type, head size and step shape."""
+def attention(q, k_cache, v_cache, block_table, ctx, nh: int, nkv: int, hd: int, scale: float, window: int | None,
+              q_prescaled: bool = False):
+    """The step's queries over the cache; picks the kernel by element type, head size and step shape.
+    ``q_prescaled``: see ``attention_prefill`` (only a prompt step on the matrix cores takes such queries)."""
+    if q_prescaled:
+        _need(mfma_attention_serves(q, hd) and not ctx.is_decode, "attention: only the prompt kernel takes scaled queries")
+        return attention_prefill(q, k_cache, v_cache, block_table, ctx.seq_slot, ctx.seq_start, ctx.seq_new, ctx.cu_new,
+                                 ctx.max_new, nh, nkv, hd, scale, window, q_prescaled=True)
     if mfma_attention_serves(q, hd):
         if ctx.is_decode:
             n_slices = slices_of_step(ctx, nh, nkv, window)

@@ -73,12 +73,16 @@ class Attention:
                 eps=self.q_norm.eps if self.q_norm else 0.0, cos=cos, sin=sin, rotary_dim=rotary_dim, pairing=pairing,
                 write_cache=lc.writes)
             return self.out(o, sink=sink)
+        # a prompt's queries carry the scale (times log2 e) into their one rounding where the prompt kernel of this
+        # head size takes them so: a score then leaves the matrix cores as the exponent of its weight
+        q_scale = 1.0 if ctx.is_decode else ops.prefill_q_scale(self.hd, self.dtype, self.scale)
         q = ops.qk_norm_rope_store(
             qkv, self.nh, self.nkv, self.hd, ctx.positions,
             q_norm_w=self.q_norm.weight if self.q_norm else None, k_norm_w=self.k_norm.weight if self.k_norm else None,
             eps=self.q_norm.eps if self.q_norm else 0.0, cos=cos, sin=sin,
             rotary_dim=rotary_dim, pairing=pairing,
             k_cache=lc.k, v_cache=lc.v, block_table=lc.kv.table_dev, tok_slot=ctx.tok_slot, write_cache=lc.writes,
-            out_dtype=self.dtype)
-        o = ops.attention(q, lc.k, lc.v, lc.kv.table_dev, ctx, self.nh, self.nkv, self.hd, self.scale, self.window)
+            out_dtype=self.dtype, q_scale=q_scale)
+        o = ops.attention(q, lc.k, lc.v, lc.kv.table_dev, ctx, self.nh, self.nkv, self.hd, self.scale, self.window,
+                          q_prescaled=q_scale != 1.0)
         return self.out(o, sink=sink)

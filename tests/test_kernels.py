@@ -335,6 +335,18 @@ def test_qk_norm_rope_store_of_many_tokens(ops, dtype, nh, nkv, hd):
                                eps=eps, cos=cos[sl].contiguous(), sin=sin[sl].contiguous(), rotary_dim=hd, pairing=0, k_cache=kc2,
                                v_cache=vc2, block_table=table.to(DEV), tok_slot=torch.tensor(tslot[sl], dtype=torch.int32).to(DEV))
     assert torch.allclose(kc2.cpu().double(), kc, atol=1e-5 if dtype == F32 else 4e-2) and torch.equal(vc2.cpu().double(), vc)
+    # a factor on the queries (what a prompt's attention kernel wants folded in before they are rounded): q times
+    # the factor, keys and values as before; through the kernel for many tokens and the one for few
+    for sl in (slice(0, n), slice(0, 9)):
+        kc3, vc3 = _paged(10, nkv, hd, dtype)
+        q3 = ops.qk_norm_rope_store(qkv[sl].contiguous().to(DEV), nh, nkv, hd, pos_d[sl].contiguous(), q_norm_w=qw.to(DEV), k_norm_w=kw.to(DEV),
+                                    eps=eps, cos=cos[sl].contiguous(), sin=sin[sl].contiguous(), rotary_dim=hd, pairing=0, k_cache=kc3,
+                                    v_cache=vc3, block_table=table.to(DEV), tok_slot=torch.tensor(tslot[sl], dtype=torch.int32).to(DEV),
+                                    q_scale=0.375).cpu()
+        m = q3.shape[0]
+        assert torch.allclose(q3.double().reshape(m, nh, hd), 0.375 * rq[sl], atol=t)
+        if m == n:
+            assert torch.allclose(kc3.cpu().double(), kc, atol=1e-5 if dtype == F32 else 4e-2) and torch.equal(vc3.cpu().double(), vc)
 
 
 def test_qk_norm_rope_store_of_many_tokens_whole_or_in_planes_and_other_rotations(ops):

@@ -323,6 +323,26 @@ def test_attention_decode_mfma(ops, nh, nkv, hd, n_slices):
         assert torch.allclose(got, ref, atol=2e-2), (lens, float((got - ref).abs().max()))
 
 
+@pytest.mark.parametrize("nh,nkv,hd", [(32, 8, 128), (6, 3, 64), (2, 1, 128), (3, 3, 64)])
+def test_attention_prefill_with_the_scale_folded_into_the_queries(ops, nh, nkv, hd):
+    """The prompt kernel of the head sizes 64 and 128 takes queries that come multiplied by scale * log2(e): the
+    same attention as with plain queries and the scale applied inside.  (Other head sizes say that they do not.)"""
+    assert ops.prefill_q_scale(hd, BF16, 0.25) == pytest.approx(0.25 * 1.4426950408889634)
+    assert ops.prefill_q_scale(80, BF16, 0.25) == 1.0 and ops.prefill_q_scale(hd, F32, 0.25) == 1.0
+
+    def folded(q, kc, vc, table, slots, starts, news, cu, max_new, nh_, nkv_, hd_, scale, window):
+        qs = (q.float() * ops.prefill_q_scale(hd, BF16, scale)).to(BF16)
+        return ops.attention_prefill(qs, kc, vc, table, slots, starts, news, cu, max_new, nh, nkv, hd, scale, window, q_prescaled=True)
+    for window in (None, 70):
+        for lens in ([(20, 20)], [(300, 44)], [(64, 64), (65, 1), (130, 70), (7, 7), (200, 17)], [(1100, 1100)], [(2304, 300), (70, 70)]):
+            got, ref = _attention_case(ops, folded, BF16, nh, nkv, hd, lens, window, seed=len(lens) + hd, poison=True)
+            assert torch.isfinite(got).all() and torch.allclose(got, ref, atol=3e-2), (lens, window, float((got - ref).abs().max()))
+    from palm_infra_amd.kernels import KernelError
+    with pytest.raises(KernelError, match="applies the scale itself"):
+        _attention_case(ops, lambda q, kc, vc, table, slots, starts, news, cu, max_new, a, b, c, scale, window: ops.attention_prefill(
+            q, kc, vc, table, slots, starts, news, cu, max_new, 6, 1, 80, scale, window, q_prescaled=True), BF16, 6, 1, 80, [(20, 20)], None)
+
+
 @pytest.mark.parametrize("nh,nkv,hd", [(32, 8, 128), (4, 2, 64), (6, 1, 80)])
 def test_attention_mfma_long_sequences(ops, nh, nkv, hd):
     """The measured lengths and beyond: a 2,048-token prompt (32 pages, query tiles paired from both ends, a
