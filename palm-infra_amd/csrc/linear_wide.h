@@ -1,4 +1,4 @@
-// C[M, N] = A[M, K] . W[N, K]^T for 17 to 64 rows (decode steps of large batches): bfloat16 on the matrix
+// C[M, N] = A[M, K] . W[N, K]^T for 17 to 128 rows (decode steps of large batches, short prompts): bfloat16 on the matrix
 // cores, 32-bit accumulation.  The thin kernels (linear_mfma.hip) let every wave fetch the activations it
 // needs straight from the caches, which for more than 16 rows is several times the weight traffic; here a
 // block shares them through LDS.
@@ -6,7 +6,8 @@
 // A block has NW waves (4, 6 or 8, chosen with the number of K ranges so that the launch fills the compute
 // units evenly), each with a strip of 16 weight rows of its own against all MB*16 rows of A, and one range of
 // K (grid.y; the ranges' partial results are float32 planes [parts, M, N] that the reader adds up in the order
-// of the planes, as the norm after a projection and the q/k/v pass do).  K goes by in chunks of 256.  A lane's
+// of the planes, as the norm after a projection and the q/k/v pass do).  K goes by in chunks of 256 (of 128 for more
+// than 64 rows, whose operands would else not fit the registers and LDS).  A lane's
 // reads are a ring of three or four slots; a slot holds the eight weight fragments of one chunk (64 contiguous bytes
 // of a row per instruction, as in the thin kernels) and the lane's share of the activations of the chunk
 // after it.  Reads come back in the order they went out, so the wait for a slot leaves the younger slots
@@ -22,13 +23,12 @@
 
 enum WideEpilogue : int { WIDE_STORE = 0, WIDE_SWIGLU = 1 };
 
-constexpr int WIDE_CHUNK = 256;                 // k-values a step
-constexpr int WIDE_PIECES = WIDE_CHUNK / 8;     // 16-byte pieces of a row of the chunk
-constexpr int WIDE_STRIDE = WIDE_CHUNK + 8;     // a row in LDS, padded: the 16 rows that lanes read together start in 16 different banks
+// k-values a step, by the blocks of 16 rows a launch holds
+__host__ __device__ constexpr int wide_chunk(int row_blocks) { return row_blocks <= 4 ? 256 : 128; }
 // Slots of reads: a slot is 8 KB of weights a wave; the slot in use is not in flight, and a compute unit wants about
 // 100 KB on their way; four slots where the registers hold them (one wave a SIMD, or 32 rows), else three
 __host__ __device__ constexpr int wide_ring(int waves, int row_blocks) { return waves <= 4 || row_blocks <= 2 ? 4 : 3; }
-constexpr int WIDE_MAX_ROWS = 64;
+constexpr int WIDE_MAX_ROWS = 128;
 constexpr int WIDE_MAX_PARTS = 4;               // as many planes as the readers of planes add up
 constexpr int WIDE_MIN_CHUNKS = 4;              // a range of K is not shorter than this
 constexpr int WIDE_UNITS = 256;                 // compute units of the chip: a launch comes in rounds of so many blocks
@@ -60,6 +60,10 @@ __global__ __launch_bounds__(NW * WAVE) void linear_wide_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, TC* __restrict__ C, int M, int N, int K,
     int chunks_per_part) {
     constexpr int ROWS = MB * 16;
+    constexpr int WIDE_CHUNK = wide_chunk(MB);                            // k-values a step
+    constexpr int WIDE_PIECES = WIDE_CHUNK / 8;                           // 16-byte pieces of a row of the chunk
+    constexpr int WIDE_STRIDE = WIDE_CHUNK + 8;                           // a row in LDS, padded: the 16 rows that lanes read together start in 16 different banks
+    constexpr int FRAGMENTS = WIDE_CHUNK / 32;                            // matrix-core steps of a chunk
     constexpr int RING = wide_ring(NW, MB);
     constexpr int THREADS = NW * WAVE;
     constexpr int XS = (ROWS * WIDE_PIECES + THREADS - 1) / THREADS;      // pieces of a chunk's activations a thread carries
@@ -98,7 +102,7 @@ __global__ __launch_bounds__(NW * WAVE) void linear_wide_kernel(
 #pragma unroll
     for (int i = 0; i < XS; ++i) x_row[i] = (uint32_t)min(x_row0 + i * ROW_STEP, M - 1) * K * sizeof(bf16_t);
 
-    bf16x8 wf[RING][8], xs[RING][XS];
+    bf16x8 wf[RING][FRAGMENTS], xs[RING][XS];
     auto ask_rows = [&](int chunk, auto slot) __attribute__((always_inline)) {
         constexpr int s = decltype(slot)::value;
         // what lies beyond M or K reads a place that exists; put_rows makes zeros of it
@@ -111,7 +115,7 @@ __global__ __launch_bounds__(NW * WAVE) void linear_wide_kernel(
     auto ask_weights = [&](int chunk, auto slot) __attribute__((always_inline)) {
         constexpr int s = decltype(slot)::value;
         const char* from = w_base + (size_t)chunk * CHUNK_BYTES;
-        static_for<8>([&](auto jc) __attribute__((always_inline)) {
+        static_for<FRAGMENTS>([&](auto jc) __attribute__((always_inline)) {
             constexpr int j = decltype(jc)::value;
             if (EXACT) {
                 wf[s][j] = load_bf16x8_at<j * 64>(from, w_lane);
@@ -145,8 +149,8 @@ __global__ __launch_bounds__(NW * WAVE) void linear_wide_kernel(
         };
         fetch(0, 0);
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            if (j + 1 < 8) fetch(j + 1, (j + 1) & 1);
+        for (int j = 0; j < FRAGMENTS; ++j) {
+            if (j + 1 < FRAGMENTS) fetch(j + 1, (j + 1) & 1);
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb) acc[mb] = mfma_16x16x32(wf[s][j], xf[j & 1][mb], acc[mb]);
             __builtin_amdgcn_sched_barrier(0);             // or all 32 operands are fetched before the first product
@@ -231,7 +235,7 @@ template <int MB, int NW, typename TC, int EPI>
 static void launch_wide(hipStream_t stream, const void* a, const void* w, void* c, int M, int N, int K, WidePlan plan) {
     const int strips = EPI == WIDE_SWIGLU ? (N / 2 + 7) / 8 : (N + 15) / 16;
     dim3 grid((strips + NW - 1) / NW, plan.parts);
-    if (K % WIDE_CHUNK == 0)
+    if (K % wide_chunk(MB) == 0)
         linear_wide_kernel<MB, NW, true, TC, EPI><<<grid, NW * WAVE, 0, stream>>>(
             (const bf16_t*)a, (const bf16_t*)w, (TC*)c, M, N, K, plan.chunks_per_part);
     else
@@ -246,11 +250,13 @@ static void launch_wide_waves(hipStream_t stream, const void* a, const void* w, 
     else launch_wide<MB, 8, TC, EPI>(stream, a, w, c, M, N, K, plan);
 }
 
-// The kernels are instantiated in four files (store or gated epilogue, 32 or 64 rows), which compile side by side.
+// The kernels are instantiated in six files (store or gated epilogue; 32, 64 or 128 rows), which compile side by side.
 void wide_launch_store_32(hipStream_t stream, const void* a, const void* w, void* c, int c_dtype, int M, int N, int K, WidePlan plan);
 void wide_launch_store_64(hipStream_t stream, const void* a, const void* w, void* c, int c_dtype, int M, int N, int K, WidePlan plan);
 void wide_launch_gated_32(hipStream_t stream, const void* a, const void* w, void* c, int c_dtype, int M, int N, int K, WidePlan plan);
 void wide_launch_gated_64(hipStream_t stream, const void* a, const void* w, void* c, int c_dtype, int M, int N, int K, WidePlan plan);
+void wide_launch_store_128(hipStream_t stream, const void* a, const void* w, void* c, int c_dtype, int M, int N, int K, WidePlan plan);
+void wide_launch_gated_128(hipStream_t stream, const void* a, const void* w, void* c, int c_dtype, int M, int N, int K, WidePlan plan);
 
 #define PALM_WIDE_INSTANCE(NAME, MB, EPI) \
     void NAME(hipStream_t stream, const void* a, const void* w, void* c, int c_dtype, int M, int N, int K, WidePlan plan) { \

@@ -1,12 +1,15 @@
-// The entry points of the product for 17 to 64 rows (linear_wide.h has the kernel): the plan of a launch and the
+// The entry points of the product for 17 to 128 rows (linear_wide.h has the kernel): the plan of a launch and the
 // choice of the instance.
 #include "linear_wide.h"
 
 // Waves a block and ranges of K: what takes the fewest rounds of blocks over the compute units, a round
 // costing its chunks (and two for its start) times the waves that share a unit's reads.
-static WidePlan wide_plan(int N, int K, int epilogue, int max_parts) {
+static int row_blocks_of(int M) { return M <= 32 ? 2 : (M <= 64 ? 4 : 8); }       // of 16 rows: the instance that serves M rows
+
+static WidePlan wide_plan(int M, int N, int K, int epilogue, int max_parts) {
     const int strips = epilogue == WIDE_SWIGLU ? (N / 2 + 7) / 8 : (N + 15) / 16;
-    const int n_chunks = (K + WIDE_CHUNK - 1) / WIDE_CHUNK;
+    const int chunk = wide_chunk(row_blocks_of(M));
+    const int n_chunks = (K + chunk - 1) / chunk;
     WidePlan best{8, 1, n_chunks};
     long best_cost = -1;
     for (int parts = 1; parts <= max_parts; ++parts) {
@@ -23,21 +26,19 @@ static WidePlan wide_plan(int N, int K, int epilogue, int max_parts) {
 
 // Into how many planes the product comes if the caller takes planes (1: the result itself).
 PALM_API int palm_linear_wide_parts(int M, int N, int K, int epilogue) {
-    (void)M;
     if (epilogue == WIDE_SWIGLU || N <= 0 || K <= 0) return 1;
-    return wide_plan(N, K, epilogue, WIDE_MAX_PARTS).parts;
+    return wide_plan(M, N, K, epilogue, WIDE_MAX_PARTS).parts;
 }
 
 // How many blocks the launch would have: a caller with another way to the product takes that when these are few.
 PALM_API int palm_linear_wide_blocks(int M, int N, int K, int epilogue, int planes_ok) {
-    (void)M;
     if (N <= 0 || K <= 0) return 0;
-    const WidePlan plan = wide_plan(N, K, epilogue, planes_ok && epilogue == WIDE_STORE ? WIDE_MAX_PARTS : 1);
+    const WidePlan plan = wide_plan(M, N, K, epilogue, planes_ok && epilogue == WIDE_STORE ? WIDE_MAX_PARTS : 1);
     const int strips = epilogue == WIDE_SWIGLU ? (N / 2 + 7) / 8 : (N + 15) / 16;
     return (strips + plan.waves - 1) / plan.waves * plan.parts;
 }
 
-// a [M, K] bfloat16 with M <= 64, w [N, K] bfloat16; c [M, N] (store) or [M, N/2] (gated) in bfloat16 or float32,
+// a [M, K] bfloat16 with M <= 128, w [N, K] bfloat16; c [M, N] (store) or [M, N/2] (gated) in bfloat16 or float32,
 // or, with parts > 1 (as palm_linear_wide_parts says; store only), float32 planes [parts, M, N].
 PALM_API int palm_linear_wide(hipStream_t stream, const void* a, const void* w, void* c, int c_dtype, int M, int N, int K,
                               int epilogue, int parts) {
@@ -51,16 +52,18 @@ PALM_API int palm_linear_wide(hipStream_t stream, const void* a, const void* w, 
     // a lane's place within its wave's rows, and a row's within the activations, are 32-bit byte offsets
     PALM_CHECK((double)(epilogue == WIDE_SWIGLU ? N / 2 + 8 : 16) * K * 2 < 4.0e9 && (double)WIDE_MAX_ROWS * K * 2 < 4.0e9,
                "linear_wide: N=%d K=%d is beyond 32-bit offsets", N, K);
-    WidePlan plan = wide_plan(N, K, epilogue, parts > 1 ? WIDE_MAX_PARTS : 1);
+    WidePlan plan = wide_plan(M, N, K, epilogue, parts > 1 ? WIDE_MAX_PARTS : 1);
     PALM_CHECK(parts == 1 || (parts == plan.parts && epilogue == WIDE_STORE && c_dtype == PALM_F32),
                "linear_wide: %d planes asked for, %d planned (planes are float32, not gated)", parts, plan.parts);
     if (M == 0) return 0;
     if (epilogue == WIDE_SWIGLU) {
         if (M <= 32) wide_launch_gated_32(stream, a, w, c, c_dtype, M, N, K, plan);
-        else wide_launch_gated_64(stream, a, w, c, c_dtype, M, N, K, plan);
+        else if (M <= 64) wide_launch_gated_64(stream, a, w, c, c_dtype, M, N, K, plan);
+        else wide_launch_gated_128(stream, a, w, c, c_dtype, M, N, K, plan);
     } else {
         if (M <= 32) wide_launch_store_32(stream, a, w, c, c_dtype, M, N, K, plan);
-        else wide_launch_store_64(stream, a, w, c, c_dtype, M, N, K, plan);
+        else if (M <= 64) wide_launch_store_64(stream, a, w, c, c_dtype, M, N, K, plan);
+        else wide_launch_store_128(stream, a, w, c, c_dtype, M, N, K, plan);
     }
     PALM_LAUNCHED();
     return 0;

@@ -208,7 +208,7 @@ class Engine:
     # new contents in the same buffers.  A graph is keyed by the batch size, rounded up (rows that pad it
     # belong to a slot of their own and write into a page that is never read), and by the longest sequence,
     # rounded up to a power of two (it only sizes how attention cuts the key range).
-    GRAPH_MAX_BATCH = 64
+    GRAPH_MAX_BATCH = 128        # as many rows as the products' own kernels take: a recorded step runs no library code
 
     @staticmethod
     def _batch_bucket(n: int) -> int:

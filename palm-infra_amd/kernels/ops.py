@@ -353,7 +353,8 @@ def linear_library(a: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
 
 
 THIN_TOKENS = 16      # up to here every wave fetches its own activations; above, a block shares them through LDS
-WIDE_TOKENS = 64      # as many rows as that block holds
+WIDE_TOKENS = 128     # as many rows as that block holds
+WIDE_FLOAT32_TOKENS = 64   # a float32 result (logits) of more rows than this goes through the tiled kernel instead
 
 
 COMPUTE_UNITS = 256     # of an MI355X; a folded product's blocks come in rounds of this many
@@ -378,10 +379,13 @@ WIDE_MIN_BLOCKS = 128   # of 256 compute units
 
 
 def wide_pays(M: int, N: int, K: int, gated: bool = False, planes_ok: bool = False) -> bool:
-    """Whether the kernel for 17 to 64 rows has enough blocks for this product to beat the library: with few
+    """Whether the kernel for 17 to 128 rows has enough blocks for this product to beat the library: with few
     weight rows it does only if the reader takes planes of partial sums.  Measured at Qwen3-8B's shapes with 64
     rows (us, own against library): q/k/v 18 and 18, output projection 14 and 16, down 27 and 37 as planes (76
-    whole), gate/up 45 gated against 46 with the activation's own pass; with 32 rows 14/17, 11/13, 23/26, 40/47."""
+    whole), gate/up 45 gated against 46 with the activation's own pass; with 32 rows 14/17, 11/13, 23/26, 40/47;
+    with 128 rows q/k/v 22 and 26, output projection 17 and 25, down 37 and 65, gate/up 65 gated against 53 and the
+    activation's pass of 8 (kept all the same: a step of up to 128 sequences then runs no library code and can be
+    recorded)."""
     return THIN_TOKENS < M <= WIDE_TOKENS and core().palm_linear_wide_blocks(
         M, N, K, 1 if gated else 0, 1 if planes_ok else 0) >= WIDE_MIN_BLOCKS
 
@@ -464,13 +468,13 @@ def linear_thin(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, gated:
                      1 if gated else 0, planes, _p(row_ss), pieces, float(row_eps), None, None, None)
         return out
     _need(row_ss is None, f"linear_thin: rows that lack their norm's factor come at most {THIN_TOKENS} at a time, not {M}")
-    if M > WIDE_TOKENS:
+    if M > WIDE_TOKENS or (M > WIDE_FLOAT32_TOKENS and out_dtype == F32 and not planes_ok):
         # a float32 result for many rows (logits at many places): the tiled kernel, which reads the weight once for
         # every 256 rows; where K is no whole number of its stages, 64 rows at a time
         if tile_serves(a, w):
             return linear_tile(a, w, out_dtype, gated=gated)
-        return torch.cat([linear_thin(a[r0:r0 + WIDE_TOKENS], w, out_dtype, gated=gated)
-                          for r0 in range(0, M, WIDE_TOKENS)])
+        return torch.cat([linear_thin(a[r0:r0 + WIDE_FLOAT32_TOKENS], w, out_dtype, gated=gated)
+                          for r0 in range(0, M, WIDE_FLOAT32_TOKENS)])
     # more rows than one block of 16: the kernel that shares the activations through LDS
     planes = core().palm_linear_wide_parts(M, N, K, 0) if planes_ok and not gated else 1
     if planes > 1:

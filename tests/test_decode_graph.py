@@ -53,6 +53,37 @@ def test_replays_equal_plain_launches(model_dirs, name, dtype):
     assert not e._decode_graphs
 
 
+@pytest.mark.parametrize("name,dtype", [("B", "bfloat16"), ("D", "bfloat16"), ("A", "float32")])
+def test_recorded_steps_of_65_to_128_sequences(model_dirs, name, dtype):
+    """Steps of more than 64 sequences are recorded too (their products go through the kernel that shares up to 128
+    rows through LDS, their logits through the tiled one): against the plain implementation, with sequences that
+    end on the way, so that the batch passes through several padded sizes, and each size is replayed."""
+    import plain_qwen3 as P
+    from palm_infra_amd.engine import Engine, StepEntry
+    n_seqs = 128
+    eng = Engine.from_dir(model_dirs[name][dtype], dtype=dtype, max_tokens=64 * 2 * n_seqs, max_seqs=n_seqs)
+    reqs = tiny.prompts(name, [9 + (7 * i) % 60 for i in range(n_seqs)], seed=36)
+    cfg, w = P.read_model(model_dirs[name][dtype])
+    refs = [P.logits(cfg, w, r) for r in reqs]
+    slots = [eng.open() for _ in reqs]
+    eng.step([StepEntry(s, r[:-8], []) for s, r in zip(slots, reqs)])
+    live = list(range(n_seqs))
+    pool = tiny.LogitsPool(dtype, f"{name}: recorded steps of many sequences")
+    for t in range(8, 0, -1):
+        if t in (6, 4, 2):                                          # 128 -> 106 -> 88 -> 73
+            gone, live = live[::6], [i for k, i in enumerate(live) if k % 6]
+            for i in gone:
+                eng.close(slots[i])
+        got = eng.step([StepEntry(slots[i], [reqs[i][-t]], [0]) for i in live])
+        pool.add(got, torch.stack([refs[i][len(reqs[i]) - t] for i in live]), f"{len(live)} sequences, {t} before the end")
+    pool.check()
+    sizes = sorted(k[0] for k, st in eng._decode_graphs.items() if k[0] != "prompt" and st["graph"] is not None)
+    assert sizes == [80, 88, 112, 128], sizes                       # each size ran twice: once plain, once recorded and replayed
+    for i in live:
+        eng.close(slots[i])
+    eng.cache.check()
+
+
 def test_a_wanted_subset_and_an_empty_one(model_dirs):
     from palm_infra_amd.engine import Engine, StepEntry
     g = Engine.from_dir(model_dirs["A"]["bfloat16"], dtype="bfloat16", max_tokens=64 * 8)

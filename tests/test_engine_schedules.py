@@ -274,10 +274,10 @@ def test_a_mixed_step_of_running_sequences_a_fresh_prompt_and_a_continuation(mod
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("n_seqs", [70, 130])
+@pytest.mark.parametrize("n_seqs", [150, 290])
 def test_decode_steps_of_more_sequences_than_a_recorded_step_takes(model_dirs, dtype, n_seqs):
-    """70 and 130 sequences one token each: beyond the batch sizes that are recorded into graphs, so these are
-    plain launches with the products of more than 64 rows and an attention grid of more than 64 sequences.
+    """150 and 290 sequences one token each: beyond the batch sizes that are recorded into graphs, so these are
+    plain launches with the products of more than 128 rows and an attention grid of as many sequences.
     Unequal lengths; some of the sequences end between the steps."""
     from palm_infra_amd.engine import Engine, StepEntry
     name = "B"
@@ -291,8 +291,8 @@ def test_decode_steps_of_more_sequences_than_a_recorded_step_takes(model_dirs, d
     live = list(range(n_seqs))
     pool = tiny.LogitsPool(dtype, f"{n_seqs} sequences a step")
     for t in (3, 2, 1):
-        if t == 1:                                                  # 130 -> 87, 70 -> 65: still more than a recorded step takes
-            every = 3 if n_seqs == 130 else 14
+        if t == 1:                                                  # 290 -> 193, 150 -> 139: still more than a recorded step takes
+            every = 3 if n_seqs == 290 else 14
             gone, live = live[::every], [i for k, i in enumerate(live) if k % every]
             for i in gone:
                 eng.close(slots[i])

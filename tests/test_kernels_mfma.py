@@ -22,7 +22,7 @@ def rand(*shape, seed=0, scale=1.0, dtype=BF16):
     return (torch.randn(*shape, generator=torch.Generator().manual_seed(seed)) * scale).to(dtype)
 
 
-@pytest.mark.parametrize("M", [1, 8, 16, 17, 33, 64, 70, 150])
+@pytest.mark.parametrize("M", [1, 8, 16, 17, 33, 64, 70, 128, 150])
 @pytest.mark.parametrize("N,K", [(7, 8), (130, 64), (515, 80), (1000, 224), (96, 4096), (4096, 1536), (300, 12288),
                                  (1000, 2048), (515, 2056), (130, 5000), (9000, 2048), (8200, 3080), (64, 8192), (48, 7000),
                                  (4200, 5120)])
@@ -33,7 +33,12 @@ def test_linear_thin_against_the_plain_product(ops, M, N, K):
     # exact products of bfloat16 values, added in 32-bit: only the order of the sum differs
     assert torch.allclose(got32.double(), ref, atol=2e-4 * (K ** 0.5), rtol=1e-5), float((got32.double() - ref).abs().max())
     got16 = ops.linear_thin(a.to(DEV), w.to(DEV), BF16).cpu()
-    assert torch.equal(got16, got32.to(BF16))                          # one rounding at the end
+    if 64 < M <= 128 and K % 8 == 0:
+        # the float32 result of so many rows comes from the tiled kernel, the bfloat16 one from the kernel that shares
+        # up to 128 rows through LDS: sums in another order, so the rounding may fall the other way
+        assert torch.allclose(got16.double(), ref, atol=2e-4 * (K ** 0.5), rtol=2.0 ** -8)
+    else:
+        assert torch.equal(got16, got32.to(BF16))                      # one rounding at the end
 
 
 @pytest.mark.parametrize("M", [1, 8, 16])
@@ -54,14 +59,14 @@ def test_linear_thin_as_planes_of_partial_sums(ops, M, N, K, planes):
     assert ops.linear_thin(a.to(DEV), w.to(DEV), BF16, planes_ok=False).shape == (M, N)
 
 
-@pytest.mark.parametrize("M", [17, 40, 64])
+@pytest.mark.parametrize("M", [17, 40, 64, 65, 100, 128])
 @pytest.mark.parametrize("N,K,cut", [(4096, 12288, True), (4096, 4096, True), (6144, 4096, True), (1000, 3000, True),
                                      (24576, 4096, False), (4096, 1000, False), (300, 12296, True)])
-def test_linear_for_17_to_64_rows_as_planes_of_partial_sums(ops, M, N, K, cut):
+def test_linear_for_17_to_128_rows_as_planes_of_partial_sums(ops, M, N, K, cut):
     a, w = rand(M, K, seed=M, dtype=BF16), rand(N, K, seed=N + K, dtype=BF16)
     got = ops.linear_thin(a.to(DEV), w.to(DEV), F32, planes_ok=True).cpu()
     want = P.linear(a, w)
-    if cut:
+    if cut or (M > 64 and got.dim() == 3):          # (more than 64 rows go by in shorter steps of K, so a short K is cut too)
         assert got.dim() == 3 and 2 <= got.shape[0] <= 4 and got.shape[1:] == (M, N) and got.dtype == F32
         assert all(float(got[p].abs().max()) > 0 for p in range(got.shape[0]))       # no range of K is empty
         got = got.double().sum(0)
@@ -142,7 +147,7 @@ def test_linear_thin_orientation(ops):
     assert torch.equal(got, ref)
 
 
-@pytest.mark.parametrize("M", [1, 8, 20, 64])
+@pytest.mark.parametrize("M", [1, 8, 20, 64, 90, 128])
 @pytest.mark.parametrize("I,K", [(5, 16), (176, 80), (224, 96), (1536, 512), (4500, 2048), (300, 3000), (100, 6000), (2200, 5120),
                                  (40, 8192)])
 def test_linear_thin_gated(ops, M, I, K):
@@ -160,7 +165,10 @@ def test_linear_thin_gated(ops, M, I, K):
     swapped = u / (1 + torch.exp(-u)) * g
     assert not torch.allclose(got.double(), swapped, atol=1e-2) or I * M < 8
     got16 = ops.linear_thin(a.to(DEV), w.to(DEV), BF16, gated=True).cpu()
-    assert torch.equal(got16, got.to(BF16))
+    if M > 64:          # bfloat16 from the kernel for up to 128 rows, float32 from the tiled one: sums in another order
+        assert bool(((got16.double() - ref).abs() <= bound + 2.0 ** -8 * ref.abs()).all())
+    else:
+        assert torch.equal(got16, got.to(BF16))
 
 
 def test_linear_thin_is_the_same_bits_every_time_and_for_every_companion(ops):
