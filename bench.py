@@ -10,7 +10,7 @@ prefill of 2,048 tokens, the decode step's fraction of the HBM roofline, and dec
 ``points`` also holds (flat, every figure under a name of its own) the other workloads that the baseline names and
 the lengths at which other kernels matter, each with tokens a second, milliseconds and its fraction of the same
 roofline by the same formulas: decode at 128 sequences and at 8 sequences of 8,192 tokens, a prompt of 32,768
-tokens, the time to the first token of prompts of 64, 256 and 512 tokens (Qwen3-8B sizes); 16 prompts of unequal
+tokens, the time to the first token of prompts of 64, 128, 256 and 512 tokens (Qwen3-8B sizes); 16 prompts of unequal
 lengths drawn from 64..2,048 and 256 decode steps at Qwen3-14B sizes; 32 prompts of 4,096 tokens and 512 decode
 steps at Qwen3-32B sizes (the decode steps of these two scale with ``--steps``: twice and four times as many).
 ``--only 8b`` (or ``14b``, ``32b``, a comma-separated list) measures a part.
@@ -245,7 +245,9 @@ def prefill_kernel_table(engine, cfg, tokens: int) -> dict:
     work = {
         "qkv_proj": (each_layer(lambda i: layers[i].mixer.qkv(h)), 2.0 * tokens * (nh + 2 * nkv) * hd * H, mfma),
         "attention": (each_layer(lambda i: ops.attention_prefill(attn, kv.k[i], kv.v[i], kv.table_dev, seq_slot, seq_start, seq_new, cu,
-                                                                 tokens, nh, nkv, hd, hd ** -0.5, None)),
+                                                                 tokens, nh, nkv, hd, hd ** -0.5, None,
+                                                                 # as the attention part calls it: queries that carry the scale
+                                                                 q_prescaled=ops.prefill_q_scale(hd, bf16, hd ** -0.5) != 1.0)),
                       4.0 * nh * hd * tokens * (tokens + 1) / 2.0, mfma),
         "o_proj": (each_layer(lambda i: layers[i].mixer.out(attn)), 2.0 * tokens * nh * hd * H, mfma),
         "gate_up_proj": (each_layer(lambda i: layers[i].feed_forward.gate_up(h)), 2.0 * tokens * 2 * I * H, mfma),
@@ -335,6 +337,8 @@ def main(argv=None) -> int:
     ap.add_argument("--batch", type=int, default=BATCH)
     ap.add_argument("--no-points", action="store_true", help="only the headline: batch 8, and the prefill of 2,048 tokens")
     ap.add_argument("--only", default="8b,14b,32b", help="which sizes' points to measure (8b is always measured)")
+    ap.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS,
+                    help="tokens of the timed prompt (2,048 is the workload's; others serve profiles of longer prompts)")
     args = ap.parse_args(argv)
     if args.gpus != 1:
         print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not measured")
@@ -349,10 +353,11 @@ def main(argv=None) -> int:
     vocab = cfg["vocab_size"]
     room = CONTEXT + args.warmup + args.steps + 64
     LONG, LONG_CONTEXT, LONG_BATCH, MANY = 32768, 8192, 8, 128
+    prompt_tokens = args.prefill_tokens
     if args.no_points:
-        cache_tokens = args.batch * room + PREFILL_TOKENS + 64
+        cache_tokens = args.batch * room + prompt_tokens + 64
     else:
-        cache_tokens = max(MANY * room, LONG_BATCH * (LONG_CONTEXT + room), LONG + 64) + PREFILL_TOKENS + 64
+        cache_tokens = max(MANY * room, LONG_BATCH * (LONG_CONTEXT + room), LONG + 64) + prompt_tokens + 64
     t_load = time.perf_counter()
     engine = Engine.from_config(cfg, seed=0, dtype="bfloat16", max_tokens=cache_tokens, max_seqs=max(args.batch, MANY) + 1)
     torch.cuda.synchronize()
@@ -389,11 +394,11 @@ def main(argv=None) -> int:
     # The prompts last: a second of a prompt's large products back to back (the per-kernel table) leaves the chip at a
     # lower clock for some 0.2 s afterwards (the first 40 decode steps after it took 4.12 ms instead of 3.98), which
     # would be charged to the decode step if that were measured next.
-    prefill_ms = time_prefill(engine, PREFILL_TOKENS, vocab)
-    pf = prefill_flops(cfg, PREFILL_TOKENS)
-    prefill_kernels = prefill_kernel_table(engine, cfg, PREFILL_TOKENS)
+    prefill_ms = time_prefill(engine, prompt_tokens, vocab)
+    pf = prefill_flops(cfg, prompt_tokens)
+    prefill_kernels = prefill_kernel_table(engine, cfg, prompt_tokens)
     if not args.no_points:
-        for n in (64, 256, 512):             # time to the first token: one prompt, logits at its last place
+        for n in (64, 128, 256, 512):        # time to the first token: one prompt, logits at its last place
             points[f"ttft_{n}_ms"] = round(time_prefill(engine, n, vocab, repeats=5), 3)
         long_ms = time_prefill(engine, LONG, vocab, repeats=2)
         points["prefill_32768"] = round(LONG * 1000.0 / long_ms, 1)
@@ -425,8 +430,8 @@ def main(argv=None) -> int:
                    "rms_norm_eps": cfg["rms_norm_eps"], "tied_head": False,
                    # the cache is one pool of pages for all live sequences; a sequence may take all of it
                    "cache_tokens": cache_room,
-                   "prefill_tokens": PREFILL_TOKENS, "decode_steps": args.steps, "load_s": round(load_s, 1)},
-        "prefill": {"value": round(PREFILL_TOKENS * 1000.0 / prefill_ms, 1), "tokens": PREFILL_TOKENS,
+                   "prefill_tokens": prompt_tokens, "decode_steps": args.steps, "load_s": round(load_s, 1)},
+        "prefill": {"value": round(prompt_tokens * 1000.0 / prefill_ms, 1), "tokens": prompt_tokens,
                     "ms": round(prefill_ms, 3), "frac": round(pf / (prefill_ms * 1e-3) / PEAK_FLOPS["bf16"], 4),
                     # the step's dominant kernels alone (a launch for each layer, event-timed): us a layer, and the
                     # fraction of the matrix cores' (or, for the two memory-bound passes, of HBM's) peak
