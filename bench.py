@@ -239,15 +239,16 @@ def prefill_kernel_table(engine, cfg, tokens: int) -> dict:
     i32 = lambda xs: torch.tensor(xs, dtype=torch.int32, device=dev)
     seq_slot, seq_start, seq_new, cu = i32([slot]), i32([0]), i32([tokens]), i32([0, tokens])
     mfma, hbm = PEAK_FLOPS["bf16"], PEAK_HBM_GBS * 1e9
+    # as the attention part hands them over: queries that carry the scale where the kernel of this head size takes them so
+    q_scale = ops.prefill_q_scale(hd, bf16, hd ** -0.5)
+    queries = (attn.float() * q_scale).to(bf16)
 
     def each_layer(fn):
         return lambda: [fn(i) for i in range(L)]
     work = {
         "qkv_proj": (each_layer(lambda i: layers[i].mixer.qkv(h)), 2.0 * tokens * (nh + 2 * nkv) * hd * H, mfma),
-        "attention": (each_layer(lambda i: ops.attention_prefill(attn, kv.k[i], kv.v[i], kv.table_dev, seq_slot, seq_start, seq_new, cu,
-                                                                 tokens, nh, nkv, hd, hd ** -0.5, None,
-                                                                 # as the attention part calls it: queries that carry the scale
-                                                                 q_prescaled=ops.prefill_q_scale(hd, bf16, hd ** -0.5) != 1.0)),
+        "attention": (each_layer(lambda i: ops.attention_prefill(queries, kv.k[i], kv.v[i], kv.table_dev, seq_slot, seq_start, seq_new, cu,
+                                                                 tokens, nh, nkv, hd, hd ** -0.5, None, q_prescaled=q_scale != 1.0)),
                       4.0 * nh * hd * tokens * (tokens + 1) / 2.0, mfma),
         "o_proj": (each_layer(lambda i: layers[i].mixer.out(attn)), 2.0 * tokens * nh * hd * H, mfma),
         "gate_up_proj": (each_layer(lambda i: layers[i].feed_forward.gate_up(h)), 2.0 * tokens * 2 * I * H, mfma),
