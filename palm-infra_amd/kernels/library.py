@@ -35,7 +35,7 @@ FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-fno-gpu-rdc",
 
 CORE_SOURCES = ["elementwise.hip", "linear.hip", "rope_store.hip", "attention_simple.hip", "sampling.hip",
                 "linear_mfma.hip", "linear_wide.hip", "linear_wide_store_32.hip", "linear_wide_store_64.hip",
-                "linear_wide_gated_32.hip", "linear_wide_gated_64.hip", "linear_wide_store_128.hip", "linear_wide_gated_128.hip",
+                "linear_wide_gated_32.hip", "linear_wide_gated_64.hip", "linear_wide_store_128.hip", "linear_wide_gated_128.hip", "linear_mid.hip",
                 "weights_prep.hip", "linear_tile.hip"]
 ATTENTION_SOURCES = ["attention_mfma.hip"]
 HEADERS = ["common.h", "mfma.h", "linear_wide.h", "attention_api.h"]

@@ -40,6 +40,9 @@ _SIGNATURES = {
     "palm_linear_wide": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int],
     "palm_linear_wide_parts": [c_int, c_int, c_int, c_int],
     "palm_linear_wide_blocks": [c_int, c_int, c_int, c_int, c_int],
+    "palm_linear_mid": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int],
+    "palm_linear_mid_parts": [c_int, c_int, c_int, c_int],
+    "palm_linear_mid_blocks": [c_int, c_int, c_int, c_int, c_int],
     "palm_linear_tile": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int,
                          c_float, c_void_p, c_void_p, c_void_p],
     "palm_linear_tile_pieces": [c_int],
@@ -388,6 +391,49 @@ def wide_pays(M: int, N: int, K: int, gated: bool = False, planes_ok: bool = Fal
     recorded)."""
     return THIN_TOKENS < M <= WIDE_TOKENS and core().palm_linear_wide_blocks(
         M, N, K, 1 if gated else 0, 1 if planes_ok else 0) >= WIDE_MIN_BLOCKS
+
+
+MID_TOKENS = 256      # rows of one block of the kernel for short prompts
+MID_CHUNK = 64        # which walks over K in steps of this many
+
+
+def mid_pays(M: int, N: int, K: int, planes_ok: bool = False) -> bool:
+    """Whether the kernel for 129 to 256 rows beats the library for this product: where the weight rows are so few
+    that it cuts K into planes of partial sums (which the reader must take) to fill the chip; the library's tiles
+    leave compute units idle there.  Measured at Qwen3-8B's shapes (us, own against library): with 256 rows q/k/v 29
+    and 40, output projection 23 and 24, down 46 and 53; with 129 rows (library at 192) 23 and 34, 18 and 33, 39 and
+    88; the planes cost their readers about 4 us each.  Not a product with weight rows enough for all compute units
+    (gate/up at 256 rows: 70 against 65, gated 79 against 65 and the activation's pass of 8; every block then reads
+    all rows again for 96 weight rows, and the way from L2 into a compute unit, 60 to 80 GB/s when all of them pull, is
+    as long as the arithmetic), and not more than 256 rows, where it ties (q/k/v 40 and 37, output projection 32 and
+    30, down 78 and 80 at 512 rows)."""
+    return (planes_ok and WIDE_TOKENS < M <= MID_TOKENS and K % MID_CHUNK == 0
+            and core().palm_linear_mid_parts(M, N, K, 0) > 1
+            and core().palm_linear_mid_blocks(M, N, K, 0, 1) >= WIDE_MIN_BLOCKS)
+
+
+def linear_mid(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, gated: bool = False,
+               planes_ok: bool = False) -> torch.Tensor:
+    """bfloat16 a [M, K] . w [N, K]^T for some hundred rows, K a multiple of 64: both operands go through rings in
+    LDS, a block of four waves holding 256 rows against 96 or 64 weight rows.  The result is [M, N] in bfloat16 or
+    float32 ([M, N/2] bfloat16 when ``gated``), or, if ``planes_ok`` and the weight rows are few, float32 planes
+    [P, M, N] over ranges of K."""
+    _dev("linear_mid", a, w)
+    _need(a.dtype == BF16 and w.dtype == BF16 and a.dim() == 2 and w.dim() == 2 and a.shape[1] == w.shape[1]
+          and a.is_contiguous() and w.is_contiguous(),
+          f"linear_mid: a {tuple(a.shape)} {a.dtype} and w {tuple(w.shape)} {w.dtype} (bfloat16, one inner size)")
+    M, K = a.shape
+    N = w.shape[0]
+    _need(K % MID_CHUNK == 0, f"linear_mid: K = {K} is no multiple of {MID_CHUNK}")
+    _need(not gated or (N % 2 == 0 and out_dtype == BF16), "linear_mid: a gated product has an even number of weight rows and a bfloat16 result")
+    planes = core().palm_linear_mid_parts(M, N, K, 0) if planes_ok and not gated else 1
+    if planes > 1:
+        out = torch.empty((planes, M, N), dtype=F32, device=a.device)
+    else:
+        out = torch.empty((M, N // 2 if gated else N), dtype=out_dtype, device=a.device)
+    library.call(core(), "palm_linear_mid", _stream(), _p(a), _p(w), _p(out), _code(out, "linear_mid out"), M, N, K,
+                 1 if gated else 0, planes)
+    return out
 
 
 def thin_serves(a: torch.Tensor, w: torch.Tensor) -> bool:

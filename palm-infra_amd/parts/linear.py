@@ -2,7 +2,9 @@
 
   float32 run, or a 32-bit weight under bfloat16 activations   the exact FMA kernel
   bfloat16 x bfloat16, up to 16 rows (decode)                   the matrix-core kernel for thin products
-  bfloat16 x bfloat16, 17 to 64 rows (large decode batches)     the matrix-core kernel that shares the rows through LDS
+  bfloat16 x bfloat16, 17 to 128 rows (large decode batches)    the matrix-core kernel that shares the rows through LDS
+  bfloat16 x bfloat16, 129 to 256 rows (short prompts)          the kernel that brings both operands through rings in
+                                                                LDS, where it beats the library (ops.mid_pays)
   bfloat16 x bfloat16, many rows (prompts)                      the BLAS library, as the reference's GPU path
                                                                 does for its products (engine/cuda_matmul.cu:245-260)
 
@@ -17,9 +19,10 @@ import torch
 from ..kernels import ops
 from .residual import Prenormed
 
-# Up to this many rows the kernel that streams the weight past one block of 16 rows serves; from there to 64 rows
+# Up to this many rows the kernel that streams the weight past one block of 16 rows serves; from there to 128 rows
 # the kernel that shares the rows through LDS, where it has blocks enough to fill the chip (ops.wide_pays), and
-# for every product with a float32 result; else the library.
+# for every product with a float32 result; from 129 to 256 rows the kernel with rings in LDS where it pays
+# (ops.mid_pays); else the library.
 THIN_ROWS = 16
 
 
@@ -66,6 +69,8 @@ class Linear:
             if (x.shape[0] <= THIN_ROWS or out_dtype != torch.bfloat16
                     or (ops.thin_serves(x, w) and ops.wide_pays(x.shape[0], self.out_features, self.in_features, planes_ok=planes_ok))):
                 return ops.linear_thin(x, w, out_dtype, planes_ok=planes_ok)
+            if x.is_contiguous() and ops.mid_pays(x.shape[0], self.out_features, self.in_features, planes_ok=planes_ok):
+                return ops.linear_mid(x, w, out_dtype, planes_ok=planes_ok)
             return ops.linear_library(x, w)
         return ops.linear_exact(x, w, out_dtype)
 

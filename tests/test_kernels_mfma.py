@@ -190,6 +190,100 @@ def test_linear_thin_falls_back_when_rows_do_not_start_on_16_bytes(ops):
                           P.linear(a32, rand(9, 16, seed=2, dtype=F32)), atol=1e-4)
 
 
+# ---- the product for some hundred rows, both operands through rings in LDS -----------------------------
+
+@pytest.mark.parametrize("M", [1, 129, 200, 256, 257, 300, 512, 515])
+@pytest.mark.parametrize("N,K", [(96, 64), (7, 128), (1000, 192), (515, 320), (4096, 4096), (300, 12288), (6144, 1024), (8200, 448)])
+def test_linear_mid_against_the_plain_product(ops, M, N, K):
+    a, w = rand(M, K, seed=M + K), rand(N, K, seed=N, scale=0.5)
+    ref = P.linear(a, w)
+    got32 = ops.linear_mid(a.to(DEV), w.to(DEV), F32).cpu()
+    assert got32.shape == (M, N)
+    assert torch.allclose(got32.double(), ref, atol=2e-4 * (K ** 0.5), rtol=1e-5), float((got32.double() - ref).abs().max())
+    got16 = ops.linear_mid(a.to(DEV), w.to(DEV), BF16).cpu()
+    assert torch.equal(got16, got32.to(BF16))                          # one rounding at the end
+
+
+@pytest.mark.parametrize("M", [129, 256, 300])
+@pytest.mark.parametrize("N,K,cut", [(4096, 12288, True), (4096, 4096, True), (6144, 4096, True), (1000, 3072, True),
+                                     (24576, 4096, False), (4096, 448, False)])
+def test_linear_mid_as_planes_of_partial_sums(ops, M, N, K, cut):
+    a, w = rand(M, K, seed=M), rand(N, K, seed=N + K, scale=0.5)
+    got = ops.linear_mid(a.to(DEV), w.to(DEV), F32, planes_ok=True).cpu()
+    want = P.linear(a, w)
+    parts = ops.core().palm_linear_mid_parts(M, N, K, 0)
+    assert parts > 1 if cut else parts == 1
+    if parts > 1:
+        assert got.shape == (parts, M, N) and parts <= 4 and got.dtype == F32
+        assert all(float(got[p].abs().max()) > 0 for p in range(parts))              # no range of K is empty
+        got = got.double().sum(0)
+    else:
+        assert got.shape == (M, N)
+    assert torch.allclose(got.double(), want, atol=2e-4 * (K ** 0.5), rtol=1e-5)
+    assert ops.linear_mid(a.to(DEV), w.to(DEV), BF16, planes_ok=False).shape == (M, N)
+
+
+def test_linear_mid_orientation_and_every_k_once(ops):
+    M, N, K = 300, 520, 448
+    a, w = torch.zeros(M, K, dtype=BF16), torch.zeros(N, K, dtype=BF16)
+    a[3] = (torch.arange(K) % 7).to(BF16)
+    a[299, 447] = 3.0
+    w[29] = 1.0
+    w[511, 100] = 2.0
+    w[519, 447] = 5.0
+    got = ops.linear_mid(a.to(DEV), w.to(DEV), F32).cpu()
+    ref = torch.zeros(M, N)
+    ref[3, 29] = float((torch.arange(K) % 7).sum())
+    ref[3, 511] = 2.0 * (100 % 7)
+    ref[3, 519] = 5.0 * (447 % 7)
+    ref[299, 29] = 3.0
+    ref[299, 519] = 15.0
+    assert torch.equal(got, ref)
+
+
+@pytest.mark.parametrize("M", [129, 256, 300])
+@pytest.mark.parametrize("I,K", [(128, 64), (176, 128), (1536, 512), (4500, 2048), (301, 3008)])
+def test_linear_mid_gated(ops, M, I, K):
+    a, w = rand(M, K, seed=M), rand(2 * I, K, seed=I, scale=0.3)
+    g, u = P.linear(a, w[:I]), P.linear(a, w[I:])
+    ref = g / (1 + torch.exp(-g)) * u
+    got = ops.linear_mid(a.to(DEV), w.to(DEV), BF16, gated=True).cpu()
+    assert got.shape == (M, I)
+    scale = float(ref.abs().max())
+    assert torch.allclose(got.double(), ref, atol=2.0 ** -8 * scale), float((got.double() - ref).abs().max()) / scale
+    swapped = u / (1 + torch.exp(-u)) * g
+    assert not torch.allclose(got.double(), swapped, atol=1e-2 * scale)
+
+
+def test_linear_mid_refuses_what_it_does_not_serve(ops):
+    from palm_infra_amd.kernels.library import KernelError
+    a, w = rand(130, 72).to(DEV), rand(96, 72).to(DEV)
+    with pytest.raises((KernelError, ValueError), match="64"):
+        ops.linear_mid(a, w, BF16)
+    assert not ops.mid_pays(130, 96, 72) and not ops.mid_pays(128, 4096, 4096, planes_ok=True)
+    assert not ops.mid_pays(300, 4096, 4096, planes_ok=True)
+    assert ops.mid_pays(200, 4096, 4096, planes_ok=True) and not ops.mid_pays(200, 4096, 4096, planes_ok=False)
+    assert not ops.mid_pays(200, 24576, 4096, planes_ok=True)           # weight rows enough: no planes, the library's
+
+
+def test_a_short_prompts_projections_take_the_kernel_with_rings(ops, monkeypatch):
+    """The linear part sends bfloat16 products of 129 to 256 rows to this kernel where its blocks fill the chip, and to
+    the library otherwise; either way the result is the plain product."""
+    from palm_infra_amd.parts.linear import Linear
+    calls = []
+    real = ops.linear_mid
+    monkeypatch.setattr(ops, "linear_mid", lambda *a, **k: (calls.append(a[0].shape[0]), real(*a, **k))[1])
+    w = rand(6144, 1024, seed=1, scale=0.5)
+    lin = Linear(w.to(DEV))
+    for M, expect in ((200, True), (256, True), (128, False), (257, False)):
+        x = rand(M, 1024, seed=M)
+        calls.clear()
+        got = lin(x.to(DEV), planes_ok=True)
+        assert bool(calls) == expect, (M, calls)
+        got = got.double().sum(0) if got.dim() == 3 else got.double()
+        assert torch.allclose(got.cpu(), P.linear(x, w), atol=2e-4 * 32 + 2.0 ** -8 * float(P.linear(x, w).abs().max()))
+
+
 # ---- the tiled product for many rows -----------------------------------------------------------------
 
 @pytest.mark.parametrize("M", [65, 128, 130, 257, 700])
