@@ -14,13 +14,10 @@
 // strips, and MFMA 16x16x32 consume them.  Several super-steps are loaded before any is used, which is what
 // keeps enough bytes in flight to fill the memory pipe with only one or two blocks on a compute unit.
 // RT = 2 halves the activation reads per weight byte but was measured slower; RT = 1 is what runs.
-#include "mfma.h"
+#include "linear_thin.h"
 
+#include <cstdlib>
 #include <type_traits>
-
-enum ThinEpilogue : int { EPI_STORE = 0, EPI_SWIGLU = 1 };
-
-constexpr int SUPER_K = 128;
 
 template <int MB, int NW, int U, int RT, typename TC, int EPI>
 __global__ __launch_bounds__(NW * WAVE) void linear_thin_kernel(const bf16_t* __restrict__ A,
@@ -141,25 +138,8 @@ static void launch_thin(hipStream_t stream, const void* a, const void* w, void* 
 // blockIdx.y of a [parts, M, N] float32 result; whoever reads the result adds the planes in their order (the
 // norm that follows adds them to the residual stream), so the sum is the same bits every time.
 //
-// The norm around a product can be folded into it (RowNorm), which saves the norm's own kernel in a decode
-// step.  RMSNorm is y = x * f * w with one factor f = 1 / sqrt(mean(x^2) + eps) for the row, so
-// (x * f * w) . W^T = f * ((x * w) . W^T): a product whose activations are x * w, not yet multiplied by f, only
-// has to multiply its result rows by f, and f needs nothing but the row's sum of squares.
-//   out side: the product is a branch's output d.  The block that owns a strip of 16 features adds d to the
-//             residual stream (x += d, each element by exactly one thread), stores x * w_out rounded to
-//             bfloat16 as the next product's activations, and the strip's share of each row's sum of squares
-//             in ss_out[row * strips + strip].
-//   in side:  every block adds up the pieces ss_in[row * pieces + piece] in a fixed order, and multiplies its
-//             results by f(row) before the epilogue.
-struct RowNorm {
-    const float* ss_in;      // [M, pieces_in] or null (a row's pieces side by side: 32 lanes read them in one go)
-    int pieces_in;
-    float eps_in;
-    int width_in;            // the row length the mean is over
-    float* resid;            // [M, N] float32, updated; or null
-    const float* w_out;      // [N]
-    float* ss_out;           // [M, strips]
-};
+// The norm around a product can be folded into it (RowNorm, linear_thin.h), which saves the norm's own kernel in a
+// decode step.
 
 // Waves that run at once in the usual launch: 8 on each of 256 compute units, one block of eight waves each.  Two
 // blocks a unit (4096) were the rule once: measured at 8 rows, the gated product of 24576 x 4096 38.2 us against 36.6
@@ -411,6 +391,10 @@ static void dispatch_thin(hipStream_t stream, const void* a, const void* w, void
     const bool folded = norm.ss_in || norm.resid;              // only the stream kernel folds a norm in
     if (M <= 16 && (deep || folded)) {
         const int per_wave = stream_steps(n_super, parts);
+        static const bool ring = !getenv("PALM_NO_RING");
+        if (ring && stream_waves(n_super) == 8 &&
+            launch_linear_ring(stream, a, w, c, sizeof(TC) == 2 ? PALM_BF16 : PALM_F32, M, N, K, EPI, parts, per_wave, norm))
+            return;
         if (stream_waves(n_super) == 4) dispatch_stream<4, TC, EPI>(stream, a, w, c, M, N, K, parts, norm, per_wave);
         else dispatch_stream<8, TC, EPI>(stream, a, w, c, M, N, K, parts, norm, per_wave);
         return;

@@ -34,11 +34,11 @@ FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-fno-gpu-rdc",
          "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option"]
 
 CORE_SOURCES = ["elementwise.hip", "linear.hip", "rope_store.hip", "attention_simple.hip", "sampling.hip",
-                "linear_mfma.hip", "linear_wide.hip", "linear_wide_store_32.hip", "linear_wide_store_64.hip",
+                "linear_mfma.hip", "linear_ring.hip", "linear_wide.hip", "linear_wide_store_32.hip", "linear_wide_store_64.hip",
                 "linear_wide_gated_32.hip", "linear_wide_gated_64.hip", "linear_wide_store_128.hip", "linear_wide_gated_128.hip", "linear_mid.hip",
                 "weights_prep.hip", "linear_tile.hip"]
 ATTENTION_SOURCES = ["attention_mfma.hip"]
-HEADERS = ["common.h", "mfma.h", "linear_wide.h", "attention_api.h"]
+HEADERS = ["common.h", "mfma.h", "linear_thin.h", "linear_wide.h", "attention_api.h"]
 
 
 class KernelBuildError(RuntimeError):
