@@ -16,7 +16,6 @@
 // RT = 2 halves the activation reads per weight byte but was measured slower; RT = 1 is what runs.
 #include "linear_thin.h"
 
-#include <cstdlib>
 #include <type_traits>
 
 template <int MB, int NW, int U, int RT, typename TC, int EPI>
@@ -126,13 +125,13 @@ static void launch_thin(hipStream_t stream, const void* a, const void* w, void* 
 // the one U ahead into the same registers, so the memory pipe never drains between a block's first and last
 // byte; only the last U steps of a block ask for nothing.  With TREG > 0 a wave's share of the activations
 // (super-steps wave, wave + NW, ..., TREG of them, the same for every strip) is read once and stays in
-// registers; with TREG == 0 it is read again beside every weight read.  At eight rows the register form is
-// what brings the gated product from 45 to 36 us and the head from 260 to 212 us: an activation read costs
+// registers; with TREG == 0 it is read again beside every weight read: an activation read costs
 // the cache path as much as a weight read although it brings nothing new.
 // T: steps a wave makes for one strip, a multiple of U; steps beyond K read the row's start and count as zeros
-// (EXACT says there are none, and then nothing is checked: 3% of a decode step at Qwen3-8B's sizes).
-// NW: waves a block, 8, or 4 for a K of fewer than 32 super-steps, which eight waves would share out badly
-// (K = 2560: 20 super-steps are 3 steps for each of eight waves with 12 of 32 turns idle, but 5 for each of four).
+// (EXACT says there are none, and then nothing is checked).
+// NW: waves a block.  This kernel runs with 4, for a K of fewer than 32 super-steps, which eight waves would share
+// out badly (K = 2560: 20 super-steps are 3 steps for each of eight waves with 12 of 32 turns idle, but 5 for each of
+// four); from 32 super-steps on the stream is linear_ring.hip's, eight waves a block, whose weights cross LDS.
 // Few strips and a long K (an output projection: 256 strips) leave most of the chip without work.  Then K is
 // cut into `parts` ranges, blockIdx.y names the range, and the block writes its partial sums to plane
 // blockIdx.y of a [parts, M, N] float32 result; whoever reads the result adds the planes in their order (the
@@ -391,12 +390,11 @@ static void dispatch_thin(hipStream_t stream, const void* a, const void* w, void
     const bool folded = norm.ss_in || norm.resid;              // only the stream kernel folds a norm in
     if (M <= 16 && (deep || folded)) {
         const int per_wave = stream_steps(n_super, parts);
-        static const bool ring = !getenv("PALM_NO_RING");
-        if (ring && stream_waves(n_super) == 8 &&
-            launch_linear_ring(stream, a, w, c, sizeof(TC) == 2 ? PALM_BF16 : PALM_F32, M, N, K, EPI, parts, per_wave, norm))
-            return;
-        if (stream_waves(n_super) == 4) dispatch_stream<4, TC, EPI>(stream, a, w, c, M, N, K, parts, norm, per_wave);
-        else dispatch_stream<8, TC, EPI>(stream, a, w, c, M, N, K, parts, norm, per_wave);
+        // eight waves: the stream whose weights cross LDS; four (a short K): the one that reads them into registers
+        if (stream_waves(n_super) == 8)
+            launch_linear_ring(stream, a, w, c, sizeof(TC) == 2 ? PALM_BF16 : PALM_F32, M, N, K, EPI, parts, per_wave, norm);
+        else
+            dispatch_stream<4, TC, EPI>(stream, a, w, c, M, N, K, parts, norm, per_wave);
         return;
     }
     // a short K: one strip a block, four waves (two strips a block, RT = 2, were measured slower at every size)
@@ -424,6 +422,8 @@ PALM_API int palm_linear_thin(hipStream_t stream, const void* a, const void* w, 
                "linear_thin: %d partial planes are not served for M=%d N=%d K=%d, this epilogue and result type", parts, M, N, K);
     PALM_CHECK(M >= 0 && N > 0 && K > 0, "linear_thin: M=%d N=%d K=%d", M, N, K);
     PALM_CHECK(K % 8 == 0, "linear_thin: K = %d is not a multiple of 8 (rows must start on 16 bytes)", K);
+    // a lane's place among a strip's rows, in the activations and in the residual stream is a 32-bit byte offset
+    PALM_CHECK((double)17 * K * 2 < 4.0e9 && (double)16 * N * 4 < 4.0e9, "linear_thin: N=%d K=%d is beyond 32-bit offsets", N, K);
     PALM_CHECK(epilogue == EPI_STORE || epilogue == EPI_SWIGLU, "linear_thin: epilogue %d", epilogue);
     PALM_CHECK(epilogue != EPI_SWIGLU || N % 2 == 0, "linear_thin: a gated product needs an even N, got %d", N);
     PALM_CHECK(((uintptr_t)a | (uintptr_t)w) % 16 == 0, "linear_thin: operands must be 16-byte aligned");

@@ -86,14 +86,24 @@ __global__ __launch_bounds__(RING_THREADS) void linear_ring_kernel(const bf16_t*
     // (lane % 8) ^ (lane / 8) of the line's eight; instruction i brings rows 8 (i % 2) .., k-values 64 (i / 2) ..
     const int row8 = lane / 8;
     const int piece = (lane % 8) ^ row8;
-    constexpr int STRIP_ROWS = EPI == EPI_SWIGLU ? 8 : 16;  // output features of a strip
-    // byte offsets of the lane's two rows from the strip's first row; rows beyond the last read the last
+    // Where a strip's rows start (the same in every lane: scalar registers), its first eight and its second eight (with
+    // the gated epilogue eight gate rows and the eight up rows that belong to them), and a lane's row among the eight
+    // as a byte offset; rows beyond the last read the last.
+    auto bases_of = [&](int strip, const char* (&base)[2]) __attribute__((always_inline)) {
+        if (EPI == EPI_SWIGLU) {
+            base[0] = reinterpret_cast<const char*>(W + (size_t)strip * 8 * K);
+            base[1] = reinterpret_cast<const char*>(W + ((size_t)inter + (size_t)strip * 8) * K);
+        } else {
+            base[0] = reinterpret_cast<const char*>(W + (size_t)strip * 16 * K);
+            base[1] = reinterpret_cast<const char*>(W + (size_t)min(strip * 16 + 8, N - 1) * K);
+        }
+    };
     auto rows_of = [&](int strip, uint32_t (&off)[2]) __attribute__((always_inline)) {
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             int rel;
-            if (EPI == EPI_SWIGLU) rel = (h ? inter : 0) + min(row8, inter - 1 - strip * 8);          // gate rows, then their up rows
-            else rel = min(h * 8 + row8, N - 1 - strip * 16);
+            if (EPI == EPI_SWIGLU) rel = min(row8, inter - 1 - strip * 8);
+            else rel = min(row8, max(0, N - 1 - min(strip * 16 + 8 * h, N - 1)));
             off[h] = (uint32_t)rel * (uint32_t)K * 2u;
         }
     };
@@ -110,8 +120,9 @@ __global__ __launch_bounds__(RING_THREADS) void linear_ring_kernel(const bf16_t*
     const int total = my_strips * T;
     int n_asked = 0, n_used = 0;
     int ask_strip = blockIdx.x, ask_t = 0;
-    const char* ask_base = reinterpret_cast<const char*>(W + (size_t)ask_strip * STRIP_ROWS * K);
+    const char* ask_base[2];
     uint32_t w_off[2];
+    bases_of(ask_strip, ask_base);
     rows_of(ask_strip, w_off);
     const uint32_t ring0 = ring_lds_address(ring) + wave * (U * SLOT);
     auto ask = [&]() __attribute__((always_inline)) {
@@ -123,7 +134,7 @@ __global__ __launch_bounds__(RING_THREADS) void linear_ring_kernel(const bf16_t*
             // K is a multiple of 8: a piece is whole or absent; an absent one reads the row's start and counts as zeros
             const bool ok = EXACT || k0 + (i / 2) * 64 + piece * 8 < K;
             const uint32_t in_row = ok ? (uint32_t)(k0 * 2 + (i / 2) * 128 + piece * 16) : 0u;
-            ring_load_16(ask_base, w_off[i % 2] + in_row, to + i * 1024);
+            ring_load_16(ask_base[i % 2], w_off[i % 2] + in_row, to + i * 1024);
             if (!AREG) ring_load_16(A, x_off[i % 2] + in_row, to + 4096 + i * 1024);
         }
         ++n_asked;
@@ -131,7 +142,7 @@ __global__ __launch_bounds__(RING_THREADS) void linear_ring_kernel(const bf16_t*
             ask_t = 0;
             ask_strip += gridDim.x;
             const int s = min(ask_strip, n_strips - 1);
-            ask_base = reinterpret_cast<const char*>(W + (size_t)s * STRIP_ROWS * K);
+            bases_of(s, ask_base);
             rows_of(s, w_off);
         }
     };
@@ -299,11 +310,8 @@ static void dispatch_ring(hipStream_t stream, const void* a, const void* w, void
     else launch_ring<2, 0, TC, EPI>(stream, a, w, c, M, N, K, parts, steps, norm);
 }
 
-bool launch_linear_ring(hipStream_t stream, const void* a, const void* w, void* c, int c_dtype, int M, int N, int K,
+void launch_linear_ring(hipStream_t stream, const void* a, const void* w, void* c, int c_dtype, int M, int N, int K,
                         int epilogue, int parts, int steps, const RowNorm& norm) {
-    // a lane's place in its strip's rows, in the activations and in the residual stream is a 32-bit byte offset
-    if ((double)(N / 2 + 16) * K * 2 >= 4.0e9 || (double)16 * K * 2 >= 4.0e9 || (double)16 * N * 4 >= 4.0e9) return false;
-    if (M < 1 || M > 16 || K % 8 != 0 || steps < 1 || parts < 1) return false;
     if (epilogue == EPI_SWIGLU) {
         if (c_dtype == PALM_BF16) dispatch_ring<bf16_t, EPI_SWIGLU>(stream, a, w, c, M, N, K, 1, steps, norm);
         else dispatch_ring<float, EPI_SWIGLU>(stream, a, w, c, M, N, K, 1, steps, norm);
@@ -311,5 +319,4 @@ bool launch_linear_ring(hipStream_t stream, const void* a, const void* w, void* 
         if (c_dtype == PALM_BF16) dispatch_ring<bf16_t, EPI_STORE>(stream, a, w, c, M, N, K, parts, steps, norm);
         else dispatch_ring<float, EPI_STORE>(stream, a, w, c, M, N, K, parts, steps, norm);
     }
-    return true;
 }

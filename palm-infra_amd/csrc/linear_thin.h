@@ -27,8 +27,9 @@ struct RowNorm {
     float* ss_out;           // [M, strips]
 };
 
-// The stream of eight waves a block whose weights cross LDS (linear_ring.hip).  steps: super-steps a wave makes for
-// one strip; parts: ranges of K (planes of the result).  False if it does not serve the product (the caller then
-// takes the kernel that reads into registers).
-bool launch_linear_ring(hipStream_t stream, const void* a, const void* w, void* c, int c_dtype, int M, int N, int K,
+// The stream of eight waves a block whose weights cross LDS (linear_ring.hip), for M <= 16 rows and K a multiple of 8.
+// steps: super-steps a wave makes for one strip; parts: ranges of K (planes of the result).  A lane's place among its
+// strip's rows, in the activations and in the residual stream is a 32-bit byte offset: 17 K and 16 N elements, which
+// the entry point checks.
+void launch_linear_ring(hipStream_t stream, const void* a, const void* w, void* c, int c_dtype, int M, int N, int K,
                         int epilogue, int parts, int steps, const RowNorm& norm);
