@@ -77,7 +77,7 @@ def test_linear_for_17_to_128_rows_as_planes_of_partial_sums(ops, M, N, K, cut):
 
 
 @pytest.mark.parametrize("M", [1, 5, 16])
-@pytest.mark.parametrize("N,K", [(80, 64), (4096, 4096), (1000, 1096), (515, 12288), (8200, 2048)])
+@pytest.mark.parametrize("N,K", [(80, 64), (4096, 4096), (1000, 1096), (515, 12288), (8200, 2048), (5120, 5120), (8200, 4224)])
 def test_linear_thin_into_the_residual_stream_and_on_with_the_row_factor(ops, M, N, K):
     """A product that adds its result to the residual stream and leaves the next norm's output but for the row
     factor; then a product (plain, in planes, gated) that takes such rows: together they are
