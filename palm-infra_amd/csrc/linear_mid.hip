@@ -1,26 +1,28 @@
-// C[M, N] = A[M, K] . W[N, K]^T for some hundred rows (prompts of 129 to 512 tokens): bfloat16 on the matrix cores,
-// 32-bit accumulation.  Too many rows for a wave to keep a strip of weights against all of them in registers (the
-// kernels for up to 128 rows), too few for the tiles of thousands of rows that a BLAS library is tuned for: the
-// weights (some tens to hundreds of MB) pass once, from HBM, and must not wait; the rows (a few MB) are read again by
-// every block, from L2; and the arithmetic is about as long as the weights' passage.
+// C[M, N] = A[M, K] . W[N, K]^T for 33 to some hundred rows (decode steps of many sequences, short prompts): bfloat16
+// on the matrix cores, 32-bit accumulation.  Too many rows for a wave to keep a strip of weights against all of them in
+// registers, too few for the tiles of thousands of rows that a BLAS library is tuned for: the weights (some tens to
+// hundreds of MB) pass once, from HBM, and must not wait; the rows (up to a few MB) are read again by every block,
+// from L2.
 //
-// A block of four waves owns 256 rows (all of them, for up to 256; more rows are more blocks beside it, numbered so
-// that the blocks that share weights run on one die at about the same time) and TN weight rows (96, or 64 where 96
-// would leave compute units without a block), and a range of K (cut in up to four where the weight rows are few; the
-// ranges' partial sums are float32 planes that the reader adds, as for the other kernels).  K goes by in chunks of 64.
-// Both operands of a chunk go from memory straight into LDS (global_load_lds: no registers, no write instruction),
-// each through a ring of its own: three chunks of rows (32 KB each; they come from L2), five chunks of weights (12 KB
-// each; they come from HBM and need the longer lead), 156 KB of the 160 KB a compute unit has.  Every lane's loads
-// are the same on every pass of the loop (beyond the range's end the last chunk is asked for once more, into a slot
-// nobody reads any more), so the wait for "this chunk has landed" is a constant number of younger loads, and the
-// compiler, which does not see the loads (they are written in assembly), adds no wait of its own.
+// A block of four waves owns R rows (64, 128 or 256: all of them, for up to 256; more rows are more blocks beside it,
+// numbered so that the blocks that share weights run on one die at about the same time) and TN weight rows (128, 96
+// or 64: the most that still gives every compute unit a block), and a range of K (cut in up to four where the weight
+// rows are few; the ranges' partial sums are float32 planes that the reader adds, as for the other kernels).  K goes
+// by in chunks of 64.  Both operands of a chunk go from memory straight into LDS (global_load_lds: no registers, no
+// write instruction, and every instruction brings eight whole 128-byte lines, which is what the vector cache takes
+// at its full rate), each through a ring of its own: three chunks of rows (8 to 32 KB each; they come from L2), five
+// chunks of weights (8 to 16 KB each; they come from HBM and need the longer lead), up to 156 KB of the 160 KB a
+// compute unit has.  Every lane's loads are the same on every pass of the loop (beyond the range's end the last chunk
+// is asked for once more, into a slot nobody reads any more), so the wait for "this chunk has landed" is a constant
+// number of younger loads, and the compiler, which does not see the loads (they are written in assembly), adds no
+// wait of its own.
 //
-// A wave multiplies its 64 rows with the block's weight rows: MFMA 32x32x16 with the weights as the first operand,
-// so that a lane ends up with four neighbouring features of one token, which leave in one store; 2 x 3 (or 2 x 2)
-// tiles of 32 x 32, 96 accumulator registers.  One barrier a chunk, placed before the chunk's last step of k: the
-// first fragments of the next chunk are then read from LDS while that step's matrix instructions run.  Rows of LDS
-// are 128 bytes, their eight 16-byte pieces permuted by the row's number so that the lanes LDS serves together hit
-// different banks.
+// A wave multiplies its rows (64 of 256, 32 of 128, or 32 of 64 against half of the weight rows) with the block's
+// weight rows: MFMA 32x32x16 with the weights as the first operand, so that a lane ends up with four neighbouring
+// features of one token, which leave in one store; up to 2 x 3 tiles of 32 x 32, 96 accumulator registers.  One
+// barrier a chunk, placed before the chunk's last step of k: the first fragments of the next chunk are then read from
+// LDS while that step's matrix instructions run.  Rows of LDS are 128 bytes, their eight 16-byte pieces permuted by
+// the row's number so that the lanes LDS serves together hit different banks.
 // With the gated epilogue (out = silu(gate) * up, engine/cuda_ops.cu:100-112) a tile of 32 weight rows is sixteen
 // gate rows and the sixteen up rows that belong to them, which one lane then holds side by side.
 #include "mfma.h"
@@ -29,14 +31,14 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 enum MidEpilogue : int { MID_STORE = 0, MID_SWIGLU = 1 };
 
-constexpr int MID_ROWS = 256;                   // rows of A a block holds
+constexpr int MID_MAX_ROWS = 256;               // rows of A a block holds: 64, 128 or 256
 constexpr int MID_WAVES = 4;
 constexpr int MID_THREADS = MID_WAVES * WAVE;
 constexpr int MID_CHUNK = 64;                   // k-values a step: a row of LDS is 128 bytes
 constexpr int MID_ROW_BYTES = MID_CHUNK * 2;
-constexpr int MID_A_STAGES = 3, MID_W_STAGES = 5;
-constexpr int MID_A_BYTES = MID_ROWS * MID_ROW_BYTES;          // 32 KB
-constexpr int MID_A_LOADS = MID_A_BYTES / 1024 / MID_WAVES;    // a wave's instructions for a chunk of rows: 8
+constexpr int MID_A_STAGES = 3;
+constexpr int MID_MAX_W_STAGES = 5;    // (eight were measured slower at every size: 47 against 46 us for gate/up at 64 rows)
+constexpr int MID_LDS_BYTES = 160 * 1024;
 constexpr int MID_MAX_PARTS = 4;
 constexpr int MID_UNITS = 256;                  // compute units of the chip
 
@@ -58,18 +60,30 @@ __device__ inline f32x16 mfma_32x32x16(bf16x8 a, bf16x8 b, f32x16 acc) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc, 0, 0, 0);
 }
 
-// TN: weight rows a block holds (a multiple of 32).  TC: element type of the result.
-template <int TN, typename TC, int EPI>
+// R: rows of A a block holds.  TN: weight rows it holds (a multiple of 32; of 64 for 64 rows).  TC: element type of the
+// result.  With 256 rows a wave has 64 of them (two tiles of 32) against all weight rows, with 128 rows 32 of them;
+// with 64 rows a wave has 32 rows against half of the weight rows.
+template <int R, int TN, typename TC, int EPI>
 __global__ __launch_bounds__(MID_THREADS) void linear_mid_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, TC* __restrict__ C, int M, int N, int K,
     int n_tiles, int m_tiles, int chunks_per_part) {
     constexpr int NT = TN / 32;                                 // tiles of 32 weight rows
+    constexpr int MT = R == 256 ? 2 : 1;                        // tiles of 32 rows a wave holds
+    constexpr int NTW = R == 64 ? NT / 2 : NT;                  // tiles of weight rows a wave holds
+    static_assert(R == 64 || R == 128 || R == 256, "a block holds 64, 128 or 256 rows");
+    static_assert(R != 64 || NT % 2 == 0, "with 64 rows the waves share the weight tiles in halves");
+    constexpr int MID_A_BYTES = R * MID_ROW_BYTES;              // a chunk of rows: 8, 16 or 32 KB
+    constexpr int MID_A_LOADS = MID_A_BYTES / 1024 / MID_WAVES; // a wave's instructions for it: 2, 4 or 8
     constexpr int W_BYTES = TN * MID_ROW_BYTES;
     constexpr int W_LOADS = W_BYTES / 1024 / MID_WAVES;         // a wave's instructions for a chunk of weights
     static_assert(W_BYTES % (1024 * MID_WAVES) == 0, "a chunk of weights is a whole number of instructions a wave");
     constexpr int YOUNGER = W_LOADS + MID_A_LOADS + W_LOADS;    // loads asked for after the chunk that is due, see the loop
+    // the weights' ring takes what LDS has left beside three chunks of rows, up to five chunks
+    constexpr int W_STAGES = (MID_LDS_BYTES - MID_A_STAGES * MID_A_BYTES) / W_BYTES < MID_MAX_W_STAGES
+                                 ? (MID_LDS_BYTES - MID_A_STAGES * MID_A_BYTES) / W_BYTES : MID_MAX_W_STAGES;
+    static_assert(W_STAGES >= 4 && (W_STAGES - 1) * W_LOADS + 2 * MID_A_LOADS < 64, "the ring's depth and the counter's six bits");
     __shared__ __attribute__((aligned(1024))) char a_lds[MID_A_STAGES * MID_A_BYTES];
-    __shared__ __attribute__((aligned(1024))) char w_lds[MID_W_STAGES * W_BYTES];
+    __shared__ __attribute__((aligned(1024))) char w_lds[W_STAGES * W_BYTES];
 
     const int lane = threadIdx.x % WAVE;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
@@ -84,7 +98,7 @@ __global__ __launch_bounds__(MID_THREADS) void linear_mid_kernel(
     const int features = EPI == MID_SWIGLU ? inter : N;
     const int f0 = n_tile * (EPI == MID_SWIGLU ? TN / 2 : TN);  // the block's first output feature
     if (f0 >= features) return;                                 // (the launch is padded to whole groups of eight)
-    const int row0 = m_tile * MID_ROWS;
+    const int row0 = m_tile * R;
     const int n_chunks = K / MID_CHUNK;
     const int c0 = part * chunks_per_part, c1 = min(n_chunks, c0 + chunks_per_part);
     if (c0 >= c1) return;
@@ -122,61 +136,62 @@ __global__ __launch_bounds__(MID_THREADS) void linear_mid_kernel(
     };
     auto ask_weights = [&](int chunk) __attribute__((always_inline)) {
         const char* base = reinterpret_cast<const char*>(W) + (size_t)min(chunk, c1 - 1) * MID_ROW_BYTES;
-        const uint32_t to = w_lds0 + ((chunk - c0) % MID_W_STAGES) * W_BYTES + wave * W_LOADS * 1024;
+        const uint32_t to = w_lds0 + ((chunk - c0) % W_STAGES) * W_BYTES + wave * W_LOADS * 1024;
 #pragma unroll
         for (int i = 0; i < W_LOADS; ++i) mid_load_16_bytes_a_lane_into_lds(base, w_from[i], to + i * 1024);
     };
 
     // fragments: lane l holds row l % 32 of a tile and the eight k-values 16 s + 8 (l / 32) .. of step s
     const int fr = lane % 32, fh = lane / 32;
-    struct Fragments { bf16x8 w[NT], x[2]; };
+    const int wave_row0 = R == 256 ? wave * 64 : R == 128 ? wave * 32 : (wave % 2) * 32;     // the wave's first row
+    const int wave_tile0 = R == 64 ? (wave / 2) * NTW : 0;                                  // and its first weight tile
+    struct Fragments { bf16x8 w[NTW], x[MT]; };
     auto read = [&](int a_stage, int w_stage, int step, Fragments& f) __attribute__((always_inline)) {
         const char* wp = w_lds + w_stage * W_BYTES;
         const char* xp = a_lds + a_stage * MID_A_BYTES;
         const int piece = 2 * step + fh;
 #pragma unroll
-        for (int t = 0; t < NT; ++t) {
-            const int row = t * 32 + fr;
+        for (int t = 0; t < NTW; ++t) {
+            const int row = (wave_tile0 + t) * 32 + fr;
             f.w[t] = *reinterpret_cast<const bf16x8*>(wp + row * MID_ROW_BYTES + ((piece ^ (row % 8)) * 16));
         }
 #pragma unroll
-        for (int mt = 0; mt < 2; ++mt) {
-            const int row = wave * 64 + mt * 32 + fr;
+        for (int mt = 0; mt < MT; ++mt) {
+            const int row = wave_row0 + mt * 32 + fr;
             f.x[mt] = *reinterpret_cast<const bf16x8*>(xp + row * MID_ROW_BYTES + ((piece ^ (row % 8)) * 16));
         }
     };
-    f32x16 acc[NT][2];
+    f32x16 acc[NTW][MT];
 #pragma unroll
-    for (int t = 0; t < NT; ++t)
+    for (int t = 0; t < NTW; ++t)
 #pragma unroll
-        for (int mt = 0; mt < 2; ++mt)
+        for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
             for (int i = 0; i < 16; ++i) acc[t][mt][i] = 0.f;
     auto products = [&](const Fragments& f) __attribute__((always_inline)) {
 #pragma unroll
-        for (int t = 0; t < NT; ++t)
+        for (int t = 0; t < NTW; ++t)
 #pragma unroll
-            for (int mt = 0; mt < 2; ++mt) acc[t][mt] = mfma_32x32x16(f.w[t], f.x[mt], acc[t][mt]);
+            for (int mt = 0; mt < MT; ++mt) acc[t][mt] = mfma_32x32x16(f.w[t], f.x[mt], acc[t][mt]);
     };
 
-    // The rings fill.  Pass c of the loop asks for the rows of chunk c + 3 and then the weights of chunk c + 5, and
-    // waits, before that, for chunk c + 1 with all that was asked for after its rows still on its way: the weights of
-    // c + 3, the rows of c + 2, the weights of c + 4.  So these three groups come last here, in that order, and the
-    // first pass finds the loads in the order every later pass does.
+    // The rings fill.  Pass c of the loop asks for the rows of chunk c + 3 and then the weights of chunk c + W_STAGES,
+    // and waits, before that, for chunk c + 1 with all that was asked for after its rows still on its way: the weights
+    // asked for in the same pass, and the rows and weights of the pass after.  So these three groups come last here, in
+    // that order, and the first pass finds the loads in the order every later pass does.
     ask_rows(c0);
-    ask_weights(c0);
-    ask_weights(c0 + 1);
-    ask_weights(c0 + 2);
+#pragma unroll
+    for (int s = 0; s < W_STAGES - 2; ++s) ask_weights(c0 + s);
     ask_rows(c0 + 1);
-    ask_weights(c0 + 3);
+    ask_weights(c0 + W_STAGES - 2);
     ask_rows(c0 + 2);
-    ask_weights(c0 + 4);
-    mid_wait_for_all_but_the_youngest_loads<4 * W_LOADS + 2 * MID_A_LOADS>();        // the first chunk's rows and weights are there
+    ask_weights(c0 + W_STAGES - 1);
+    mid_wait_for_all_but_the_youngest_loads<(W_STAGES - 1) * W_LOADS + 2 * MID_A_LOADS>();      // the first chunk's rows and weights are there
     mid_barrier();
     Fragments f[2];
     read(0, 0, 0, f[0]);
     for (int c = c0; c < c1; ++c) {
-        const int a_stage = (c - c0) % MID_A_STAGES, w_stage = (c - c0) % MID_W_STAGES;
+        const int a_stage = (c - c0) % MID_A_STAGES, w_stage = (c - c0) % W_STAGES;
 #pragma unroll
         for (int step = 0; step < MID_CHUNK / 16 - 1; ++step) {
             read(a_stage, w_stage, step + 1, f[(step + 1) & 1]);
@@ -187,8 +202,8 @@ __global__ __launch_bounds__(MID_THREADS) void linear_mid_kernel(
         mid_wait_for_all_but_the_youngest_loads<YOUNGER>();
         mid_barrier();
         ask_rows(c + MID_A_STAGES);                             // into the slots that this chunk's readers have left
-        ask_weights(c + MID_W_STAGES);
-        if (c + 1 < c1) read((c + 1 - c0) % MID_A_STAGES, (c + 1 - c0) % MID_W_STAGES, 0, f[0]);
+        ask_weights(c + W_STAGES);
+        if (c + 1 < c1) read((c + 1 - c0) % MID_A_STAGES, (c + 1 - c0) % W_STAGES, 0, f[0]);
         products(f[(MID_CHUNK / 16 - 1) & 1]);
     }
     mid_wait_for_all_but_the_youngest_loads<0>();               // nothing of this block is on its way when it ends
@@ -196,16 +211,16 @@ __global__ __launch_bounds__(MID_THREADS) void linear_mid_kernel(
     // lane l holds token column l % 32 of each tile and, of the tile's 32 weight rows, rows 8 j + 4 (l / 32) + 0..3 as
     // elements 4 j .. 4 j + 3
 #pragma unroll
-    for (int mt = 0; mt < 2; ++mt) {
-        const int token = row0 + wave * 64 + mt * 32 + fr;
+    for (int mt = 0; mt < MT; ++mt) {
+        const int token = row0 + wave_row0 + mt * 32 + fr;
         if (token >= M) continue;
 #pragma unroll
-        for (int t = 0; t < NT; ++t) {
+        for (int t = 0; t < NTW; ++t) {
             if (EPI == MID_SWIGLU) {
                 // rows 0..15 of the tile are gate rows, 16..31 their up rows: elements 4 j + i and 4 (j + 2) + i
 #pragma unroll
                 for (int j = 0; j < 2; ++j) {
-                    const int feature = f0 + t * 16 + 8 * j + 4 * fh;
+                    const int feature = f0 + (wave_tile0 + t) * 16 + 8 * j + 4 * fh;
                     float out[4];
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
@@ -230,7 +245,7 @@ __global__ __launch_bounds__(MID_THREADS) void linear_mid_kernel(
             } else {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    const int feature = f0 + t * 32 + 8 * j + 4 * fh;
+                    const int feature = f0 + (wave_tile0 + t) * 32 + 8 * j + 4 * fh;
                     const float out[4] = {acc[t][mt][4 * j], acc[t][mt][4 * j + 1], acc[t][mt][4 * j + 2], acc[t][mt][4 * j + 3]};
                     TC* to = C + (size_t)token * N + feature;
                     if (feature + 3 < N && N % 4 == 0) {
@@ -252,16 +267,22 @@ __global__ __launch_bounds__(MID_THREADS) void linear_mid_kernel(
     }
 }
 
-struct MidPlan { int tn, parts, chunks_per_part, n_tiles, m_tiles; };
+struct MidPlan { int rows, tn, parts, chunks_per_part, n_tiles, m_tiles; };
 
-// Weight rows a block (96 or 64) and ranges of K: what takes the fewest rounds of blocks over the compute units, a
-// round costing its chunks (and a few for filling the rings) times the block's weight rows.
+// rows a block holds for a product of M rows
+static int mid_rows(int M) { return M <= 64 ? 64 : M <= 128 ? 128 : MID_MAX_ROWS; }
+
+// Weight rows a block (128, 96 or 64: what fits LDS beside the rows, and with 64 rows an even number of tiles) and
+// ranges of K: what takes the fewest rounds of blocks over the compute units, a round costing its chunks (and a few
+// for filling the rings) times the block's weight rows.
 static MidPlan mid_plan(int M, int N, int K, int epilogue, int max_parts) {
     const int n_chunks = K / MID_CHUNK;
-    const int m_tiles = (M + MID_ROWS - 1) / MID_ROWS;
-    MidPlan best{96, 1, n_chunks, 1, m_tiles};
+    const int rows = mid_rows(M);
+    const int m_tiles = (M + rows - 1) / rows;
+    MidPlan best{rows, 64, 1, n_chunks, 1, m_tiles};
     long best_cost = -1;
-    for (int tn = 96; tn >= 64; tn -= 32) {
+    for (int tn = 128; tn >= 64; tn -= 32) {
+        if ((rows == 256 && tn == 128) || (rows == 64 && tn == 96)) continue;
         const int per_block = epilogue == MID_SWIGLU ? tn / 2 : tn;
         const int features = epilogue == MID_SWIGLU ? N / 2 : N;
         const int n_tiles = (features + per_block - 1) / per_block;
@@ -270,7 +291,7 @@ static MidPlan mid_plan(int M, int N, int K, int epilogue, int max_parts) {
             if (parts > 1 && (per < 8 || (parts - 1) * per >= n_chunks)) continue;       // short, or an empty range
             const long blocks = (long)n_tiles * parts * m_tiles;
             const long cost = ((blocks + MID_UNITS - 1) / MID_UNITS) * (per + 6) * tn;
-            if (best_cost < 0 || cost < best_cost) { best_cost = cost; best = MidPlan{tn, parts, per, n_tiles, m_tiles}; }
+            if (best_cost < 0 || cost < best_cost) { best_cost = cost; best = MidPlan{rows, tn, parts, per, n_tiles, m_tiles}; }
         }
     }
     return best;
@@ -289,12 +310,20 @@ PALM_API int palm_linear_mid_blocks(int M, int N, int K, int epilogue, int plane
     return plan.n_tiles * plan.parts * plan.m_tiles;
 }
 
-template <int TN, typename TC, int EPI>
+template <int R, int TN, typename TC, int EPI>
 static void launch_mid(hipStream_t stream, const void* a, const void* w, void* c, int M, int N, int K, MidPlan plan) {
     const int work = plan.n_tiles * plan.parts;
     const int groups = (work + 7) / 8;                          // whole groups of eight tiles of weights, a die each
-    linear_mid_kernel<TN, TC, EPI><<<groups * 8 * plan.m_tiles, MID_THREADS, 0, stream>>>(
+    linear_mid_kernel<R, TN, TC, EPI><<<groups * 8 * plan.m_tiles, MID_THREADS, 0, stream>>>(
         (const bf16_t*)a, (const bf16_t*)w, (TC*)c, M, N, K, plan.n_tiles, plan.m_tiles, plan.chunks_per_part);
+}
+
+template <int R, int TN>
+static void launch_mid_as(hipStream_t stream, const void* a, const void* w, void* c, int c_dtype, int M, int N, int K,
+                          int epilogue, MidPlan plan) {
+    if (epilogue == MID_SWIGLU) launch_mid<R, TN, bf16_t, MID_SWIGLU>(stream, a, w, c, M, N, K, plan);
+    else if (c_dtype == PALM_BF16) launch_mid<R, TN, bf16_t, MID_STORE>(stream, a, w, c, M, N, K, plan);
+    else launch_mid<R, TN, float, MID_STORE>(stream, a, w, c, M, N, K, plan);
 }
 
 // a [M, K] bfloat16, w [N, K] bfloat16, K a multiple of 64; c [M, N] (store) or [M, N/2] (gated) in bfloat16, or, with
@@ -315,11 +344,10 @@ PALM_API int palm_linear_mid(hipStream_t stream, const void* a, const void* w, v
                "linear_mid: %d planes asked for, %d planned (planes are float32, not gated)", parts, plan.parts);
     PALM_CHECK(epilogue == MID_STORE || c_dtype == PALM_BF16, "linear_mid: a gated product comes in bfloat16");
     if (M == 0) return 0;
-#define PALM_MID(TN) do { \
-        if (epilogue == MID_SWIGLU) launch_mid<TN, bf16_t, MID_SWIGLU>(stream, a, w, c, M, N, K, plan); \
-        else if (c_dtype == PALM_BF16) launch_mid<TN, bf16_t, MID_STORE>(stream, a, w, c, M, N, K, plan); \
-        else launch_mid<TN, float, MID_STORE>(stream, a, w, c, M, N, K, plan); } while (0)
-    if (plan.tn == 96) PALM_MID(96); else PALM_MID(64);
+#define PALM_MID(R, TN) launch_mid_as<R, TN>(stream, a, w, c, c_dtype, M, N, K, epilogue, plan)
+    if (plan.rows == 64) { if (plan.tn == 128) PALM_MID(64, 128); else PALM_MID(64, 64); }
+    else if (plan.rows == 128) { if (plan.tn == 128) PALM_MID(128, 128); else if (plan.tn == 96) PALM_MID(128, 96); else PALM_MID(128, 64); }
+    else { if (plan.tn == 96) PALM_MID(256, 96); else PALM_MID(256, 64); }
 #undef PALM_MID
     PALM_LAUNCHED();
     return 0;

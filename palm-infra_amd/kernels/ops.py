@@ -393,23 +393,35 @@ def wide_pays(M: int, N: int, K: int, gated: bool = False, planes_ok: bool = Fal
         M, N, K, 1 if gated else 0, 1 if planes_ok else 0) >= WIDE_MIN_BLOCKS
 
 
-MID_TOKENS = 256      # rows of one block of the kernel for short prompts
-MID_CHUNK = 64        # which walks over K in steps of this many
+MID_TOKENS = 256      # rows of one block of the kernel whose operands both cross LDS
+MID_FROM = 32         # above this many rows it beats the kernel that keeps the weights in registers
+MID_CHUNK = 64        # it walks over K in steps of this many
 
 
-def mid_pays(M: int, N: int, K: int, planes_ok: bool = False) -> bool:
-    """Whether the kernel for 129 to 256 rows beats the library for this product: where the weight rows are so few
-    that it cuts K into planes of partial sums (which the reader must take) to fill the chip; the library's tiles
-    leave compute units idle there.  Measured at Qwen3-8B's shapes (us, own against library): with 256 rows q/k/v 29
-    and 40, output projection 23 and 24, down 46 and 53; with 129 rows (library at 192) 23 and 34, 18 and 33, 39 and
-    88; the planes cost their readers about 4 us each.  Not a product with weight rows enough for all compute units
-    (gate/up at 256 rows: 70 against 65, gated 79 against 65 and the activation's pass of 8; every block then reads
-    all rows again for 96 weight rows, and the way from L2 into a compute unit, 60 to 80 GB/s when all of them pull, is
-    as long as the arithmetic), and not more than 256 rows, where it ties (q/k/v 40 and 37, output projection 32 and
-    30, down 78 and 80 at 512 rows)."""
-    return (planes_ok and WIDE_TOKENS < M <= MID_TOKENS and K % MID_CHUNK == 0
-            and core().palm_linear_mid_parts(M, N, K, 0) > 1
-            and core().palm_linear_mid_blocks(M, N, K, 0, 1) >= WIDE_MIN_BLOCKS)
+def mid_pays(M: int, N: int, K: int, planes_ok: bool = False, gated: bool = False,
+             out_dtype: torch.dtype = BF16) -> bool:
+    """Whether the kernel that brings both operands through rings in LDS serves this product of bfloat16 operands.
+
+    33 to 128 rows (decode steps of many sequences, short prompts): wherever its blocks fill the chip (for few weight
+    rows that needs a reader that takes planes); a float32 result of up to 64 rows stays with the kernel that shares
+    the rows through LDS.  Measured at Qwen3-8B's shapes (us, this kernel against that one): 64 rows gate/up gated 46
+    and 49, down 25 and 27, output projection 11 and 14, q/k/v 16 and 17, head 284 and 275; 128 rows 51 and 67, 30 and
+    36, 14 and 17, 19 and 21, 308 and 338; 32 rows 45 and 41, 23 and 24, 10 and 11, 15 and 14.
+
+    129 to 256 rows (short prompts): where the weight rows are so few that it cuts K into planes; the library's tiles
+    leave compute units idle there.  Own against library at 256 rows: q/k/v 29 and 40, output projection 23 and 24,
+    down 46 and 53; at 129 rows (library at 192) 23 and 34, 18 and 33, 39 and 88; the planes cost their readers about
+    4 us each.  Not a product with weight rows enough for all compute units (gate/up at 256 rows: 70 against 65, gated
+    79 against 65 and the activation's pass of 8; every block then reads all rows again for 96 weight rows, and the
+    way from L2 into a compute unit, 60 to 80 GB/s when all of them pull, is as long as the arithmetic), and not more
+    than 256 rows, where it ties (q/k/v 40 and 37, output projection 32 and 30, down 78 and 80 at 512 rows)."""
+    if K % MID_CHUNK != 0 or not MID_FROM < M <= MID_TOKENS:
+        return False
+    planes = planes_ok and not gated
+    blocks = core().palm_linear_mid_blocks(M, N, K, 1 if gated else 0, 1 if planes else 0)
+    if M <= WIDE_TOKENS:
+        return blocks >= WIDE_MIN_BLOCKS and (out_dtype == BF16 or planes or M > WIDE_FLOAT32_TOKENS)
+    return planes and out_dtype == BF16 and core().palm_linear_mid_parts(M, N, K, 0) > 1 and blocks >= WIDE_MIN_BLOCKS
 
 
 def linear_mid(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, gated: bool = False,

@@ -2,9 +2,9 @@
 
   float32 run, or a 32-bit weight under bfloat16 activations   the exact FMA kernel
   bfloat16 x bfloat16, up to 16 rows (decode)                   the matrix-core kernel for thin products
-  bfloat16 x bfloat16, 17 to 128 rows (large decode batches)    the matrix-core kernel that shares the rows through LDS
-  bfloat16 x bfloat16, 129 to 256 rows (short prompts)          the kernel that brings both operands through rings in
-                                                                LDS, where it beats the library (ops.mid_pays)
+  bfloat16 x bfloat16, 17 to 32 rows (decode batches)           the matrix-core kernel that shares the rows through LDS
+  bfloat16 x bfloat16, 33 to 256 rows (large decode batches,    the kernel that brings both operands through rings in
+  short prompts)                                                LDS, where it beats the others (ops.mid_pays)
   bfloat16 x bfloat16, many rows (prompts)                      the BLAS library, as the reference's GPU path
                                                                 does for its products (engine/cuda_matmul.cu:245-260)
 
@@ -19,10 +19,10 @@ import torch
 from ..kernels import ops
 from .residual import Prenormed
 
-# Up to this many rows the kernel that streams the weight past one block of 16 rows serves; from there to 128 rows
-# the kernel that shares the rows through LDS, where it has blocks enough to fill the chip (ops.wide_pays), and
-# for every product with a float32 result; from 129 to 256 rows the kernel with rings in LDS where it pays
-# (ops.mid_pays); else the library.
+# Up to this many rows the kernel that streams the weight past one block of 16 rows serves; from 33 to 256 rows the
+# kernel with rings in LDS where it pays (ops.mid_pays); else, up to 128 rows, the kernel that shares the rows through
+# LDS, where it has blocks enough to fill the chip (ops.wide_pays), and for every product with a float32 result; else
+# the library.
 THIN_ROWS = 16
 
 
@@ -66,11 +66,12 @@ class Linear:
             x = x.materialize()
         out_dtype = out_dtype or x.dtype
         if x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16:
-            if (x.shape[0] <= THIN_ROWS or out_dtype != torch.bfloat16
-                    or (ops.thin_serves(x, w) and ops.wide_pays(x.shape[0], self.out_features, self.in_features, planes_ok=planes_ok))):
-                return ops.linear_thin(x, w, out_dtype, planes_ok=planes_ok)
-            if x.is_contiguous() and ops.mid_pays(x.shape[0], self.out_features, self.in_features, planes_ok=planes_ok):
+            rows = x.shape[0]
+            if x.is_contiguous() and ops.mid_pays(rows, self.out_features, self.in_features, planes_ok=planes_ok, out_dtype=out_dtype):
                 return ops.linear_mid(x, w, out_dtype, planes_ok=planes_ok)
+            if (rows <= THIN_ROWS or out_dtype != torch.bfloat16
+                    or (ops.thin_serves(x, w) and ops.wide_pays(rows, self.out_features, self.in_features, planes_ok=planes_ok))):
+                return ops.linear_thin(x, w, out_dtype, planes_ok=planes_ok)
             return ops.linear_library(x, w)
         return ops.linear_exact(x, w, out_dtype)
 
@@ -96,6 +97,9 @@ class Linear:
             if self._folds(x.values):
                 return ops.linear_thin(x.values, self.weight, x.dtype, gated=True, row_ss=x.ss, row_eps=x.eps)
             x = x.materialize()
+        if (x.dtype == torch.bfloat16 and self.weight.dtype == torch.bfloat16 and x.is_contiguous()
+                and ops.mid_pays(x.shape[0], self.out_features, self.in_features, gated=True)):
+            return ops.linear_mid(x, self.weight, x.dtype, gated=True)
         if ops.thin_serves(x, self.weight) and (
                 x.shape[0] <= THIN_ROWS or ops.wide_pays(x.shape[0], self.out_features, self.in_features, gated=True)):
             return ops.linear_thin(x, self.weight, x.dtype, gated=True)
