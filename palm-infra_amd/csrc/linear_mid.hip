@@ -36,8 +36,7 @@ constexpr int MID_WAVES = 4;
 constexpr int MID_THREADS = MID_WAVES * WAVE;
 constexpr int MID_CHUNK = 64;                   // k-values a step: a row of LDS is 128 bytes
 constexpr int MID_ROW_BYTES = MID_CHUNK * 2;
-constexpr int MID_A_STAGES = 3;
-constexpr int MID_MAX_W_STAGES = 5;    // (eight were measured slower at every size: 47 against 46 us for gate/up at 64 rows)
+constexpr int MID_MAX_STAGES = 6;
 constexpr int MID_LDS_BYTES = 160 * 1024;
 constexpr int MID_MAX_PARTS = 4;
 constexpr int MID_UNITS = 256;                  // compute units of the chip
@@ -66,7 +65,7 @@ __device__ inline f32x16 mfma_32x32x16(bf16x8 a, bf16x8 b, f32x16 acc) {
 template <int R, int TN, typename TC, int EPI>
 __global__ __launch_bounds__(MID_THREADS) void linear_mid_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, TC* __restrict__ C, int M, int N, int K,
-    int n_tiles, int m_tiles, int chunks_per_part) {
+    int n_tiles, int m_tiles, int chunks_per_part, int turn_blocks) {
     constexpr int NT = TN / 32;                                 // tiles of 32 weight rows
     constexpr int MT = R == 256 ? 2 : 1;                        // tiles of 32 rows a wave holds
     constexpr int NTW = R == 64 ? NT / 2 : NT;                  // tiles of weight rows a wave holds
@@ -77,12 +76,22 @@ __global__ __launch_bounds__(MID_THREADS) void linear_mid_kernel(
     constexpr int W_BYTES = TN * MID_ROW_BYTES;
     constexpr int W_LOADS = W_BYTES / 1024 / MID_WAVES;         // a wave's instructions for a chunk of weights
     static_assert(W_BYTES % (1024 * MID_WAVES) == 0, "a chunk of weights is a whole number of instructions a wave");
-    constexpr int YOUNGER = W_LOADS + MID_A_LOADS + W_LOADS;    // loads asked for after the chunk that is due, see the loop
-    // the weights' ring takes what LDS has left beside three chunks of rows, up to five chunks
-    constexpr int W_STAGES = (MID_LDS_BYTES - MID_A_STAGES * MID_A_BYTES) / W_BYTES < MID_MAX_W_STAGES
-                                 ? (MID_LDS_BYTES - MID_A_STAGES * MID_A_BYTES) / W_BYTES : MID_MAX_W_STAGES;
-    static_assert(W_STAGES >= 4 && (W_STAGES - 1) * W_LOADS + 2 * MID_A_LOADS < 64, "the ring's depth and the counter's six bits");
-    __shared__ __attribute__((aligned(1024))) char a_lds[MID_A_STAGES * MID_A_BYTES];
+    // The rings.  All loads come back in the order they went out, and one counter counts them all: a wait for the rows
+    // of the next chunk is also a wait for every load asked for before them.  So what is still on its way after a
+    // pass's wait is what was asked for after the younger of the next chunk's two operands, and the rings are as deep
+    // in flight as the shallower of them.  With 64 or 128 rows both rings have the same depth, as many chunks as LDS
+    // holds, up to six (64 rows x 128 weight rows: 6 x 24 KB, of which four are on their way after a wait; with three
+    // chunks of rows and five of weights only two chunks of weights were, 32 KB a compute unit, and the stream of
+    // weights alone took 46 us for 201 MB).  256 rows leave room for three chunks of rows and five of weights.
+    constexpr bool SAME = R != 256;
+    constexpr int BOTH = (MID_LDS_BYTES / (MID_A_BYTES + W_BYTES)) < MID_MAX_STAGES ? (MID_LDS_BYTES / (MID_A_BYTES + W_BYTES)) : MID_MAX_STAGES;
+    constexpr int A_STAGES = SAME ? BOTH : 3;
+    constexpr int W_STAGES = SAME ? BOTH : (MID_LDS_BYTES - 3 * MID_A_BYTES) / W_BYTES < 5 ? (MID_LDS_BYTES - 3 * MID_A_BYTES) / W_BYTES : 5;
+    // loads asked for after the chunk that is due, see the loop
+    constexpr int YOUNGER = SAME ? (A_STAGES - 2) * (MID_A_LOADS + W_LOADS) : W_LOADS + MID_A_LOADS + W_LOADS;
+    constexpr int YOUNGER_AT_START = SAME ? (A_STAGES - 1) * (MID_A_LOADS + W_LOADS) : (W_STAGES - 1) * W_LOADS + 2 * MID_A_LOADS;
+    static_assert(A_STAGES >= 3 && W_STAGES >= 4 && YOUNGER_AT_START < 64, "the rings' depth and the counter's six bits");
+    __shared__ __attribute__((aligned(1024))) char a_lds[A_STAGES * MID_A_BYTES];
     __shared__ __attribute__((aligned(1024))) char w_lds[W_STAGES * W_BYTES];
 
     const int lane = threadIdx.x % WAVE;
@@ -127,15 +136,24 @@ __global__ __launch_bounds__(MID_THREADS) void linear_mid_kernel(
         w_from[i] = (uint32_t)feature * (uint32_t)K * 2u + piece * 16;
     }
     const uint32_t a_lds0 = mid_lds_address(a_lds), w_lds0 = mid_lds_address(w_lds);
+    // Where a block begins in its range of K.  Weight rows are K elements apart, a power of two in most models, and
+    // blocks that walk over K in step ask the memory for the same few hundred bytes of every row at the same time:
+    // the same few channels.  Where K is not cut (many weight rows: the gated product, the head) tile b of the weights begins b
+    // chunks into K and wraps around, which spreads the blocks over the channels: the head for 64 rows 283 to 231 us,
+    // gate/up for 128 rows 52 to 47.  Where K is cut the rows' share of the traffic is larger, and blocks out of step
+    // no longer find each other's rows in L2 (down projection for 128 rows 33 to 38 us; with only the dies out of step
+    // with each other nothing changes): those keep step.
+    const int turn = turn_blocks ? work % (c1 - c0) : 0;       // (the row tiles of one tile of weights keep step)
+    auto turned = [&](int chunk) __attribute__((always_inline)) { const int t = chunk - c0 + turn; return c0 + (t >= c1 - c0 ? t - (c1 - c0) : t); };
     // beyond the range's end: its last chunk once more, into a slot that nobody reads any more
     auto ask_rows = [&](int chunk) __attribute__((always_inline)) {
-        const char* base = reinterpret_cast<const char*>(A) + (size_t)min(chunk, c1 - 1) * MID_ROW_BYTES;
-        const uint32_t to = a_lds0 + ((chunk - c0) % MID_A_STAGES) * MID_A_BYTES + wave * MID_A_LOADS * 1024;
+        const char* base = reinterpret_cast<const char*>(A) + (size_t)turned(min(chunk, c1 - 1)) * MID_ROW_BYTES;
+        const uint32_t to = a_lds0 + ((chunk - c0) % A_STAGES) * MID_A_BYTES + wave * MID_A_LOADS * 1024;
 #pragma unroll
         for (int i = 0; i < MID_A_LOADS; ++i) mid_load_16_bytes_a_lane_into_lds(base, a_from[i], to + i * 1024);
     };
     auto ask_weights = [&](int chunk) __attribute__((always_inline)) {
-        const char* base = reinterpret_cast<const char*>(W) + (size_t)min(chunk, c1 - 1) * MID_ROW_BYTES;
+        const char* base = reinterpret_cast<const char*>(W) + (size_t)turned(min(chunk, c1 - 1)) * MID_ROW_BYTES;
         const uint32_t to = w_lds0 + ((chunk - c0) % W_STAGES) * W_BYTES + wave * W_LOADS * 1024;
 #pragma unroll
         for (int i = 0; i < W_LOADS; ++i) mid_load_16_bytes_a_lane_into_lds(base, w_from[i], to + i * 1024);
@@ -175,23 +193,30 @@ __global__ __launch_bounds__(MID_THREADS) void linear_mid_kernel(
             for (int mt = 0; mt < MT; ++mt) acc[t][mt] = mfma_32x32x16(f.w[t], f.x[mt], acc[t][mt]);
     };
 
-    // The rings fill.  Pass c of the loop asks for the rows of chunk c + 3 and then the weights of chunk c + W_STAGES,
-    // and waits, before that, for chunk c + 1 with all that was asked for after its rows still on its way: the weights
-    // asked for in the same pass, and the rows and weights of the pass after.  So these three groups come last here, in
-    // that order, and the first pass finds the loads in the order every later pass does.
-    ask_rows(c0);
+    // The rings fill.  Pass c of the loop asks for the rows of chunk c + A_STAGES and then the weights of chunk
+    // c + W_STAGES, and waits, before that, for chunk c + 1 with all that was asked for after the younger of its
+    // operands still on its way.  The loads go out here in the order in which the passes before the first would have
+    // asked for them, so that the first pass finds them as every later pass does.  Rings of the same depth: rows and
+    // weights of a chunk side by side.  Three chunks of rows and more of weights: the weights asked for in the pass of
+    // the next chunk's rows, and the rows and weights of the pass after, come last.
+    if (SAME) {
 #pragma unroll
-    for (int s = 0; s < W_STAGES - 2; ++s) ask_weights(c0 + s);
-    ask_rows(c0 + 1);
-    ask_weights(c0 + W_STAGES - 2);
-    ask_rows(c0 + 2);
-    ask_weights(c0 + W_STAGES - 1);
-    mid_wait_for_all_but_the_youngest_loads<(W_STAGES - 1) * W_LOADS + 2 * MID_A_LOADS>();      // the first chunk's rows and weights are there
+        for (int s = 0; s < A_STAGES; ++s) { ask_rows(c0 + s); ask_weights(c0 + s); }
+    } else {
+        ask_rows(c0);
+#pragma unroll
+        for (int s = 0; s < W_STAGES - 2; ++s) ask_weights(c0 + s);
+        ask_rows(c0 + 1);
+        ask_weights(c0 + W_STAGES - 2);
+        ask_rows(c0 + 2);
+        ask_weights(c0 + W_STAGES - 1);
+    }
+    mid_wait_for_all_but_the_youngest_loads<YOUNGER_AT_START>();      // the first chunk's rows and weights are there
     mid_barrier();
     Fragments f[2];
     read(0, 0, 0, f[0]);
     for (int c = c0; c < c1; ++c) {
-        const int a_stage = (c - c0) % MID_A_STAGES, w_stage = (c - c0) % W_STAGES;
+        const int a_stage = (c - c0) % A_STAGES, w_stage = (c - c0) % W_STAGES;
 #pragma unroll
         for (int step = 0; step < MID_CHUNK / 16 - 1; ++step) {
             read(a_stage, w_stage, step + 1, f[(step + 1) & 1]);
@@ -201,9 +226,9 @@ __global__ __launch_bounds__(MID_THREADS) void linear_mid_kernel(
         // must have landed, for every wave's share of it: all but the loads asked for after it are done.
         mid_wait_for_all_but_the_youngest_loads<YOUNGER>();
         mid_barrier();
-        ask_rows(c + MID_A_STAGES);                             // into the slots that this chunk's readers have left
+        ask_rows(c + A_STAGES);                                 // into the slots that this chunk's readers have left
         ask_weights(c + W_STAGES);
-        if (c + 1 < c1) read((c + 1 - c0) % MID_A_STAGES, (c + 1 - c0) % W_STAGES, 0, f[0]);
+        if (c + 1 < c1) read((c + 1 - c0) % A_STAGES, (c + 1 - c0) % W_STAGES, 0, f[0]);
         products(f[(MID_CHUNK / 16 - 1) & 1]);
     }
     mid_wait_for_all_but_the_youngest_loads<0>();               // nothing of this block is on its way when it ends
@@ -315,7 +340,8 @@ static void launch_mid(hipStream_t stream, const void* a, const void* w, void* c
     const int work = plan.n_tiles * plan.parts;
     const int groups = (work + 7) / 8;                          // whole groups of eight tiles of weights, a die each
     linear_mid_kernel<R, TN, TC, EPI><<<groups * 8 * plan.m_tiles, MID_THREADS, 0, stream>>>(
-        (const bf16_t*)a, (const bf16_t*)w, (TC*)c, M, N, K, plan.n_tiles, plan.m_tiles, plan.chunks_per_part);
+        (const bf16_t*)a, (const bf16_t*)w, (TC*)c, M, N, K, plan.n_tiles, plan.m_tiles, plan.chunks_per_part,
+        plan.parts == 1 ? 1 : 0);
 }
 
 template <int R, int TN>

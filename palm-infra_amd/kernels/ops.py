@@ -403,11 +403,9 @@ def mid_pays(M: int, N: int, K: int, planes_ok: bool = False, gated: bool = Fals
     """Whether the kernel that brings both operands through rings in LDS serves this product of bfloat16 operands.
 
     33 to 128 rows (decode steps of many sequences, short prompts): wherever its blocks fill the chip (for few weight
-    rows that needs a reader that takes planes); a whole float32 result (logits) stays with the kernel that shares
-    the rows through LDS, up to 64 rows, and with the tiled kernel beyond (the head for 128 rows: 323 us here, 289
-    there).  Measured at Qwen3-8B's shapes (us, this kernel against that one): 64 rows gate/up gated 46
-    and 49, down 25 and 27, output projection 11 and 14, q/k/v 16 and 17, head 284 and 275; 128 rows 51 and 67, 30 and
-    36, 14 and 17, 19 and 21, 308 and 338; 32 rows 45 and 41, 23 and 24, 10 and 11, 15 and 14.
+    rows that needs a reader that takes planes).  Measured at Qwen3-8B's shapes (us, this kernel against that one): 64 rows gate/up gated 46
+    and 49, down 25 and 27, output projection 11 and 14, q/k/v 16 and 17, head 231 and 275; 128 rows 47 and 67, 30 and
+    36, 14 and 17, 19 and 21, 273 and 338 (the tiled kernel 289); 32 rows 45 and 41, 23 and 24, 10 and 11, 15 and 14.
 
     129 to 256 rows (short prompts): where the weight rows are so few that it cuts K into planes; the library's tiles
     leave compute units idle there.  Own against library at 256 rows: q/k/v 29 and 40, output projection 23 and 24,
@@ -421,7 +419,7 @@ def mid_pays(M: int, N: int, K: int, planes_ok: bool = False, gated: bool = Fals
     planes = planes_ok and not gated
     blocks = core().palm_linear_mid_blocks(M, N, K, 1 if gated else 0, 1 if planes else 0)
     if M <= WIDE_TOKENS:
-        return blocks >= WIDE_MIN_BLOCKS and (out_dtype == BF16 or planes)
+        return blocks >= WIDE_MIN_BLOCKS
     return planes and out_dtype == BF16 and core().palm_linear_mid_parts(M, N, K, 0) > 1 and blocks >= WIDE_MIN_BLOCKS
 
 

@@ -264,10 +264,10 @@ def test_linear_mid_refuses_what_it_does_not_serve(ops):
     assert not ops.mid_pays(300, 4096, 4096, planes_ok=True)
     assert ops.mid_pays(200, 4096, 4096, planes_ok=True) and not ops.mid_pays(200, 4096, 4096, planes_ok=False)
     assert not ops.mid_pays(200, 24576, 4096, planes_ok=True)           # weight rows enough: no planes, the library's
-    # 33 to 128 rows: wherever the blocks fill the chip; no whole float32 result
+    # 33 to 128 rows: wherever the blocks fill the chip
     assert ops.mid_pays(64, 24576, 4096, gated=True) and ops.mid_pays(100, 4096, 4096, planes_ok=True)
     assert not ops.mid_pays(100, 4096, 4096, planes_ok=False) and not ops.mid_pays(64, 96, 128)
-    assert not ops.mid_pays(128, 151936, 4096, out_dtype=F32) and not ops.mid_pays(64, 151936, 4096, out_dtype=F32)
+    assert ops.mid_pays(128, 151936, 4096, out_dtype=F32) and ops.mid_pays(64, 151936, 4096, out_dtype=F32)
 
 
 def test_a_short_prompts_projections_take_the_kernel_with_rings(ops, monkeypatch):
