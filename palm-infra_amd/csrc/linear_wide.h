@@ -89,6 +89,14 @@ __global__ __launch_bounds__(NW * WAVE) void linear_wide_kernel(
     const int c0 = blockIdx.y * chunks_per_part, c1 = min(n_chunks, c0 + chunks_per_part);
     if (c0 >= c1) return;                      // (the host plans no empty range)
     if (gridDim.y > 1) C += (size_t)blockIdx.y * M * N;
+    // Where a block begins in K.  Weight rows are K elements apart, a power of two in most models, and blocks that
+    // walk over K in step ask the memory for the same few hundred bytes of every row at the same time: the same few
+    // channels.  Where K is not cut and all blocks run at once (the gated product) block b begins b chunks into K
+    // and wraps around: 44 to 40 us for 32 rows.  Where K is cut the blocks keep step: the rows' share of the traffic
+    // is larger there, and blocks out of step no longer find each other's rows in L2.  Where the blocks come in
+    // several rounds (the head) they are out of step by themselves, and turning them made it slower (252 to 279 us).
+    const int turn = gridDim.y == 1 && gridDim.x <= WIDE_UNITS ? (int)(blockIdx.x % (unsigned)(c1 - c0)) : 0;
+    auto turned = [&](int chunk) __attribute__((always_inline)) { const int t = chunk - c0 + turn; return c0 + (t >= c1 - c0 ? t - (c1 - c0) : t); };
 
     f32x4 acc[MB];
 #pragma unroll
@@ -103,8 +111,9 @@ __global__ __launch_bounds__(NW * WAVE) void linear_wide_kernel(
     for (int i = 0; i < XS; ++i) x_row[i] = (uint32_t)min(x_row0 + i * ROW_STEP, M - 1) * K * sizeof(bf16_t);
 
     bf16x8 wf[RING][FRAGMENTS], xs[RING][XS];
-    auto ask_rows = [&](int chunk, auto slot) __attribute__((always_inline)) {
+    auto ask_rows = [&](int logical, auto slot) __attribute__((always_inline)) {
         constexpr int s = decltype(slot)::value;
+        const int chunk = turned(logical);
         // what lies beyond M or K reads a place that exists; put_rows makes zeros of it
         const bool ok = EXACT || chunk * WIDE_CHUNK + x_piece * 8 < K;
         const char* from = x_base + (ok ? chunk * CHUNK_BYTES : 0);
@@ -112,8 +121,9 @@ __global__ __launch_bounds__(NW * WAVE) void linear_wide_kernel(
 #pragma unroll
         for (int i = 0; i < XS; ++i) xs[s][i] = load_bf16x8_at(from, x_row[i] + at);
     };
-    auto ask_weights = [&](int chunk, auto slot) __attribute__((always_inline)) {
+    auto ask_weights = [&](int logical, auto slot) __attribute__((always_inline)) {
         constexpr int s = decltype(slot)::value;
+        const int chunk = turned(logical);
         const char* from = w_base + (size_t)chunk * CHUNK_BYTES;
         static_for<FRAGMENTS>([&](auto jc) __attribute__((always_inline)) {
             constexpr int j = decltype(jc)::value;
@@ -125,8 +135,9 @@ __global__ __launch_bounds__(NW * WAVE) void linear_wide_kernel(
             }
         });
     };
-    auto put_rows = [&](int buf, int chunk, auto slot) __attribute__((always_inline)) {
+    auto put_rows = [&](int buf, int logical, auto slot) __attribute__((always_inline)) {
         constexpr int s = decltype(slot)::value;
+        const int chunk = turned(logical);
         const bool in_k = EXACT || chunk * WIDE_CHUNK + x_piece * 8 < K;
 #pragma unroll
         for (int i = 0; i < XS; ++i) {
