@@ -394,7 +394,7 @@ def wide_pays(M: int, N: int, K: int, gated: bool = False, planes_ok: bool = Fal
 
 
 MID_TOKENS = 256      # rows of one block of the kernel whose operands both cross LDS
-MID_FROM = 32         # above this many rows it beats the kernel that keeps the weights in registers
+MID_FROM = 16         # above this many rows it serves (up to 16: the stream whose activations stay in registers)
 MID_CHUNK = 64        # it walks over K in steps of this many
 
 
@@ -402,10 +402,11 @@ def mid_pays(M: int, N: int, K: int, planes_ok: bool = False, gated: bool = Fals
              out_dtype: torch.dtype = BF16) -> bool:
     """Whether the kernel that brings both operands through rings in LDS serves this product of bfloat16 operands.
 
-    33 to 128 rows (decode steps of many sequences, short prompts): wherever its blocks fill the chip (for few weight
+    17 to 128 rows (decode steps of many sequences, short prompts): wherever its blocks fill the chip (for few weight
     rows that needs a reader that takes planes).  Measured at Qwen3-8B's shapes (us, this kernel against that one): 64 rows gate/up gated 46
     and 49, down 25 and 27, output projection 11 and 14, q/k/v 16 and 17, head 231 and 275; 128 rows 47 and 67, 30 and
-    36, 14 and 17, 19 and 21, 273 and 338 (the tiled kernel 289); 32 rows 45 and 41, 23 and 24, 10 and 11, 15 and 14.
+    36, 14 and 17, 19 and 21, 273 and 338 (the tiled kernel 289); 32 rows 42 and 40, 22 and 23, 10 and 11, 14 and 14,
+    222 and 252 (a decode step of 32 sequences at Qwen3-32B's sizes 20.7 against 21.3 ms).
 
     129 to 256 rows (short prompts): where the weight rows are so few that it cuts K into planes; the library's tiles
     leave compute units idle there.  Own against library at 256 rows: q/k/v 29 and 40, output projection 23 and 24,

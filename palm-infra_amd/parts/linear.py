@@ -2,9 +2,12 @@
 
   float32 run, or a 32-bit weight under bfloat16 activations   the exact FMA kernel
   bfloat16 x bfloat16, up to 16 rows (decode)                   the matrix-core kernel for thin products
-  bfloat16 x bfloat16, 17 to 32 rows (decode batches)           the matrix-core kernel that shares the rows through LDS
-  bfloat16 x bfloat16, 33 to 256 rows (large decode batches,    the kernel that brings both operands through rings in
-  short prompts)                                                LDS, where it beats the others (ops.mid_pays)
+  bfloat16 x bfloat16, 17 to 256 rows (decode batches, short    the kernel that brings both operands through rings in
+  prompts)                                                      LDS, where it beats the others (ops.mid_pays); where
+                                                                it does not serve (K no multiple of 64, few weight
+                                                                rows), up to 128 rows, the kernel that shares the
+                                                                rows through LDS, a strip of weights in each wave's
+                                                                registers
   bfloat16 x bfloat16, many rows (prompts)                      the BLAS library, as the reference's GPU path
                                                                 does for its products (engine/cuda_matmul.cu:245-260)
 
@@ -19,7 +22,7 @@ import torch
 from ..kernels import ops
 from .residual import Prenormed
 
-# Up to this many rows the kernel that streams the weight past one block of 16 rows serves; from 33 to 256 rows the
+# Up to this many rows the kernel that streams the weight past one block of 16 rows serves; from 17 to 256 rows the
 # kernel with rings in LDS where it pays (ops.mid_pays); else, up to 128 rows, the kernel that shares the rows through
 # LDS, where it has blocks enough to fill the chip (ops.wide_pays), and for every product with a float32 result; else
 # the library.

@@ -260,11 +260,11 @@ def test_linear_mid_refuses_what_it_does_not_serve(ops):
     a, w = rand(130, 72).to(DEV), rand(96, 72).to(DEV)
     with pytest.raises((KernelError, ValueError), match="64"):
         ops.linear_mid(a, w, BF16)
-    assert not ops.mid_pays(130, 96, 72) and not ops.mid_pays(32, 4096, 4096, planes_ok=True)
+    assert not ops.mid_pays(130, 96, 72) and not ops.mid_pays(16, 4096, 4096, planes_ok=True)
     assert not ops.mid_pays(300, 4096, 4096, planes_ok=True)
     assert ops.mid_pays(200, 4096, 4096, planes_ok=True) and not ops.mid_pays(200, 4096, 4096, planes_ok=False)
     assert not ops.mid_pays(200, 24576, 4096, planes_ok=True)           # weight rows enough: no planes, the library's
-    # 33 to 128 rows: wherever the blocks fill the chip
+    # 17 to 128 rows: wherever the blocks fill the chip
     assert ops.mid_pays(64, 24576, 4096, gated=True) and ops.mid_pays(100, 4096, 4096, planes_ok=True)
     assert not ops.mid_pays(100, 4096, 4096, planes_ok=False) and not ops.mid_pays(64, 96, 128)
     assert ops.mid_pays(128, 151936, 4096, out_dtype=F32) and ops.mid_pays(64, 151936, 4096, out_dtype=F32)
@@ -279,7 +279,7 @@ def test_a_short_prompts_projections_take_the_kernel_with_rings(ops, monkeypatch
     monkeypatch.setattr(ops, "linear_mid", lambda *a, **k: (calls.append(a[0].shape[0]), real(*a, **k))[1])
     w = rand(6144, 1024, seed=1, scale=0.5)
     lin = Linear(w.to(DEV))
-    for M, expect in ((200, True), (256, True), (128, True), (40, True), (32, False), (257, False)):
+    for M, expect in ((200, True), (256, True), (128, True), (40, True), (17, True), (16, False), (257, False)):
         x = rand(M, 1024, seed=M)
         calls.clear()
         got = lin(x.to(DEV), planes_ok=True)
