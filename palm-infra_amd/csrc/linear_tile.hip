@@ -1,9 +1,9 @@
-// C[M, N] = X[M, K] . W[N, K]^T for many rows (prompts, decode steps of more than 64 sequences): bfloat16
-// operands on the matrix cores, 32-bit accumulation.  The product is the reference's matmul
-// (kernels/matmul_dense.cpp:939-953), which its GPU path hands to a library (engine/cuda_matmul.cu:245-260);
-// this kernel is here for what a library call cannot do: an epilogue that applies the gated activation, or
-// adds the product to the residual stream and prepares the next norm, so that neither [M, 2I] nor the branch
-// output ever goes to memory, and tiles sized for some hundred rows, where the weight should go by once.
+// C[M, N] = X[M, K] . W[N, K]^T for many rows: bfloat16 operands on the matrix cores, 32-bit accumulation.  The
+// product is the reference's matmul (kernels/matmul_dense.cpp:939-953), which its GPU path hands to a library
+// (engine/cuda_matmul.cu:245-260), and so does this engine for a prompt's products.  This kernel is here for what
+// that library call cannot give: a float32 result from bfloat16 operands, the logits at many places of a prompt.
+// (It once had epilogues that applied the gated activation or added the product to the residual stream; for many
+// rows the library's kernel with a pass of its own after it was the faster way, and they are gone.)
 //
 // Tiling.  A block of eight waves owns TOK tokens x FEAT features and walks over K (or, with K cut into ranges, over
 // its range) in stages of 64.  A stage of both operands lies in LDS as rows of 128 bytes (64 k-values: a whole
@@ -18,7 +18,7 @@
 // flight; a long prompt's operands are far larger than L2), 11 to 12 TB/s for the chip; a tile of 256 x 256 needs 128 KB for every 64 k-values, which is 270 us for the gate/up product of
 // 2,048 rows, about what the library's kernel of the same tile takes in all.  This kernel overlaps its products
 // and its reads less well (360 us), so prompts keep the library; it serves where a library call cannot: float32
-// results of many rows (logits at many places), and the epilogues below.
+// results of many rows (logits at many places).
 // MFMA 32x32x16: the A operand is 32 weight rows (features), the B operand 32 activation rows (tokens); a lane
 // of the result holds one token and 16 features in runs of four, so results leave as 8-byte (bfloat16) or
 // 16-byte (float32) pieces of a token's row.
@@ -35,8 +35,6 @@ PALM_DEFINE_LAST_ERROR()
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-enum TileEpilogue : int { TILE_STORE = 0, TILE_SWIGLU = 1, TILE_RESIDUAL = 2 };
-
 constexpr int TK = 64;                       // k-values of a stage
 constexpr int ROW_BYTES = TK * 2;            // a row of a stage in LDS
 constexpr int ROW_CHUNKS = ROW_BYTES / 16;   // 16-byte chunks of such a row
@@ -46,16 +44,6 @@ constexpr int LDS_BYTES = 160 * 1024;
 constexpr int TILE_WAVES = 8;
 constexpr int TILE_THREADS = TILE_WAVES * WAVE;
 constexpr int DIES = 8;
-
-struct TileNorm {
-    const float* ss_in;      // [M, pieces_in]: the rows of X lack the factor 1 / sqrt(sum / width_in + eps_in); or null
-    int pieces_in;
-    float eps_in;
-    int width_in;
-    float* resid;            // TILE_RESIDUAL: [M, N] float32, updated in place
-    const float* w_out;      // [N]: the next norm's weight
-    float* ss_out;           // [M, feature tiles]: each tile's share of the rows' sums of squares
-};
 
 __device__ __forceinline__ void row_chunk_into_lds(const void* from, uint32_t lds_base) {
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(from), "s"(lds_base) : "m0", "memory");
@@ -67,10 +55,10 @@ template <int N> __device__ __forceinline__ void all_but_the_youngest_have_arriv
     __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
 }
 
-template <int TOK, int FEAT, int WAVES_F, typename TC, int EPI>
+template <int TOK, int FEAT, int WAVES_F, typename TC>
 __global__ __launch_bounds__(TILE_THREADS) void linear_tile_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
                                                                    TC* __restrict__ C, int M, int N, int K, int tiles_t,
-                                                                   int tiles_f, TileNorm norm) {
+                                                                   int tiles_f) {
     constexpr int WAVES_T = TILE_WAVES / WAVES_F;
     constexpr int NF = FEAT / WAVES_F / 32, NT = TOK / WAVES_T / 32;
     constexpr int ROWS = FEAT + TOK, STAGE = ROWS * ROW_BYTES, PER_WAVE = ROWS / ROWS_AN_INSTRUCTION / TILE_WAVES;
@@ -78,7 +66,6 @@ __global__ __launch_bounds__(TILE_THREADS) void linear_tile_kernel(const bf16_t*
     constexpr int AHEAD = RING - 1;                                                                      // of which on their way
     static_assert(FEAT % (32 * WAVES_F) == 0 && TOK % (32 * WAVES_T) == 0 && ROWS % (ROWS_AN_INSTRUCTION * TILE_WAVES) == 0,
                   "tile and waves do not fit");
-    static_assert(EPI != TILE_SWIGLU || NF % 2 == 0, "a gated tile needs gate and up features in every wave");
     static_assert(RING >= 2 && (AHEAD - 1) * PER_WAVE < 64, "the ring does not fit LDS or the load counter");
     __shared__ __attribute__((aligned(1024))) char lds[RING * STAGE];
 
@@ -89,11 +76,10 @@ __global__ __launch_bounds__(TILE_THREADS) void linear_tile_kernel(const bf16_t*
     // this block's range of K, in stages, and the plane its sums go to
     const int all_stages = K / TK, per_range = (all_stages + (int)gridDim.y - 1) / (int)gridDim.y;
     const int first_stage = blockIdx.y * per_range, stages = min(per_range, all_stages - first_stage);
-    if (EPI == TILE_STORE) C += (size_t)blockIdx.y * M * N;
+    C += (size_t)blockIdx.y * M * N;
     const int tile_t = pid % tiles_t, tile_f = pid / tiles_t;       // the token tiles of a feature tile side by side
     const int t0 = tile_t * TOK;
-    const int out_feats = EPI == TILE_SWIGLU ? N / 2 : N;           // features of the result
-    const int f0 = tile_f * (EPI == TILE_SWIGLU ? FEAT / 2 : FEAT);
+    const int f0 = tile_f * FEAT;
 
     const int lane = threadIdx.x % WAVE;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
@@ -107,10 +93,7 @@ __global__ __launch_bounds__(TILE_THREADS) void linear_tile_kernel(const bf16_t*
         const int chunk = (lane % ROW_CHUNKS) ^ ((R >> 1) & (ROW_CHUNKS - 1));
         const bf16_t* row;
         if (R < FEAT) {
-            int wrow;
-            if (EPI == TILE_SWIGLU) wrow = R < FEAT / 2 ? min(f0 + R, out_feats - 1) : out_feats + min(f0 + R - FEAT / 2, out_feats - 1);
-            else wrow = min(f0 + R, N - 1);
-            row = W + (size_t)wrow * K;
+            row = W + (size_t)min(f0 + R, N - 1) * K;
         } else {
             row = X + (size_t)min(t0 + R - FEAT, M - 1) * K;
         }
@@ -127,10 +110,7 @@ __global__ __launch_bounds__(TILE_THREADS) void linear_tile_kernel(const bf16_t*
     int w_off[NF], x_off[NT], cs[SUB_STEPS];
 #pragma unroll
     for (int f = 0; f < NF; ++f) {
-        int row;
-        if (EPI == TILE_SWIGLU) row = (f / (NF / 2)) * (FEAT / 2) + wave_f * (FEAT / 2 / WAVES_F) + (f % (NF / 2)) * 32 + lane % 32;
-        else row = wave_f * (FEAT / WAVES_F) + f * 32 + lane % 32;
-        w_off[f] = row * ROW_BYTES;
+        w_off[f] = (wave_f * (FEAT / WAVES_F) + f * 32 + lane % 32) * ROW_BYTES;
     }
 #pragma unroll
     for (int t = 0; t < NT; ++t) x_off[t] = (FEAT + wave_t * (TOK / WAVES_T) + t * 32 + lane % 32) * ROW_BYTES;
@@ -188,144 +168,52 @@ __global__ __launch_bounds__(TILE_THREADS) void linear_tile_kernel(const bf16_t*
         }
         slot = slot + 1 == RING ? 0 : slot + 1;
     }
-    __syncthreads();                                           // the epilogue may use LDS: everyone is past the last stage
 
     // ---- epilogue.  Element v of a result tile: token lane % 32, feature 8 (v / 4) + 4 (lane / 32) + v % 4.
-    int tok[NT];
-    float factor[NT];
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
-        tok[t] = t0 + wave_t * (TOK / WAVES_T) + t * 32 + lane % 32;
-        factor[t] = 1.0f;
-        if (norm.ss_in) {                                      // the pieces of the row's sum of squares, in their order
-            const float* p = norm.ss_in + (size_t)min(tok[t], M - 1) * norm.pieces_in;
-            float sum = 0.f;
-            for (int i = 0; i < norm.pieces_in; ++i) sum += p[i];
-            factor[t] = 1.0f / sqrtf(sum / (float)norm.width_in + norm.eps_in);
-        }
-    }
-    if (EPI == TILE_SWIGLU) {
+        const int tok = t0 + wave_t * (TOK / WAVES_T) + t * 32 + lane % 32;
+        if (tok >= M) continue;
 #pragma unroll
-        for (int f = 0; f < NF / 2; ++f)
-#pragma unroll
-            for (int t = 0; t < NT; ++t)
-#pragma unroll
-                for (int q4 = 0; q4 < 4; ++q4) {
-                    const int feat = f0 + wave_f * (FEAT / 2 / WAVES_F) + f * 32 + 8 * q4 + 4 * (lane / 32);
-                    float o[4];
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const float gate = acc[f][t][4 * q4 + i] * factor[t], up = acc[f + NF / 2][t][4 * q4 + i] * factor[t];
-                        o[i] = gate / (1.0f + __expf(-gate)) * up;
-                    }
-                    if (tok[t] < M) {
-                        TC* dst = C + (size_t)tok[t] * out_feats + feat;
-                        if (feat + 3 < out_feats && out_feats % 4 == 0) {
-                            if constexpr (sizeof(TC) == 2) {
-                                uint2 four;
-                                four.x = (uint32_t)f32_to_bf16(o[0]).bits | ((uint32_t)f32_to_bf16(o[1]).bits << 16);
-                                four.y = (uint32_t)f32_to_bf16(o[2]).bits | ((uint32_t)f32_to_bf16(o[3]).bits << 16);
-                                *reinterpret_cast<uint2*>(dst) = four;
-                            } else {
-                                *reinterpret_cast<float4*>(dst) = make_float4(o[0], o[1], o[2], o[3]);
-                            }
-                        } else {
-#pragma unroll
-                            for (int i = 0; i < 4; ++i)
-                                if (feat + i < out_feats) dst[i] = from_float<TC>(o[i]);
-                        }
-                    }
-                }
-        return;
-    }
-    float sq[NT];
-#pragma unroll
-    for (int t = 0; t < NT; ++t) sq[t] = 0.f;
-#pragma unroll
-    for (int f = 0; f < NF; ++f)
-#pragma unroll
-        for (int t = 0; t < NT; ++t)
+        for (int f = 0; f < NF; ++f)
 #pragma unroll
             for (int q4 = 0; q4 < 4; ++q4) {
                 const int feat = f0 + wave_f * (FEAT / WAVES_F) + f * 32 + 8 * q4 + 4 * (lane / 32);
-                float o[4];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) o[i] = acc[f][t][4 * q4 + i] * factor[t];
-                const bool whole = feat + 3 < N && N % 4 == 0;
-                if (tok[t] < M && feat < N) {
-                    const size_t at = (size_t)tok[t] * N + feat;
-                    if (EPI == TILE_RESIDUAL) {
-                        if (whole) {
-                            const float4 xo = *reinterpret_cast<const float4*>(norm.resid + at);
-                            const float4 wn = *reinterpret_cast<const float4*>(norm.w_out + feat);
-                            o[0] += xo.x; o[1] += xo.y; o[2] += xo.z; o[3] += xo.w;
-                            *reinterpret_cast<float4*>(norm.resid + at) = make_float4(o[0], o[1], o[2], o[3]);
-                            sq[t] += o[0] * o[0] + o[1] * o[1] + o[2] * o[2] + o[3] * o[3];
-                            o[0] *= wn.x; o[1] *= wn.y; o[2] *= wn.z; o[3] *= wn.w;
-                        } else {
-#pragma unroll
-                            for (int i = 0; i < 4; ++i)
-                                if (feat + i < N) {
-                                    o[i] += norm.resid[at + i];
-                                    norm.resid[at + i] = o[i];
-                                    sq[t] += o[i] * o[i];
-                                    o[i] *= norm.w_out[feat + i];
-                                }
-                        }
-                    }
-                    TC* dst = C + at;
-                    if (whole) {
-                        if constexpr (sizeof(TC) == 2) {
-                            uint2 four;
-                            four.x = (uint32_t)f32_to_bf16(o[0]).bits | ((uint32_t)f32_to_bf16(o[1]).bits << 16);
-                            four.y = (uint32_t)f32_to_bf16(o[2]).bits | ((uint32_t)f32_to_bf16(o[3]).bits << 16);
-                            *reinterpret_cast<uint2*>(dst) = four;
-                        } else {
-                            *reinterpret_cast<float4*>(dst) = make_float4(o[0], o[1], o[2], o[3]);
-                        }
+                if (feat >= N) continue;
+                const float o[4] = {acc[f][t][4 * q4], acc[f][t][4 * q4 + 1], acc[f][t][4 * q4 + 2], acc[f][t][4 * q4 + 3]};
+                TC* dst = C + (size_t)tok * N + feat;
+                if (feat + 3 < N && N % 4 == 0) {
+                    if constexpr (sizeof(TC) == 2) {
+                        uint2 four;
+                        four.x = (uint32_t)f32_to_bf16(o[0]).bits | ((uint32_t)f32_to_bf16(o[1]).bits << 16);
+                        four.y = (uint32_t)f32_to_bf16(o[2]).bits | ((uint32_t)f32_to_bf16(o[3]).bits << 16);
+                        *reinterpret_cast<uint2*>(dst) = four;
                     } else {
-#pragma unroll
-                        for (int i = 0; i < 4; ++i)
-                            if (feat + i < N) dst[i] = from_float<TC>(o[i]);
+                        *reinterpret_cast<float4*>(dst) = make_float4(o[0], o[1], o[2], o[3]);
                     }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        if (feat + i < N) dst[i] = from_float<TC>(o[i]);
                 }
             }
-    if (EPI == TILE_RESIDUAL) {
-        // a token's sum of squares over this tile's features: the two halves of a wave, then the waves that share
-        // the token, in a fixed order
-        float* red = reinterpret_cast<float*>(lds);               // [WAVES_F][TOK]; every wave is past its last stage
-#pragma unroll
-        for (int t = 0; t < NT; ++t) {
-            const float both = sq[t] + __shfl_xor(sq[t], 32, WAVE);
-            if (lane < 32) red[wave_f * TOK + wave_t * (TOK / WAVES_T) + t * 32 + lane] = both;
-        }
-        __syncthreads();
-        for (int i = threadIdx.x; i < TOK; i += TILE_THREADS) {
-            float sum = 0.f;
-#pragma unroll
-            for (int w = 0; w < WAVES_F; ++w) sum += red[w * TOK + i];
-            if (t0 + i < M) norm.ss_out[(size_t)(t0 + i) * tiles_f + tile_f] = sum;
-        }
     }
 }
 
 // ---- launch -----------------------------------------------------------------------------------------
 constexpr int TILE_FEAT = 256;
 
-template <int TOK, int WAVES_F, typename TC, int EPI>
-static void launch_tile(hipStream_t stream, const void* x, const void* w, void* c, int M, int N, int K, int parts,
-                        const TileNorm& norm) {
-    const int feats_a_tile = EPI == TILE_SWIGLU ? TILE_FEAT / 2 : TILE_FEAT;
-    const int out_feats = EPI == TILE_SWIGLU ? N / 2 : N;
-    const int tiles_t = (M + TOK - 1) / TOK, tiles_f = (out_feats + feats_a_tile - 1) / feats_a_tile;
+template <int TOK, int WAVES_F, typename TC>
+static void launch_tile(hipStream_t stream, const void* x, const void* w, void* c, int M, int N, int K, int parts) {
+    const int tiles_t = (M + TOK - 1) / TOK, tiles_f = (N + TILE_FEAT - 1) / TILE_FEAT;
     const int total = tiles_t * tiles_f, blocks = (total + DIES - 1) / DIES * DIES;
-    linear_tile_kernel<TOK, TILE_FEAT, WAVES_F, TC, EPI><<<dim3(blocks, parts), TILE_THREADS, 0, stream>>>(
-        (const bf16_t*)x, (const bf16_t*)w, (TC*)c, M, N, K, tiles_t, tiles_f, norm);
+    linear_tile_kernel<TOK, TILE_FEAT, WAVES_F, TC><<<dim3(blocks, parts), TILE_THREADS, 0, stream>>>(
+        (const bf16_t*)x, (const bf16_t*)w, (TC*)c, M, N, K, tiles_t, tiles_f);
 }
 
 // How many tokens a block takes: 256 where that still gives most compute units a block, else 128.
-static int tile_tokens(int M, int out_feats, int feats_a_tile, int parts) {
-    const int tiles_f = (out_feats + feats_a_tile - 1) / feats_a_tile;
+static int tile_tokens(int M, int N, int parts) {
+    const int tiles_f = (N + TILE_FEAT - 1) / TILE_FEAT;
     if (M <= 128) return 128;
     return ((M + 255) / 256) * tiles_f * parts >= 192 ? 256 : 128;
 }
@@ -340,52 +228,26 @@ static int tile_parts(int M, int N, int K) {
 }
 PALM_API int palm_linear_tile_parts(int M, int N, int K) { return tile_parts(M, N, K); }
 
-template <typename TC, int EPI>
-static void dispatch_tile(hipStream_t stream, const void* x, const void* w, void* c, int M, int N, int K, int parts,
-                          const TileNorm& norm) {
-    const int out_feats = EPI == TILE_SWIGLU ? N / 2 : N;
-    if (tile_tokens(M, out_feats, EPI == TILE_SWIGLU ? TILE_FEAT / 2 : TILE_FEAT, parts) == 256)
-        launch_tile<256, 2, TC, EPI>(stream, x, w, c, M, N, K, parts, norm);
-    else
-        launch_tile<128, 4, TC, EPI>(stream, x, w, c, M, N, K, parts, norm);
+template <typename TC>
+static void dispatch_tile(hipStream_t stream, const void* x, const void* w, void* c, int M, int N, int K, int parts) {
+    if (tile_tokens(M, N, parts) == 256) launch_tile<256, 2, TC>(stream, x, w, c, M, N, K, parts);
+    else launch_tile<128, 4, TC>(stream, x, w, c, M, N, K, parts);
 }
 
-// The pieces a row's sum of squares comes in (TILE_RESIDUAL): one for each tile of 256 features.
-PALM_API int palm_linear_tile_pieces(int N) { return (N + TILE_FEAT - 1) / TILE_FEAT; }
-
-// x [M, K] bfloat16, w [N, K] bfloat16, K a multiple of 64.
-//   TILE_STORE:    c [M, N] bfloat16 or float32; or, with parts > 1 (at most palm_linear_tile_parts(M, N, K)), float32
-//                  planes [parts, M, N], each the sum over one range of K, for a reader that adds them in their order.
-//   TILE_SWIGLU:   w is [gate rows | up rows]; c [M, N / 2] = silu(x gate^T) * (x up^T).
-//   TILE_RESIDUAL: resid [M, N] float32 += x w^T; c [M, N] bfloat16 = resid * w_out (the next norm's output but for
-//                  its row factor); ss_out [M, palm_linear_tile_pieces(N)] the pieces of each row's sum of squares.
-// ss_in [M, pieces_in] with eps_in: the rows of x lack the factor 1 / sqrt(sum of pieces / K + eps_in), which the
-// result rows get instead.
+// x [M, K] bfloat16, w [N, K] bfloat16, K a multiple of 64; c [M, N] bfloat16 or float32; or, with parts > 1 (at most
+// palm_linear_tile_parts(M, N, K)), float32 planes [parts, M, N], each the sum over one range of K, for a reader that
+// adds them in their order.
 PALM_API int palm_linear_tile(hipStream_t stream, const void* x, const void* w, void* c, int c_dtype, int M, int N, int K,
-                              int epilogue, int parts, const float* ss_in, int pieces_in, float eps_in, float* resid,
-                              const float* w_out, float* ss_out) {
+                              int parts) {
     PALM_CHECK(M >= 0 && N > 0 && K > 0, "linear_tile: M=%d N=%d K=%d", M, N, K);
     PALM_CHECK(K % TK == 0, "linear_tile: K = %d is not a multiple of %d", K, TK);
-    PALM_CHECK(parts >= 1 && (parts == 1 || (epilogue == TILE_STORE && c_dtype == PALM_F32 && parts <= 4 && K / TK >= parts)),
-               "linear_tile: %d planes of partial sums (they are float32, of a plain product, at most four)", parts);
-    PALM_CHECK(epilogue >= TILE_STORE && epilogue <= TILE_RESIDUAL, "linear_tile: epilogue %d", epilogue);
-    PALM_CHECK(epilogue != TILE_SWIGLU || N % 2 == 0, "linear_tile: a gated product needs an even N, got %d", N);
+    PALM_CHECK(parts >= 1 && (parts == 1 || (c_dtype == PALM_F32 && parts <= 4 && K / TK >= parts)),
+               "linear_tile: %d planes of partial sums (they are float32, at most four)", parts);
     PALM_CHECK(c_dtype == PALM_BF16 || c_dtype == PALM_F32, "linear_tile: result type %d", c_dtype);
     PALM_CHECK(((uintptr_t)x | (uintptr_t)w | (uintptr_t)c) % 16 == 0, "linear_tile: operands must be 16-byte aligned");
-    PALM_CHECK(!ss_in || pieces_in > 0, "linear_tile: %d pieces of the rows' sums of squares", pieces_in);
-    PALM_CHECK(epilogue != TILE_RESIDUAL || (resid && w_out && ss_out && c_dtype == PALM_BF16 && ((uintptr_t)resid | (uintptr_t)w_out) % 16 == 0),
-               "linear_tile: adding to the residual stream needs the stream, the next norm's weight, room for the sums of "
-               "squares and a bfloat16 result");
     PALM_CHECK((double)M * N < 2.0e9 * 4, "linear_tile: the result is beyond this kernel's index range");
     if (M == 0) return 0;
-    TileNorm norm{ss_in, pieces_in, eps_in, K, resid, w_out, ss_out};
-    if (epilogue == TILE_SWIGLU) {
-        PALM_DTYPE_SWITCH(c_dtype, TC, dispatch_tile<TC, TILE_SWIGLU>(stream, x, w, c, M, N, K, 1, norm));
-    } else if (epilogue == TILE_RESIDUAL) {
-        dispatch_tile<bf16_t, TILE_RESIDUAL>(stream, x, w, c, M, N, K, 1, norm);
-    } else {
-        PALM_DTYPE_SWITCH(c_dtype, TC, dispatch_tile<TC, TILE_STORE>(stream, x, w, c, M, N, K, parts, norm));
-    }
+    PALM_DTYPE_SWITCH(c_dtype, TC, dispatch_tile<TC>(stream, x, w, c, M, N, K, parts));
     PALM_LAUNCHED();
     return 0;
 }

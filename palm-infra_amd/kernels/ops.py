@@ -43,9 +43,7 @@ _SIGNATURES = {
     "palm_linear_mid": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int],
     "palm_linear_mid_parts": [c_int, c_int, c_int, c_int],
     "palm_linear_mid_blocks": [c_int, c_int, c_int, c_int, c_int],
-    "palm_linear_tile": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int,
-                         c_float, c_void_p, c_void_p, c_void_p],
-    "palm_linear_tile_pieces": [c_int],
+    "palm_linear_tile": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int],
     "palm_linear_tile_parts": [c_int, c_int, c_int],
     "palm_argmax": [c_void_p, c_void_p, c_int, c_int, c_void_p],
     "palm_apply_penalties": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_float, c_float, c_float],
@@ -529,8 +527,8 @@ def linear_thin(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, gated:
     if M > WIDE_TOKENS or (M > WIDE_FLOAT32_TOKENS and out_dtype == F32 and not planes_ok):
         # a float32 result for many rows (logits at many places): the tiled kernel, which reads the weight once for
         # every 256 rows; where K is no whole number of its stages, 64 rows at a time
-        if tile_serves(a, w):
-            return linear_tile(a, w, out_dtype, gated=gated)
+        if tile_serves(a, w) and not gated:
+            return linear_tile(a, w, out_dtype)
         return torch.cat([linear_thin(a[r0:r0 + WIDE_FLOAT32_TOKENS], w, out_dtype, gated=gated)
                           for r0 in range(0, M, WIDE_FLOAT32_TOKENS)])
     # more rows than one block of 16: the kernel that shares the activations through LDS
@@ -552,56 +550,22 @@ def tile_serves(a: torch.Tensor, w: torch.Tensor) -> bool:
     return a.dtype == BF16 and w.dtype == BF16 and a.shape[1] % TILE_K == 0 and a.shape[1] == w.shape[1]
 
 
-def _tile_row_ss(what: str, a: torch.Tensor, row_ss) -> int:
-    if row_ss is None:
-        return 0
-    _dev(what, a, row_ss)
-    _need(row_ss.dim() == 2 and row_ss.shape[0] == a.shape[0] and row_ss.dtype == F32 and row_ss.shape[1] > 0,
-          f"{what}: sums of squares {tuple(row_ss.shape)} {row_ss.dtype} for {a.shape[0]} rows")
-    return row_ss.shape[1]
-
-
-def linear_tile(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, gated: bool = False, planes_ok: bool = False,
-                row_ss=None, row_eps: float = 0.0) -> torch.Tensor:
+def linear_tile(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, planes_ok: bool = False) -> torch.Tensor:
     """bfloat16 a [M, K] . w [N, K]^T for many rows, tiled over the matrix cores; result bfloat16 or float32.
-    ``gated``: w is [gate rows | up rows] and the result is silu(a gate^T) * (a up^T), [M, N/2].
     ``planes_ok``: the caller takes float32 planes [P, M, N] of partial sums (see linear_thin); the kernel then
-    cuts K into ranges where the tiles alone would leave most of the chip without work.
-    ``row_ss`` with ``row_eps``: the rows of a lack their norm's factor (see linear_thin)."""
+    cuts K into ranges where the tiles alone would leave most of the chip without work."""
     _dev("linear_tile", a, w)
     _need(a.dim() == 2 and w.dim() == 2 and tile_serves(a, w), f"linear_tile: a {tuple(a.shape)} {a.dtype}, w {tuple(w.shape)} "
           f"{w.dtype} (bfloat16, one inner size, a multiple of {TILE_K})")
     M, K = a.shape
     N = w.shape[0]
-    _need(not gated or N % 2 == 0, f"linear_tile: a gated product needs an even number of weight rows, got {N}")
-    pieces = _tile_row_ss("linear_tile", a, row_ss)
-    parts = core().palm_linear_tile_parts(M, N, K) if planes_ok and not gated and row_ss is None else 1
+    parts = core().palm_linear_tile_parts(M, N, K) if planes_ok else 1
     if parts > 1:
         out = torch.empty((parts, M, N), dtype=F32, device=a.device)
     else:
-        out = torch.empty((M, N // 2 if gated else N), dtype=out_dtype, device=a.device)
-    library.call(core(), "palm_linear_tile", _stream(), _p(a), _p(w), _p(out), _code(out, "linear_tile out"), M, N, K,
-                 1 if gated else 0, parts, _p(row_ss), pieces, float(row_eps), None, None, None)
+        out = torch.empty((M, N), dtype=out_dtype, device=a.device)
+    library.call(core(), "palm_linear_tile", _stream(), _p(a), _p(w), _p(out), _code(out, "linear_tile out"), M, N, K, parts)
     return out
-
-
-def linear_tile_into_residual(a: torch.Tensor, w: torch.Tensor, x: torch.Tensor, norm_w: torch.Tensor, row_ss=None,
-                              row_eps: float = 0.0):
-    """A branch's last product and what follows it, for many rows: x += a . w^T (x float32 [M, N], in place);
-    returns (x * norm_w rounded to bfloat16, the pieces [M, N/256] of each row's sum of squares of x)."""
-    _dev("linear_tile_into_residual", a, w, x, norm_w)
-    _need(a.dim() == 2 and w.dim() == 2 and tile_serves(a, w), f"linear_tile_into_residual: a {tuple(a.shape)} {a.dtype}, "
-          f"w {tuple(w.shape)} {w.dtype}")
-    M, K = a.shape
-    N = w.shape[0]
-    _need(x.shape == (M, N) and x.dtype == F32 and x.is_contiguous(), f"linear_tile_into_residual: residual {tuple(x.shape)} {x.dtype}")
-    _need(norm_w.shape == (N,) and norm_w.dtype == F32, "linear_tile_into_residual: the norm's weight is float32 [N]")
-    pieces = _tile_row_ss("linear_tile_into_residual", a, row_ss)
-    values = torch.empty((M, N), dtype=BF16, device=a.device)
-    ss = torch.empty((M, core().palm_linear_tile_pieces(N)), dtype=F32, device=a.device)
-    library.call(core(), "palm_linear_tile", _stream(), _p(a), _p(w), _p(values), _code(values, "values"), M, N, K, 2, 1,
-                 _p(row_ss), pieces, float(row_eps), _p(x), _p(norm_w), _p(ss))
-    return values, ss
 
 
 # ---- attention on the matrix cores (one library for each head size) ---------------------------------

@@ -343,46 +343,6 @@ def test_linear_tile_orientation_and_every_k_once(ops):
     assert torch.equal(got, ref)
 
 
-@pytest.mark.parametrize("M", [65, 200, 300])
-@pytest.mark.parametrize("I,K", [(128, 64), (176, 128), (1536, 512), (4500, 2048), (300, 3008)])
-def test_linear_tile_gated(ops, M, I, K):
-    a, w = rand(M, K, seed=M), rand(2 * I, K, seed=I, scale=0.3)
-    g, u = P.linear(a, w[:I]), P.linear(a, w[I:])
-    ref = g / (1 + torch.exp(-g)) * u
-    got = ops.linear_tile(a.to(DEV), w.to(DEV), F32, gated=True).cpu()
-    assert got.shape == (M, I)
-    scale = float(ref.abs().max())
-    assert torch.allclose(got.double(), ref, atol=2e-5 * scale * (K ** 0.5)), float((got.double() - ref).abs().max()) / scale
-    swapped = u / (1 + torch.exp(-u)) * g
-    assert not torch.allclose(got.double(), swapped, atol=1e-2 * scale)
-
-
-@pytest.mark.parametrize("M", [70, 256, 300])
-@pytest.mark.parametrize("N,K", [(256, 64), (4096, 4096), (1000, 1088), (520, 12288)])
-def test_linear_tile_into_the_residual_stream_and_on_with_the_row_factor(ops, M, N, K):
-    """x += a W1^T with the next norm's elementwise part and sums of squares; then a product that takes such rows."""
-    eps = 1e-5
-    a, w1 = rand(M, K, seed=M), rand(N, K, seed=N, scale=0.1)
-    x0, nw = rand(M, N, seed=3, dtype=F32) * 3, rand(N, seed=4, dtype=F32) + 1.0
-    xd = x0.to(DEV)
-    values, ss = ops.linear_tile_into_residual(a.to(DEV), w1.to(DEV), xd, nw.to(DEV))
-    x_ref = x0.double() + P.linear(a, w1)
-    assert torch.allclose(xd.cpu().double(), x_ref, atol=2e-4 * (K ** 0.5), rtol=1e-5)
-    assert values.dtype == BF16 and ss.shape == (M, (N + 255) // 256)
-    assert torch.allclose(ss.cpu().double().sum(1), (x_ref ** 2).sum(1), rtol=1e-4)
-    assert torch.allclose(values.cpu().double(), x_ref * nw.double(), atol=3e-2, rtol=1e-2)
-    if N % 64 == 0:
-        for N2, gated in ((96, False), (2 * 176, True)):
-            w2 = rand(N2, N, seed=N2, scale=0.2)
-            got = ops.linear_tile(values, w2.to(DEV), F32, gated=gated, row_ss=ss, row_eps=eps).cpu().double()
-            normed = P.rms_norm(x_ref, nw.double(), eps)
-            want = P.linear(normed, w2)
-            if gated:
-                want = want[:, :N2 // 2] / (1 + torch.exp(-want[:, :N2 // 2])) * want[:, N2 // 2:]
-            scale = float(want.abs().max())
-            assert torch.allclose(got, want, atol=1.5e-2 * scale), (N2, gated, float((got - want).abs().max()), scale)
-
-
 def test_linear_tile_refuses_what_it_does_not_serve(ops):
     from palm_infra_amd.kernels import KernelError
     with pytest.raises(KernelError, match="multiple of 64"):
