@@ -36,7 +36,7 @@ constexpr int MID_WAVES = 4;
 constexpr int MID_THREADS = MID_WAVES * WAVE;
 constexpr int MID_CHUNK = 64;                   // k-values a step: a row of LDS is 128 bytes
 constexpr int MID_ROW_BYTES = MID_CHUNK * 2;
-constexpr int MID_MAX_STAGES = 6;
+constexpr int MID_MAX_STAGES = 4;    // (a decode step of 64 sequences: 8.04 ms with three, 7.83 with four, 7.87 with five, 7.90 with six)
 constexpr int MID_LDS_BYTES = 160 * 1024;
 constexpr int MID_MAX_PARTS = 4;
 constexpr int MID_UNITS = 256;                  // compute units of the chip
@@ -79,10 +79,9 @@ __global__ __launch_bounds__(MID_THREADS) void linear_mid_kernel(
     // The rings.  All loads come back in the order they went out, and one counter counts them all: a wait for the rows
     // of the next chunk is also a wait for every load asked for before them.  So what is still on its way after a
     // pass's wait is what was asked for after the younger of the next chunk's two operands, and the rings are as deep
-    // in flight as the shallower of them.  With 64 or 128 rows both rings have the same depth, as many chunks as LDS
-    // holds, up to six (64 rows x 128 weight rows: 6 x 24 KB, of which four are on their way after a wait; with three
-    // chunks of rows and five of weights only two chunks of weights were, 32 KB a compute unit, and the stream of
-    // weights alone took 46 us for 201 MB).  256 rows leave room for three chunks of rows and five of weights.
+    // in flight as the shallower of them.  With 64 or 128 rows both rings have the same depth, four chunks (64 rows x
+    // 128 weight rows: 4 x 24 KB, of which two are on their way after a wait).  256 rows leave room for three chunks
+    // of rows and five of weights.
     constexpr bool SAME = R != 256;
     constexpr int BOTH = (MID_LDS_BYTES / (MID_A_BYTES + W_BYTES)) < MID_MAX_STAGES ? (MID_LDS_BYTES / (MID_A_BYTES + W_BYTES)) : MID_MAX_STAGES;
     constexpr int A_STAGES = SAME ? BOTH : 3;
@@ -90,7 +89,7 @@ __global__ __launch_bounds__(MID_THREADS) void linear_mid_kernel(
     // loads asked for after the chunk that is due, see the loop
     constexpr int YOUNGER = SAME ? (A_STAGES - 2) * (MID_A_LOADS + W_LOADS) : W_LOADS + MID_A_LOADS + W_LOADS;
     constexpr int YOUNGER_AT_START = SAME ? (A_STAGES - 1) * (MID_A_LOADS + W_LOADS) : (W_STAGES - 1) * W_LOADS + 2 * MID_A_LOADS;
-    static_assert(A_STAGES >= 3 && W_STAGES >= 4 && YOUNGER_AT_START < 64, "the rings' depth and the counter's six bits");
+    static_assert(A_STAGES >= 3 && W_STAGES >= 3 && YOUNGER_AT_START < 64, "the rings' depth and the counter's six bits");
     __shared__ __attribute__((aligned(1024))) char a_lds[A_STAGES * MID_A_BYTES];
     __shared__ __attribute__((aligned(1024))) char w_lds[W_STAGES * W_BYTES];
 
