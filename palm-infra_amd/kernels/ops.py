@@ -652,10 +652,16 @@ def attention_decode(q, k_cache, v_cache, block_table, seq_slot, seq_start, nh: 
     return out
 
 
+DECODE_FUSED_ROWS = 96      # sequences up to which the q/k/v pass rides in the decode attention kernel
+
+
 def decode_fused_serves(qkv: torch.Tensor, hd: int, out_dtype, rotary_dim: int, pairing: int) -> bool:
     """Whether attention_decode_fused takes this step's q/k/v rows: bfloat16 attention on the matrix cores, a head
-    size and a rotation for which a rotation pair lies in one lane."""
-    if out_dtype != BF16 or hd not in MFMA_HEAD_DIMS:
+    size and a rotation for which a rotation pair lies in one lane, and not too many sequences: every wave of a
+    sequence's slices makes the queries anew, which for many sequences costs more than the pass of its own that it
+    saves (a step of Qwen3-8B's sizes, fused against apart: 64 sequences 7.80 and 7.93 ms, 96: 10.15 and 10.11,
+    128: 12.23 and 11.87)."""
+    if out_dtype != BF16 or hd not in MFMA_HEAD_DIMS or qkv.shape[-2] > DECODE_FUSED_ROWS:
         return False
     if not (qkv.dim() == 3 and qkv.dtype == F32 or qkv.dim() == 2 and qkv.dtype == BF16):
         return False
