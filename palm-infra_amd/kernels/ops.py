@@ -410,8 +410,8 @@ def mid_pays(M: int, N: int, K: int, planes_ok: bool = False, gated: bool = Fals
     leave compute units idle there.  Own against library at 256 rows: q/k/v 29 and 40, output projection 23 and 24,
     down 46 and 53; at 129 rows (library at 192) 23 and 34, 18 and 33, 39 and 88; the planes cost their readers about
     4 us each.  Not a product with weight rows enough for all compute units (gate/up at 256 rows: 70 against 65, gated
-    79 against 65 and the activation's pass of 8; every block then reads all rows again for 96 weight rows, and the
-    way from L2 into a compute unit, 60 to 80 GB/s when all of them pull, is as long as the arithmetic), and not more
+    72 to 79 against 65 and the activation's pass of 8; every block then reads all rows again for 96 weight rows, and
+    one wave a SIMD does not overlap those loads, the fragment reads from LDS and 39 us of arithmetic), and not more
     than 256 rows, where it ties (q/k/v 40 and 37, output projection 32 and 30, down 78 and 80 at 512 rows)."""
     if K % MID_CHUNK != 0 or not MID_FROM < M <= MID_TOKENS:
         return False
