@@ -49,6 +49,14 @@ __device__ __forceinline__ void mid_load_16_bytes_a_lane_into_lds(const void* ba
 template <int N> __device__ __forceinline__ void mid_wait_for_all_but_the_youngest_loads() {
     __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));          // s_waitcnt vmcnt(N)
 }
+// all but the youngest `groups` groups of LOADS loads each (at most three groups)
+template <int LOADS> __device__ __forceinline__ void mid_wait_for_all_but_groups(int groups) {
+    static_assert(3 * LOADS < 64, "the counter has six bits");
+    if (groups >= 3) mid_wait_for_all_but_the_youngest_loads<3 * LOADS>();
+    else if (groups == 2) mid_wait_for_all_but_the_youngest_loads<2 * LOADS>();
+    else if (groups == 1) mid_wait_for_all_but_the_youngest_loads<1 * LOADS>();
+    else mid_wait_for_all_but_the_youngest_loads<0>();
+}
 __device__ __forceinline__ void mid_barrier() {        // LDS reads done, then the block's barrier; loads stay in flight
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
@@ -89,7 +97,7 @@ __global__ __launch_bounds__(MID_THREADS) void linear_mid_kernel(
     // loads asked for after the chunk that is due, see the loop
     constexpr int YOUNGER = SAME ? (A_STAGES - 2) * (MID_A_LOADS + W_LOADS) : W_LOADS + MID_A_LOADS + W_LOADS;
     constexpr int YOUNGER_AT_START = SAME ? (A_STAGES - 1) * (MID_A_LOADS + W_LOADS) : (W_STAGES - 1) * W_LOADS + 2 * MID_A_LOADS;
-    static_assert(A_STAGES >= 3 && W_STAGES >= 3 && YOUNGER_AT_START < 64, "the rings' depth and the counter's six bits");
+    static_assert(A_STAGES >= 3 && W_STAGES >= 3 && A_STAGES <= 4 + (SAME ? 0 : 8) && YOUNGER_AT_START < 64, "the rings' depth and the counter's six bits");
     __shared__ __attribute__((aligned(1024))) char a_lds[A_STAGES * MID_A_BYTES];
     __shared__ __attribute__((aligned(1024))) char w_lds[W_STAGES * W_BYTES];
 
@@ -199,8 +207,11 @@ __global__ __launch_bounds__(MID_THREADS) void linear_mid_kernel(
     // weights of a chunk side by side.  Three chunks of rows and more of weights: the weights asked for in the pass of
     // the next chunk's rows, and the rows and weights of the pass after, come last.
     if (SAME) {
+        // (a short range asks for no chunk beyond its end, and the waits count what was asked for)
 #pragma unroll
-        for (int s = 0; s < A_STAGES; ++s) { ask_rows(c0 + s); ask_weights(c0 + s); }
+        for (int s = 0; s < A_STAGES; ++s)
+            if (c0 + s < c1) { ask_rows(c0 + s); ask_weights(c0 + s); }
+        mid_wait_for_all_but_groups<MID_A_LOADS + W_LOADS>(min(A_STAGES, c1 - c0) - 1);
     } else {
         ask_rows(c0);
 #pragma unroll
@@ -209,8 +220,8 @@ __global__ __launch_bounds__(MID_THREADS) void linear_mid_kernel(
         ask_weights(c0 + W_STAGES - 2);
         ask_rows(c0 + 2);
         ask_weights(c0 + W_STAGES - 1);
+        mid_wait_for_all_but_the_youngest_loads<YOUNGER_AT_START>();      // the first chunk's rows and weights are there
     }
-    mid_wait_for_all_but_the_youngest_loads<YOUNGER_AT_START>();      // the first chunk's rows and weights are there
     mid_barrier();
     Fragments f[2];
     read(0, 0, 0, f[0]);
@@ -223,10 +234,18 @@ __global__ __launch_bounds__(MID_THREADS) void linear_mid_kernel(
         }
         // The chunk's last fragments are in registers (or on their way: the barrier waits for them).  The next chunk
         // must have landed, for every wave's share of it: all but the loads asked for after it are done.
-        mid_wait_for_all_but_the_youngest_loads<YOUNGER>();
-        mid_barrier();
-        ask_rows(c + A_STAGES);                                 // into the slots that this chunk's readers have left
-        ask_weights(c + W_STAGES);
+        if (SAME) {
+            // after chunk c + 1 come the chunks up to c + A_STAGES - 1, as far as the range goes; at its end nothing
+            // is asked for any more, and the last passes wait for fewer
+            mid_wait_for_all_but_groups<MID_A_LOADS + W_LOADS>(min(A_STAGES - 2, c1 - 2 - c));
+            mid_barrier();
+            if (c + A_STAGES < c1) { ask_rows(c + A_STAGES); ask_weights(c + A_STAGES); }       // into the slots this chunk's readers have left
+        } else {
+            mid_wait_for_all_but_the_youngest_loads<YOUNGER>();
+            mid_barrier();
+            ask_rows(c + A_STAGES);                             // into the slots that this chunk's readers have left
+            ask_weights(c + W_STAGES);
+        }
         if (c + 1 < c1) read((c + 1 - c0) % A_STAGES, (c + 1 - c0) % W_STAGES, 0, f[0]);
         products(f[(MID_CHUNK / 16 - 1) & 1]);
     }
